@@ -837,11 +837,15 @@ class ViewNode(Node):
         self._val: Optional[Value] = None
 
     def forward(self):
-        # the reference checks its own cached value only, not the parent's (view.rs:18-20)
-        if self._val is not None:
-            return self._val.clone()
-        v = self.parent.forward()
-        self._val = c_view(v, self.target_dim, None)
+        # The reference returns its cached value without looking at the parent (view.rs:18-20), so a
+        # predicate whose chain contains a view (every `.all()` does) is never refreshed when
+        # `ir_while` re-forwards it.  Like every other node, the view is re-emitted here (with the
+        # same id) when something below it was invalidated.
+        v = self.val()
+        if v is not None:
+            return v.clone()
+        p = self.parent.forward()
+        self._val = c_view(p, self.target_dim, self._val.id if self._val is not None else None)
         return self._val.clone()
 
     def dim(self):

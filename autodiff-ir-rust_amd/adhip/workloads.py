@@ -1,0 +1,234 @@
+"""The five synthetic workloads the backend is measured and parity-tested on, written against the
+caller-side API exactly as a user of the reference would write them.  Sizes are parameters: the
+benchmark uses the full sizes, the parity tests the same programs at sizes a CPU oracle finishes
+in seconds.
+
+Every builder takes the device, installs it with `autodiff.set_device`, builds the graph, and
+returns a `Workload` whose `.run()` executes it and whose `.outputs` maps names to `Value`s to
+`get()` afterwards.  Inputs come from `numpy.random.default_rng(seed)`, float32.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Optional
+
+import numpy as np
+
+from . import autodiff, nn
+from .core import STATE, Tensor, Value, concat, constant
+
+
+class Workload:
+    def __init__(self, name: str, outputs: Dict[str, Value], inputs: Dict[str, np.ndarray],
+                 algorithmic_bytes: Optional[float] = None, flops: Optional[float] = None):
+        self.name = name
+        self.outputs = outputs
+        self.inputs = inputs
+        self.algorithmic_bytes = algorithmic_bytes
+        self.flops = flops
+
+    def finish(self):
+        """Append EX (what `autodiff.execute()` does first) and return (procedure, keep list)
+        without running anything; used to compile a resident program."""
+        from . import ir as IR
+        if not STATE.irb.proc.main or not isinstance(STATE.irb.proc.main[-1], IR.EX):
+            STATE.irb.add_cmd(IR.EX())
+        return STATE.irb.proc, set(STATE.dep_tracker)
+
+    def run(self):
+        autodiff.execute()
+        return self.get()
+
+    def get(self):
+        return {k: v.get() for k, v in self.outputs.items()}
+
+
+def _uniform(rng, shape, lo=-1.0, hi=1.0):
+    return rng.uniform(lo, hi, size=shape).astype(np.float32)
+
+
+# ---- config 1: README MLP ---------------------------------------------------------------
+
+def readme_mlp(dev, seed: int = 0) -> Workload:
+    """x [2,5]; Linear(5,3, no bias) -> sigmoid -> Linear(3,2, bias); forward, backward of
+    sum(output) (seed of ones), one SGD step with lr 0.1."""
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    w1 = _uniform(rng, (5, 3))
+    w2 = _uniform(rng, (3, 2))
+    b2 = _uniform(rng, (2,))
+    xs = np.array([1, 2, 3, 4, 5, 6, 7, 8, 3.2, 6.3], dtype=np.float32)
+    x = autodiff.tensor(xs, [2, 5])
+    W1 = autodiff.tensor(w1, [5, 3])
+    W2 = autodiff.tensor(w2, [3, 2])
+    B2 = autodiff.tensor(b2, [2])
+    net = nn.Sequential()
+    net.insert(nn.LinearWithWeights(W1, None))
+    net.insert(nn.Sigmoid())
+    net.insert(nn.LinearWithWeights(W2, B2))
+    opt = nn.SGD(net.params(), 0.1)
+    y = net.f(x)
+    y.forward()
+    y.backward()
+    grads = {"dW1": W1.grad(), "dW2": W2.grad(), "db2": B2.grad(), "dx": x.grad()}
+    for g in grads.values():
+        g.keep()
+    y.val().keep()
+    opt.step()
+    outs = {"y": y.val(), "W1": W1.val(), "W2": W2.val(), "b2": B2.val()}
+    outs.update(grads)
+    return Workload("readme_mlp", outs, {"x": xs, "W1": w1, "W2": w2, "b2": b2})
+
+
+# ---- config 2: fused element-wise + broadcast -------------------------------------------
+
+def fused_elw(dev, rows: int = 8192, cols: int = 8192, seed: int = 0, backward: bool = True) -> Workload:
+    """y = sigmoid(a*b + c + bias) - 0.5*exp(a) + sin(b)*cos(c), bias [cols] broadcast over rows;
+    L = y.sum(0).sum(0); backward of L to a, b, c, bias."""
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    an, bn, cn = (_uniform(rng, (rows, cols)) for _ in range(3))
+    biasn = _uniform(rng, (cols,))
+    a = autodiff.tensor(an, [rows, cols])
+    b = autodiff.tensor(bn, [rows, cols])
+    c = autodiff.tensor(cn, [rows, cols])
+    bias = autodiff.tensor(biasn, [cols])
+    y = (a * b + c + bias).sigmoid() - 0.5 * a.exp() + b.sin() * c.cos()
+    L = y.sum(0).sum(0)
+    L.forward()
+    y.val().keep()
+    L.val().keep()
+    outs = {"y": y.val(), "L": L.val()}
+    n = rows * cols
+    nbytes = 4.0 * (4 * n + cols)          # forward: read a,b,c,bias; write y
+    if backward:
+        L.backward()
+        outs.update({"da": a.grad(), "db": b.grad(), "dc": c.grad(), "dbias": bias.grad()})
+        nbytes += 4.0 * (6 * n + 2 * cols)  # backward: read a,b,c,bias; write da,db,dc,dbias
+    return Workload("fused_elw", outs, {"a": an, "b": bn, "c": cn, "bias": biasn}, algorithmic_bytes=nbytes)
+
+
+# ---- config 3: reductions ---------------------------------------------------------------
+
+def reductions(dev, rows: int = 16384, cols: int = 4096, seed: int = 0, backward: bool = True) -> Workload:
+    """s0 = x.powf(2).sum(1); s1 = x.sum(0); s2 = (x*x).sum(1).sum(0); backward of each to x."""
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    xn = rng.standard_normal((rows, cols), dtype=np.float32)
+    x = autodiff.tensor(xn, [rows, cols])
+    s0 = x.powf(2.0).sum(1)
+    s1 = x.sum(0)
+    s2 = (x * x).sum(1).sum(0)
+    outs = {}
+    for name, s in (("s0", s0), ("s1", s1), ("s2", s2)):
+        s.forward()
+        s.val().keep()
+        outs[name] = s.val()
+    n = rows * cols
+    nbytes = 3 * 4.0 * n + 4.0 * (rows + cols + 1)
+    if backward:
+        s0.backward()
+        s1.backward()
+        s2.backward()
+        outs["dx"] = x.grad()
+        nbytes += 2 * 4.0 * n
+    return Workload("reductions", outs, {"x": xn}, algorithmic_bytes=nbytes)
+
+
+# ---- config 4: dense MLP training -------------------------------------------------------
+
+def mlp_train(dev, batch: int = 4096, dims=(4096, 4096, 4096, 1024), iters: int = 10, lr: float = 0.01,
+              seed: int = 0) -> Workload:
+    """Linear(d0,d1)+sigmoid, Linear(d1,d2)+sigmoid, Linear(d2,d3), all with bias; Xavier-uniform
+    weights, biases U(-0.05,0.05); loss = mean((y-t)^2) composed from IR ops; forward + backward +
+    SGD for `iters` iterations inside an IR for-loop."""
+    autodiff.set_device(dev)
+    autodiff.eager_dep_opt()  # read back only what is kept explicitly, as the reference's nn test does
+    rng = np.random.default_rng(seed)
+    xn = rng.standard_normal((batch, dims[0]), dtype=np.float32)
+    tn = _uniform(rng, (batch, dims[-1]), 0.0, 1.0)
+    inputs = {"x": xn, "t": tn}
+    x = autodiff.tensor(xn, [batch, dims[0]])
+    t = autodiff.tensor(tn, [batch, dims[-1]])
+    net = nn.Sequential()
+    weights = []
+    for li in range(len(dims) - 1):
+        fan_in, fan_out = dims[li], dims[li + 1]
+        bound = np.sqrt(6.0 / (fan_in + fan_out))
+        wn = _uniform(rng, (fan_in, fan_out), -bound, bound)
+        bn = _uniform(rng, (fan_out,), -0.05, 0.05)
+        inputs[f"W{li}"] = wn
+        inputs[f"b{li}"] = bn
+        W = autodiff.tensor(wn, [fan_in, fan_out])
+        B = autodiff.tensor(bn, [fan_out])
+        weights.append((W, B))
+        net.insert(nn.LinearWithWeights(W, B))
+        if li + 2 < len(dims):
+            net.insert(nn.Sigmoid())
+    opt = nn.SGD(net.params(), lr)
+    scale = 1.0 / float(batch * dims[-1])
+    box = {}
+
+    def body(_):
+        y = net.f(x)
+        d = y - t
+        loss = (d * d).sum(1).sum(0) * scale
+        opt.zero_grad()
+        loss.forward()
+        loss.backward()
+        opt.step()
+        box["loss"] = loss
+
+    autodiff.ir_for(range(0, iters), body)
+    loss = box["loss"]
+    loss.val().keep()
+    x.grad().keep()  # keeps the first layer's dX product alive, as in the flop count of the config
+    outs = {"loss": loss.val(), "dx": x.grad()}
+    for li, (W, B) in enumerate(weights):
+        W.val().keep()
+        B.val().keep()
+        outs[f"W{li}"] = W.val()
+        outs[f"b{li}"] = B.val()
+    flops = 0.0
+    for li in range(len(dims) - 1):
+        flops += 3 * 2.0 * batch * dims[li] * dims[li + 1]  # forward, dX, dW
+    return Workload("mlp_train", outs, inputs, flops=flops * iters)
+
+
+# ---- config 5: tensor manipulation + data-dependent loop ---------------------------------
+
+def manip_loop(dev, nb: int = 64, n1: int = 512, n2: int = 1024, n3: int = 256, lo: int = 128, hi: int = 896,
+               max_iters: int = 50, seed: int = 0, snapshot_at: Optional[int] = None) -> Workload:
+    """p [nb,n1,n2], q [nb,n2,n3], w [n1+n3]; r = concat(p.permute(0,2,1), q, dim=2)[:, lo:hi, :]
+    .view([nb*(hi-lo), n1+n3]) * w; while not (r.sum(1) < 1).all() and i < max_iters:
+    r -= 0.01 * r.sum(1)[:, None]."""
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    pn = _uniform(rng, (nb, n1, n2))
+    qn = _uniform(rng, (nb, n2, n3))
+    wn = _uniform(rng, (n1 + n3,))
+    p = autodiff.tensor(pn, [nb, n1, n2])
+    q = autodiff.tensor(qn, [nb, n2, n3])
+    w = autodiff.tensor(wn, [n1 + n3])
+    rows, width = nb * (hi - lo), n1 + n3
+    gathered = concat([p.permute([0, 2, 1]), q], 2).r(range(lo, hi), 1).view([rows, width])
+    g0 = gathered.contigious()           # the gather stage on its own (bit-exact check)
+    g0.forward()
+    g0.val().keep()
+    r = gathered * w
+    i = autodiff.scalar(0.0)
+    limit = float(max_iters if snapshot_at is None else snapshot_at)
+    not_done = 1.0 - r.sum(1).less_than(constant(1.0, [rows])).all()
+    pred = not_done * i.less_than(constant(limit, [1]))
+    r.forward()
+
+    def body():
+        nonlocal r, i
+        rv = r.val().to_node()
+        r -= 0.01 * rv.sum(1).unsqueeze(-1)
+        i += 1.0
+
+    autodiff.ir_while(pred, body)
+    r.val().keep()
+    outs = {"gathered": g0.val(), "r": r.val(), "i": i.val()}
+    return Workload("manip_loop", outs, {"p": pn, "q": qn, "w": wn},
+                    algorithmic_bytes=4.0 * 2 * rows * width)

@@ -1,0 +1,845 @@
+#include "codegen.hpp"
+
+#include <algorithm>
+#include <cstring>
+#include <functional>
+
+namespace adhip {
+
+const char* op_name(Op o) {
+    switch (o) {
+    case Op::LIVEIN: return "livein";
+    case Op::UPLOAD: return "upload";
+    case Op::ADD: return "add";
+    case Op::MUL: return "mul";
+    case Op::EXP2: return "exp2";
+    case Op::LOG2: return "log2";
+    case Op::SIN: return "sin";
+    case Op::RECIP: return "recip";
+    case Op::SQRT: return "sqrt";
+    case Op::EQ0: return "eq0";
+    case Op::GT0: return "gt0";
+    case Op::LT0: return "lt0";
+    case Op::COPY: return "copy";
+    case Op::FILL: return "fill";
+    case Op::SUM: return "sum";
+    case Op::DOT: return "dot";
+    }
+    return "?";
+}
+
+const char* kernel_prelude() {
+    // Everything the generated kernels need besides what hipRTC provides by itself.
+    return R"(
+typedef float float4_t __attribute__((ext_vector_type(4)));
+static __device__ __forceinline__ float u2f(unsigned u) { return __builtin_bit_cast(float, u); }
+static __device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+)";
+}
+
+namespace {
+
+// ---------------------------------------------------------------------------------------
+// symbolic integer index arithmetic: c + sum(coef * atom), atoms with known ranges
+// ---------------------------------------------------------------------------------------
+
+struct Atom {
+    std::string name;
+    int64_t range = 1;  // value in [0, range) whenever the access it feeds is selected
+    bool lane = false;  // differs between the lanes of one thread's vector
+};
+
+struct Aff {
+    int64_t c = 0;
+    std::vector<std::pair<int, int64_t>> t;  // (atom, coef), sorted by atom, coef != 0
+};
+
+Aff aff_const(int64_t c) { Aff a; a.c = c; return a; }
+Aff aff_atom(int id, int64_t coef = 1) { Aff a; if (coef) a.t.push_back({id, coef}); return a; }
+
+Aff aff_add(const Aff& a, const Aff& b) {
+    Aff r;
+    r.c = a.c + b.c;
+    size_t i = 0, j = 0;
+    while (i < a.t.size() || j < b.t.size()) {
+        if (j >= b.t.size() || (i < a.t.size() && a.t[i].first < b.t[j].first)) r.t.push_back(a.t[i++]);
+        else if (i >= a.t.size() || b.t[j].first < a.t[i].first) r.t.push_back(b.t[j++]);
+        else {
+            int64_t k = a.t[i].second + b.t[j].second;
+            if (k) r.t.push_back({a.t[i].first, k});
+            ++i; ++j;
+        }
+    }
+    return r;
+}
+
+Aff aff_scale(const Aff& a, int64_t k) {
+    Aff r;
+    if (k == 0) return r;
+    r.c = a.c * k;
+    for (auto& x : a.t) r.t.push_back({x.first, x.second * k});
+    return r;
+}
+
+std::string aff_key(const Aff& a) {
+    std::string s = std::to_string(a.c);
+    for (auto& x : a.t) s += "+" + std::to_string(x.second) + "*" + std::to_string(x.first);
+    return s;
+}
+
+struct Val {
+    std::string expr;
+    bool lane = false;
+};
+
+struct LoadRec {
+    const Node* node;
+    Aff idx;
+    bool predicated;
+};
+
+struct Gen {
+    int vec = 1;
+    int lane_atom = -1;
+    bool wide = false;
+    std::vector<Atom> atoms;
+    std::vector<std::string> codeA, codeB;  // per-thread / per-lane statements
+    std::map<std::string, int> atom_memo;
+    std::map<std::string, Val> val_memo;
+    std::map<std::string, bool> pred_lane;
+    std::map<const Node*, int> buf_index;
+    std::vector<GenBuffer> bufs;
+    std::set<const Node*> members;  // computed in this kernel, never loaded
+    std::vector<LoadRec> loads;
+    std::vector<Aff> recorded;  // every index expression over base atoms, for dim merging
+    int tmp = 0;
+    double flops = 0;  // per lane element
+
+    const char* idx_t() const { return wide ? "unsigned long long" : "unsigned int"; }
+
+    int add_atom(const std::string& name, int64_t range, bool lane) {
+        atoms.push_back({name, range, lane});
+        return (int)atoms.size() - 1;
+    }
+
+    int64_t aff_max(const Aff& a) const {
+        int64_t m = a.c;
+        for (auto& x : a.t)
+            if (x.second > 0) m += x.second * (atoms[x.first].range - 1);
+        return m;
+    }
+    int64_t aff_min(const Aff& a) const {
+        int64_t m = a.c;
+        for (auto& x : a.t)
+            if (x.second < 0) m += x.second * (atoms[x.first].range - 1);
+        return m;
+    }
+    bool aff_lane(const Aff& a) const {
+        for (auto& x : a.t)
+            if (atoms[x.first].lane) return true;
+        return false;
+    }
+
+    std::string aff_str(const Aff& a) {
+        recorded.push_back(a);
+        if (a.t.empty()) return strf("(%s)%lld", idx_t(), (long long)a.c) + (wide ? "ull" : "u");
+        std::string s = "(";
+        bool first = true;
+        for (auto& x : a.t) {
+            if (!first) s += " + ";
+            first = false;
+            if (x.second == 1) s += atoms[x.first].name;
+            else s += strf("%lld%s * %s", (long long)x.second, wide ? "ull" : "u", atoms[x.first].name.c_str());
+        }
+        if (a.c) s += strf(" + %lld%s", (long long)a.c, wide ? "ull" : "u");
+        return s + ")";
+    }
+
+    void emit(bool lane, const std::string& stmt) { (lane ? codeB : codeA).push_back(stmt); }
+
+    // an atom defined by an expression over other atoms
+    int expr_atom(const std::string& code, int64_t range, bool lane) {
+        auto it = atom_memo.find(code);
+        if (it != atom_memo.end()) return it->second;
+        std::string name = "a" + std::to_string(tmp++);
+        emit(lane, strf("const %s %s = %s;", idx_t(), name.c_str(), code.c_str()));
+        int id = add_atom(name, range, lane);
+        atom_memo[code] = id;
+        return id;
+    }
+
+    // exact a / k when every term divides, else an opaque quotient atom
+    Aff aff_div(const Aff& a, int64_t k) {
+        if (k == 1) return a;
+        bool exact = a.c % k == 0;
+        for (auto& x : a.t) exact = exact && (x.second % k == 0);
+        if (exact) {
+            Aff r;
+            r.c = a.c / k;
+            for (auto& x : a.t) r.t.push_back({x.first, x.second / k});
+            return r;
+        }
+        int64_t mx = aff_max(a);
+        if (mx < k && aff_min(a) >= 0) return aff_const(0);
+        std::string code = strf("%s / %lld%s", aff_str(a).c_str(), (long long)k, wide ? "ull" : "u");
+        return aff_atom(expr_atom(code, mx / k + 1, aff_lane(a)));
+    }
+
+    Aff aff_mod(const Aff& a, int64_t k) {
+        if (aff_max(a) < k && aff_min(a) >= 0) return a;
+        std::string code = strf("%s %% %lld%s", aff_str(a).c_str(), (long long)k, wide ? "ull" : "u");
+        return aff_atom(expr_atom(code, k, aff_lane(a)));
+    }
+
+    // Split a linear row-major index over `shape` into coordinates.
+    std::vector<Aff> split(const Aff& e, const Shape& shape) {
+        const size_t n = shape.size();
+        std::vector<Aff> out(n);
+        if (n == 0) return out;
+        if (n == 1) { out[0] = e; return out; }
+        Shape r = row_major_strides(shape);
+        Aff rem = e;
+        for (size_t j = n - 1; j >= 1; --j) {
+            const int64_t M = r[j] * shape[j];
+            Aff low, high;
+            bool ok = rem.c >= 0;
+            low.c = rem.c >= 0 ? rem.c % M : 0;
+            high.c = rem.c - low.c;
+            if (low.c % r[j] != 0) ok = false;
+            for (auto& x : rem.t) {
+                if (x.second < 0) { ok = false; break; }
+                if (x.second % M == 0) high.t.push_back(x);
+                else if (x.second < M && x.second % r[j] == 0) low.t.push_back(x);
+                else { ok = false; break; }
+            }
+            if (ok && aff_max(low) < M) {
+                out[j] = aff_div(low, r[j]);
+                rem = high;
+                continue;
+            }
+            // Fall back to explicit div/mod from this dim outwards.
+            Aff q = aff_div(rem, r[j]);
+            for (size_t jj = j; jj >= 1; --jj) {
+                out[jj] = aff_mod(q, shape[jj]);
+                q = aff_div(q, shape[jj]);
+            }
+            out[0] = q;
+            return out;
+        }
+        out[0] = aff_div(rem, r[0]);
+        return out;
+    }
+
+    static bool stage_row_major(const Stage& s) {
+        int64_t expect = 1;
+        for (int i = (int)s.shape.size() - 1; i >= 0; --i) {
+            if (s.shape[i] == 1) continue;
+            if (s.stride[i] != expect) return false;
+            expect *= s.shape[i];
+        }
+        return true;
+    }
+
+    Aff apply_stage_coords(const Stage& s, const std::vector<Aff>& coords) {
+        Aff l = aff_const(s.offset);
+        for (size_t i = 0; i < s.shape.size(); ++i) {
+            if (s.shape[i] == 1 || s.stride[i] == 0) continue;
+            l = aff_add(l, aff_scale(coords[i], s.stride[i]));
+        }
+        return l;
+    }
+
+    Aff apply_view_from(const View& v, size_t k, Aff l) {
+        for (; k < v.st.size(); ++k) {
+            const Stage& s = v.st[k];
+            if (stage_row_major(s)) { l = aff_add(l, aff_const(s.offset)); continue; }
+            l = apply_stage_coords(s, split(l, s.shape));
+        }
+        return l;
+    }
+
+    int buffer_of(const Node* n) {
+        auto it = buf_index.find(n);
+        if (it != buf_index.end()) return it->second;
+        GenBuffer b;
+        b.node = const_cast<Node*>(n);
+        b.param = "b" + std::to_string(bufs.size());
+        bufs.push_back(b);
+        buf_index[n] = (int)bufs.size() - 1;
+        return (int)bufs.size() - 1;
+    }
+
+    static std::string flit(float f) {
+        unsigned u;
+        memcpy(&u, &f, 4);
+        return strf("u2f(0x%08xu)", u);
+    }
+
+    bool vectorizable(const Aff& idx) const {
+        if (vec == 1 || lane_atom < 0) return false;
+        if (idx.c % vec != 0) return false;
+        bool has_lane = false;
+        for (auto& x : idx.t) {
+            if (x.first == lane_atom) {
+                if (x.second != 1) return false;
+                has_lane = true;
+            } else {
+                if (atoms[x.first].lane) return false;
+                if (x.second % vec != 0) return false;
+            }
+        }
+        return has_lane;
+    }
+
+    Val load(const Node* n, const Aff& idx, const std::string& pred) {
+        const bool plane = !pred.empty() && pred_lane[pred];
+        std::string key = "L" + std::to_string(n->id) + "@" + aff_key(idx) + "?" + pred;
+        auto it = val_memo.find(key);
+        if (it != val_memo.end()) return it->second;
+        const int64_t ne = numel(n->shape);
+        ADHIP_CHECK(aff_min(idx) >= 0 && aff_max(idx) < ne,
+                    "internal: generated load of node %d (%s) spans [%lld,%lld] outside its %lld elements", n->id,
+                    n->name.c_str(), (long long)aff_min(idx), (long long)aff_max(idx), (long long)ne);
+        loads.push_back({n, idx, !pred.empty()});
+        const std::string& bp = bufs[buffer_of(n)].param;
+        std::string name = "l" + std::to_string(tmp++);
+        Val v;
+        const bool ilane = aff_lane(idx);
+        if (!ilane && !plane) {
+            if (pred.empty()) emit(false, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
+            else emit(false, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
+            v = {name, false};
+        } else if (!plane && vectorizable(idx)) {
+            Aff base = idx;
+            for (auto it2 = base.t.begin(); it2 != base.t.end(); ++it2)
+                if (it2->first == lane_atom) { base.t.erase(it2); break; }
+            std::string addr = strf("*(const float4_t*)(%s + %s)", bp.c_str(), aff_str(base).c_str());
+            if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
+            else emit(false, strf("float4_t %sv = {0.f, 0.f, 0.f, 0.f}; if (%s) %sv = %s;", name.c_str(), pred.c_str(), name.c_str(), addr.c_str()));
+            emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
+            v = {name + "[" + atoms[lane_atom].name + "]", true};
+        } else {
+            if (pred.empty()) emit(true, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
+            else emit(true, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
+            v = {name, true};
+        }
+        val_memo[key] = v;
+        return v;
+    }
+
+    std::string and_pred(const std::string& pred, const std::string& cond, bool cond_lane) {
+        std::string key = "P" + pred + "&" + cond;
+        auto it = val_memo.find(key);
+        if (it != val_memo.end()) return it->second.expr;
+        std::string name = "p" + std::to_string(tmp++);
+        bool lane = cond_lane || (!pred.empty() && pred_lane[pred]);
+        emit(lane, strf("const bool %s = %s%s;", name.c_str(), pred.empty() ? "" : (pred + " && ").c_str(), cond.c_str()));
+        pred_lane[name] = lane;
+        val_memo[key] = {name, lane};
+        return name;
+    }
+
+    Val gen_src(const Piece& p, const Aff& idx, const std::string& pred) {
+        switch (p.src.kind) {
+        case Src::CONST: return {flit(p.src.c), false};
+        case Src::NODE: return gen_node(p.src.node, idx, pred);
+        default: throw Error("internal: unresolved tensor reference reached code generation");
+        }
+    }
+
+    // value of tensor reference `t` at linear (row-major over t.shape) index l
+    Val gen_tref(const TRef& t, const Aff& l, const std::string& pred) {
+        ADHIP_CHECK(!t.pieces.empty(), "internal: empty tensor reference in code generation");
+        if (t.single_full()) {
+            const Piece& p = t.pieces[0];
+            if (p.src.kind == Src::CONST) return {flit(p.src.c), false};
+            return gen_src(p, apply_view_from(p.view, 0, l), pred);
+        }
+        std::vector<Aff> coords = split(l, t.shape);
+        std::vector<Val> vals;
+        std::vector<std::string> conds;
+        std::vector<bool> cond_lanes;
+        for (size_t pi = 0; pi < t.pieces.size(); ++pi) {
+            const Piece& p = t.pieces[pi];
+            std::string cond;
+            bool clane = false;
+            std::vector<Aff> local(coords.size());
+            for (size_t d = 0; d < coords.size(); ++d) {
+                const bool partial = p.lo[d] != 0 || p.hi[d] != t.shape[d];
+                if (!partial) { local[d] = coords[d]; continue; }
+                clane = clane || aff_lane(coords[d]);
+                std::string cs = aff_str(coords[d]);
+                if (p.lo[d] != 0) cond += strf("%s%s >= %lldu", cond.empty() ? "" : " && ", cs.c_str(), (long long)p.lo[d]);
+                if (p.hi[d] != t.shape[d]) cond += strf("%s%s < %lldu", cond.empty() ? "" : " && ", cs.c_str(), (long long)p.hi[d]);
+                if (p.lo[d] != 0) {
+                    std::string code = strf("%s - %lld%s", cs.c_str(), (long long)p.lo[d], wide ? "ull" : "u");
+                    local[d] = aff_atom(expr_atom(code, p.hi[d] - p.lo[d], aff_lane(coords[d])));
+                } else {
+                    // same variable, tighter range while this piece is selected
+                    std::string code = strf("%s + 0u", cs.c_str());
+                    local[d] = aff_atom(expr_atom(code + strf("/*<%lld*/", (long long)p.hi[d]), p.hi[d], aff_lane(coords[d])));
+                }
+            }
+            std::string ppred = cond.empty() ? pred : and_pred(pred, "(" + cond + ")", clane);
+            Val v;
+            if (p.src.kind == Src::CONST) v = {flit(p.src.c), false};
+            else {
+                Aff idx = apply_stage_coords(p.view.st[0], local);
+                idx = apply_view_from(p.view, 1, idx);
+                v = gen_src(p, idx, ppred);
+            }
+            vals.push_back(v);
+            conds.push_back(cond.empty() ? "" : ppred);
+            cond_lanes.push_back(!cond.empty() && pred_lane[ppred]);
+        }
+        // select chain; the last piece is the default
+        std::string e = vals.back().expr;
+        bool lane = vals.back().lane;
+        for (size_t pi = t.pieces.size() - 1; pi-- > 0;) {
+            if (conds[pi].empty()) { e = vals[pi].expr; lane = vals[pi].lane; continue; }
+            e = "(" + conds[pi] + " ? " + vals[pi].expr + " : " + e + ")";
+            lane = lane || vals[pi].lane || cond_lanes[pi];
+        }
+        std::string name = "s" + std::to_string(tmp++);
+        emit(lane, strf("const float %s = %s;", name.c_str(), e.c_str()));
+        return {name, lane};
+    }
+
+    bool in_memory(const Node* n) const { return (op_is_leaf(n->op) || n->root) && !members.count(n); }
+
+    Val gen_node(const Node* n, const Aff& l, const std::string& pred) {
+        if (in_memory(n)) return load(n, l, pred);
+        if (n->op == Op::FILL) return {flit(n->cval), false};
+        ADHIP_CHECK(op_is_elw(n->op), "internal: node %d (%s) is neither in memory nor element-wise", n->id, op_name(n->op));
+        std::string key = "N" + std::to_string(n->id) + "@" + aff_key(l) + "?" + pred;
+        auto it = val_memo.find(key);
+        if (it != val_memo.end()) return it->second;
+        std::vector<Val> a;
+        for (const TRef& t : n->in) a.push_back(gen_tref(t, l, pred));
+        bool lane = false;
+        for (auto& v : a) lane = lane || v.lane;
+        std::string e;
+        const std::string& x = a[0].expr;
+        switch (n->op) {
+        case Op::ADD: e = x + " + " + a[1].expr; break;
+        case Op::MUL: e = x + " * " + a[1].expr; break;
+        case Op::EXP2: e = "exp2f(" + x + ")"; break;
+        case Op::LOG2: e = "log2f(" + x + ")"; break;
+        case Op::SIN: e = "sinf(" + x + ")"; break;
+        case Op::RECIP: e = "1.0f / " + x; break;
+        case Op::SQRT: e = "sqrtf(fabsf(" + x + "))"; break;
+        case Op::EQ0: e = "(" + x + " == 0.0f) ? 1.0f : 0.0f"; break;
+        case Op::GT0: e = "(" + x + " > 0.0f) ? 1.0f : 0.0f"; break;
+        case Op::LT0: e = "(" + x + " < 0.0f) ? 1.0f : 0.0f"; break;
+        case Op::COPY: e = x; break;
+        default: throw Error("internal: unexpected op in element-wise code generation");
+        }
+        if (n->op != Op::COPY) flops += op_is_transcendental(n->op) ? 8 : 1;
+        std::string name = "v" + std::to_string(tmp++);
+        emit(lane, strf("const float %s = %s;", name.c_str(), e.c_str()));
+        Val v{name, lane};
+        val_memo[key] = v;
+        return v;
+    }
+};
+
+std::string join(const std::vector<std::string>& v, const char* indent) {
+    std::string s;
+    for (auto& x : v) s += std::string(indent) + x + "\n";
+    return s;
+}
+
+bool needs_wide(const std::vector<Node*>& nodes) {
+    int64_t m = 0;
+    std::set<const Node*> seen;
+    std::function<void(const Node*)> walk = [&](const Node* n) {
+        if (!seen.insert(n).second) return;
+        m = std::max(m, numel(n->shape));
+        for (auto& t : n->in)
+            for (auto& p : t.pieces)
+                if (p.src.kind == Src::NODE) walk(p.src.node);
+    };
+    for (auto n : nodes) walk(n);
+    return m >= (int64_t(1) << 31) - 1024;
+}
+
+Shape drop_ones(const Shape& s) {
+    Shape r;
+    for (auto d : s)
+        if (d != 1) r.push_back(d);
+    if (r.empty()) r.push_back(1);
+    return r;
+}
+
+// bytes moved by a kernel, counting each distinct buffer once
+double traffic_bytes(const Gen& g, int64_t work_elems) {
+    double b = 0;
+    for (auto& gb : g.bufs) b += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), gb.written ? numel(gb.node->shape) : std::max<int64_t>(work_elems, 1));
+    return b;
+}
+
+// Iteration shapes: merge adjacent dims whose atoms always appear as one linear combination.
+Shape merge_dims(const Shape& shape, const std::vector<Aff>& recorded, const std::vector<int>& dim_atoms) {
+    // dim_atoms[i] = atom id of dim i (base atoms); returns merged shape
+    std::vector<bool> merge_with_next(shape.size(), false);
+    for (size_t i = 0; i + 1 < shape.size(); ++i) {
+        bool ok = true;
+        for (const Aff& a : recorded) {
+            int64_t ci = 0, cn = 0;
+            for (auto& x : a.t) {
+                if (x.first == dim_atoms[i]) ci = x.second;
+                if (x.first == dim_atoms[i + 1]) cn = x.second;
+            }
+            if (ci != cn * shape[i + 1]) { ok = false; break; }
+        }
+        merge_with_next[i] = ok;
+    }
+    Shape out;
+    int64_t cur = shape.empty() ? 1 : shape[0];
+    for (size_t i = 0; i + 1 < shape.size(); ++i) {
+        if (merge_with_next[i]) cur *= shape[i + 1];
+        else { out.push_back(cur); cur = shape[i + 1]; }
+    }
+    out.push_back(cur);
+    return out;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------
+// element-wise kernels
+// ---------------------------------------------------------------------------------------
+
+namespace {
+
+struct ElwBody {
+    Gen g;
+    std::vector<std::string> out_exprs;
+    std::vector<int> dim_atoms;
+    Shape iter_shape;
+};
+
+ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members, const Shape& iter_shape, int vec,
+                 bool wide) {
+    ElwBody b;
+    b.iter_shape = iter_shape;
+    Gen& g = b.g;
+    g.vec = vec;
+    g.wide = wide;
+    g.members = members;
+    const size_t nd = iter_shape.size();
+    Shape rs = row_major_strides(iter_shape);
+    Aff lin;
+    for (size_t i = 0; i < nd; ++i) {
+        const bool last = i + 1 == nd;
+        int64_t range = last ? iter_shape[i] / vec : iter_shape[i];
+        int a = g.add_atom("c" + std::to_string(i), range, false);
+        b.dim_atoms.push_back(a);
+        lin = aff_add(lin, aff_atom(a, last ? vec : rs[i]));
+    }
+    if (vec > 1) {
+        g.lane_atom = g.add_atom("j", vec, true);
+        lin = aff_add(lin, aff_atom(g.lane_atom, 1));
+    }
+    for (Node* out : spec.outputs) {
+        // an output is computed from its operands even though it ends up in memory
+        std::vector<Val> a;
+        ADHIP_CHECK(op_is_elw(out->op), "internal: element-wise kernel asked to produce %s", op_name(out->op));
+        Val v = g.gen_node(out, lin, "");
+        b.out_exprs.push_back(v.expr);
+    }
+    return b;
+}
+
+}  // namespace
+
+GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members) {
+    ADHIP_CHECK(!spec.outputs.empty(), "internal: element-wise kernel without outputs");
+    const int64_t N = numel(spec.outputs[0]->shape);
+    for (Node* o : spec.outputs) ADHIP_CHECK(numel(o->shape) == N, "internal: fused outputs differ in size");
+    ADHIP_CHECK(N > 0, "internal: empty element-wise kernel");
+    const bool wide = needs_wide(spec.outputs);
+
+    // pass 1: natural shape, scalar lanes, to learn which dims can be merged
+    Shape shape = drop_ones(spec.outputs[0]->shape);
+    {
+        ElwBody dry = elw_body(spec, members, shape, 1, wide);
+        // atom definitions are recorded through aff_str as well
+        shape = merge_dims(shape, dry.g.recorded, dry.dim_atoms);
+    }
+    int vec = (shape.back() % 4 == 0 && N >= 1024) ? 4 : 1;
+    ElwBody b = elw_body(spec, members, shape, vec, wide);
+    Gen& g = b.g;
+
+    GeneratedKernel k;
+    k.kind = "elw";
+    k.entry = spec.name;
+    const int64_t threads = N / vec;
+    std::string sig = "const int* __restrict__ guard";
+    std::vector<Node*> order;
+    // outputs first, then inputs
+    std::vector<std::string> out_params;
+    for (size_t i = 0; i < spec.outputs.size(); ++i) {
+        out_params.push_back("o" + std::to_string(i));
+        sig += ", float* o" + std::to_string(i);
+        order.push_back(spec.outputs[i]);
+    }
+    for (auto& gb : g.bufs) {
+        // a buffer that is also written in this kernel (in-place update) must not be restrict-qualified
+        sig += ", const float* " + gb.param;
+        order.push_back(gb.node);
+    }
+    std::string src = kernel_prelude();
+    src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+    src += "    if (guard && *guard == 0) return;\n";
+    src += strf("    const %s t = (%s)blockIdx.x * 256u + threadIdx.x;\n", g.idx_t(), g.idx_t());
+    src += strf("    if (t >= %lld%s) return;\n", (long long)threads, wide ? "ull" : "u");
+    // decompose t into iteration atoms
+    {
+        std::string rem = "t";
+        for (size_t i = shape.size(); i-- > 0;) {
+            int64_t range = (i + 1 == shape.size()) ? shape[i] / vec : shape[i];
+            if (i == 0) src += strf("    const %s c0 = %s;\n", g.idx_t(), rem.c_str());
+            else {
+                src += strf("    const %s c%zu = %s %% %lld%s;\n", g.idx_t(), i, rem.c_str(), (long long)range, wide ? "ull" : "u");
+                src += strf("    const %s r%zu = %s / %lld%s;\n", g.idx_t(), i, rem.c_str(), (long long)range, wide ? "ull" : "u");
+                rem = "r" + std::to_string(i);
+            }
+        }
+    }
+    src += join(g.codeA, "    ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("    float w%zu[%d];\n", i, vec);
+    if (vec > 1) src += strf("#pragma unroll\n    for (int j = 0; j < %d; ++j) {\n", vec);
+    else src += "    {\n";
+    src += join(g.codeB, "        ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i)
+        src += strf("        w%zu[%s] = %s;\n", i, vec > 1 ? "j" : "0", b.out_exprs[i].c_str());
+    src += "    }\n";
+    for (size_t i = 0; i < spec.outputs.size(); ++i) {
+        if (vec == 4) src += strf("    { float4_t q = {w%zu[0], w%zu[1], w%zu[2], w%zu[3]}; *(float4_t*)(o%zu + t * 4u) = q; }\n", i, i, i, i, i);
+        else src += strf("    o%zu[t] = w%zu[0];\n", i, i);
+    }
+    src += "}\n";
+    k.source = src;
+    k.buffer_args = order;
+    k.block[0] = 256;
+    k.grid[0] = (unsigned)((threads + 255) / 256);
+    k.bytes = 4.0 * (double)N * (double)spec.outputs.size();
+    for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), N);
+    k.flops = g.flops * (double)N;
+    return k;
+}
+
+// ---------------------------------------------------------------------------------------
+// reductions
+// ---------------------------------------------------------------------------------------
+
+namespace {
+
+enum class RedLayout { ROW, COL };
+
+struct RedBody {
+    Gen g;
+    std::string value;  // per-lane value expression
+    bool value_lane = false;
+};
+
+// atoms: ROW: x, yv (+ lane j along y); COL: xv, y (+ lane j along x)
+RedBody red_body(const Node* n, RedLayout layout, int vec, bool wide) {
+    RedBody b;
+    Gen& g = b.g;
+    g.vec = vec;
+    g.wide = wide;
+    const TRef& t = n->in[0];
+    const int64_t V = t.shape[0], R = t.shape[1];
+    Aff lin;
+    if (layout == RedLayout::ROW) {
+        int ax = g.add_atom("x", V, false);
+        int ay = g.add_atom("yv", R / vec, false);
+        lin = aff_add(aff_atom(ax, R), aff_atom(ay, vec));
+    } else {
+        int ax = g.add_atom("xv", V / vec, false);
+        int ay = g.add_atom("y", R, false);
+        lin = aff_add(aff_atom(ax, R * vec), aff_atom(ay, 1));
+    }
+    if (vec > 1) {
+        g.lane_atom = g.add_atom("j", vec, true);
+        lin = aff_add(lin, aff_atom(g.lane_atom, layout == RedLayout::ROW ? 1 : R));
+    }
+    Val v = g.gen_tref(t, lin, "");
+    b.value = v.expr;
+    b.value_lane = v.lane;
+    return b;
+}
+
+}  // namespace
+
+GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks) {
+    const Node* n = spec.node;
+    ADHIP_CHECK(n->op == Op::SUM && n->in.size() == 1 && n->in[0].shape.size() == 2, "internal: malformed reduction");
+    const int64_t V = n->in[0].shape[0], R = n->in[0].shape[1];
+    ADHIP_CHECK(V > 0 && R > 0, "internal: empty reduction");
+    std::vector<Node*> roots{const_cast<Node*>(n)};
+    const bool wide = needs_wide(roots);
+
+    // Decide the thread layout from how the largest operand is addressed.
+    RedLayout layout = RedLayout::ROW;
+    {
+        RedBody dry = red_body(n, RedLayout::ROW, 1, wide);
+        int64_t best = -1;
+        int64_t cx = 0, cy = 0;
+        for (auto& l : dry.g.loads) {
+            int64_t ne = numel(l.node->shape);
+            if (ne <= best) continue;
+            best = ne;
+            cx = cy = 0;
+            for (auto& x : l.idx.t) {
+                if (x.first == 0) cx = x.second;
+                if (x.first == 1) cy = x.second;
+            }
+        }
+        if (cy != 1 && cx == 1 && V >= 64) layout = RedLayout::COL;
+    }
+    GeneratedKernel k;
+    k.entry = spec.name;
+    int vec;
+    std::string src = kernel_prelude();
+    if (layout == RedLayout::ROW) {
+        vec = (R % 4 == 0 && R >= 256) ? 4 : 1;
+        RedBody b = red_body(n, layout, vec, wide);
+        Gen& g = b.g;
+        const int64_t RV = R / vec;
+        // threads per row
+        int T = RV <= 64 ? 64 : (RV <= 512 ? 64 : 256);
+        if (V < 64 && RV >= 4096) T = 256;
+        const int rows_per_block = 256 / T;
+        // split long rows over several blocks when there are too few rows to fill the GPU
+        int64_t chunks = 1;
+        if (force_chunks > 0) chunks = force_chunks;
+        else if (V * T < 131072 && RV >= (int64_t)T * 32) {
+            chunks = std::min<int64_t>((131072 + V * T - 1) / (V * T), RV / ((int64_t)T * 8));
+            chunks = std::max<int64_t>(chunks, 1);
+        }
+        const int64_t CH = (RV + chunks - 1) / chunks;  // vector elements per chunk
+        k.kind = "reduce_row";
+        std::string sig = "const int* __restrict__ guard, float* __restrict__ out";
+        std::vector<Node*> order{const_cast<Node*>(n)};
+        for (auto& gb : g.bufs) { sig += ", const float* __restrict__ " + gb.param; order.push_back(gb.node); }
+        src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+        src += "    if (guard && *guard == 0) return;\n";
+        src += strf("    const unsigned lane = threadIdx.x %% %du;\n", T);
+        src += strf("    const %s x = (%s)blockIdx.x * %du + threadIdx.x / %du;\n", g.idx_t(), g.idx_t(), rows_per_block, T);
+        src += "    const unsigned chunk = blockIdx.y;\n";
+        src += strf("    const bool row_ok = x < %lld%s;\n", (long long)V, wide ? "ull" : "u");
+        src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = 0.0f;\n", vec, vec);
+        src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)RV);
+        src += strf("    if (row_ok) for (%s yv = (%s)chunk * %lldu + lane; yv < y_end; yv += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, T);
+        src += join(g.codeA, "        ");
+        if (vec > 1) src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
+        else src += "        { const int j = 0;\n";
+        src += join(g.codeB, "            ");
+        src += strf("            acc[j] += %s;\n        }\n    }\n", b.value.c_str());
+        if (vec == 4) src += "    float s = (acc[0] + acc[1]) + (acc[2] + acc[3]);\n";
+        else src += "    float s = acc[0];\n";
+        if (T == 64) {
+            src += "    s = wave_sum(s);\n";
+            src += strf("    if (lane == 0 && row_ok) out[(%s)chunk * %lldu + x] = s;\n", g.idx_t(), (long long)V);
+        } else {
+            src += "    __shared__ float part[4];\n    s = wave_sum(s);\n";
+            src += "    if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = s;\n    __syncthreads();\n";
+            src += strf("    if (threadIdx.x == 0 && row_ok) out[(%s)chunk * %lldu + x] = (part[0] + part[1]) + (part[2] + part[3]);\n", g.idx_t(), (long long)V);
+        }
+        src += "}\n";
+        k.buffer_args = order;
+        k.block[0] = 256;
+        k.grid[0] = (unsigned)((V + rows_per_block - 1) / rows_per_block);
+        k.grid[1] = (unsigned)chunks;
+        k.chunks = chunks;
+        k.bytes = 4.0 * (double)V * (double)chunks;
+        for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), V * R);
+        k.flops = (g.flops + 1) * (double)V * (double)R;
+    } else {
+        vec = (V % 4 == 0 && V >= 1024) ? 4 : 1;
+        RedBody b = red_body(n, layout, vec, wide);
+        Gen& g = b.g;
+        const int64_t XV = V / vec;
+        const int YG = 4;  // row groups per block; block = 64 x YG threads
+        const int64_t bx = (XV + 63) / 64;
+        int64_t chunks = 1;
+        if (force_chunks > 0) chunks = force_chunks;
+        else {
+            chunks = (2048 + bx - 1) / bx;
+            chunks = std::min<int64_t>(chunks, std::max<int64_t>(R / (YG * 8), 1));
+            chunks = std::max<int64_t>(chunks, 1);
+        }
+        const int64_t CH = (R + chunks - 1) / chunks;
+        k.kind = "reduce_col";
+        std::string sig = "const int* __restrict__ guard, float* __restrict__ out";
+        std::vector<Node*> order{const_cast<Node*>(n)};
+        for (auto& gb : g.bufs) { sig += ", const float* __restrict__ " + gb.param; order.push_back(gb.node); }
+        src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+        src += "    if (guard && *guard == 0) return;\n";
+        src += strf("    __shared__ float part[%d][64][%d];\n", YG, vec);
+        src += "    const unsigned lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;\n";
+        src += strf("    const %s xv = (%s)blockIdx.x * 64u + lx;\n", g.idx_t(), g.idx_t());
+        src += "    const unsigned chunk = blockIdx.y;\n";
+        src += strf("    const bool col_ok = xv < %lld%s;\n", (long long)XV, wide ? "ull" : "u");
+        src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = 0.0f;\n", vec, vec);
+        src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)R);
+        src += strf("    if (col_ok) for (%s y = (%s)chunk * %lldu + ly; y < y_end; y += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, YG);
+        src += join(g.codeA, "        ");
+        if (vec > 1) src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
+        else src += "        { const int j = 0;\n";
+        src += join(g.codeB, "            ");
+        src += strf("            acc[j] += %s;\n        }\n    }\n", b.value.c_str());
+        src += strf("#pragma unroll\n    for (int j = 0; j < %d; ++j) part[ly][lx][j] = acc[j];\n    __syncthreads();\n", vec);
+        src += "    if (ly == 0 && col_ok) {\n";
+        src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
+        src += "            float s = (part[0][lx][j] + part[1][lx][j]) + (part[2][lx][j] + part[3][lx][j]);\n";
+        src += strf("            out[(%s)chunk * %lldu + xv * %du + j] = s;\n        }\n    }\n}\n", g.idx_t(), (long long)V, vec);
+        k.buffer_args = order;
+        k.block[0] = 256;
+        k.grid[0] = (unsigned)bx;
+        k.grid[1] = (unsigned)chunks;
+        k.chunks = chunks;
+        k.bytes = 4.0 * (double)V * (double)chunks;
+        for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), V * R);
+        k.flops = (g.flops + 1) * (double)V * (double)R;
+    }
+    k.source = src;
+    return k;
+}
+
+bool tref_affine2d(const TRef& t, Affine2D& out) {
+    if (t.shape.size() != 2 || !t.single_full()) return false;
+    const Piece& p = t.pieces[0];
+    if (p.src.kind != Src::NODE) return false;
+    Gen g;
+    g.wide = true;
+    int ar = g.add_atom("r", t.shape[0], false);
+    int ak = g.add_atom("k", t.shape[1], false);
+    Aff lin = aff_add(aff_atom(ar, t.shape[1]), aff_atom(ak, 1));
+    const size_t before = g.atoms.size();
+    Aff idx;
+    try {
+        idx = g.apply_view_from(p.view, 0, lin);
+    } catch (const Error&) {
+        return false;
+    }
+    if (g.atoms.size() != before) return false;
+    out.base = p.src.node;
+    out.offset = idx.c;
+    out.s0 = out.s1 = 0;
+    for (auto& x : idx.t) {
+        if (x.first == ar) out.s0 = x.second;
+        else if (x.first == ak) out.s1 = x.second;
+    }
+    if (out.s0 < 0 || out.s1 < 0) return false;
+    return true;
+}
+
+}  // namespace adhip

@@ -1,0 +1,68 @@
+// HIP C++ source generation for fused kernels.
+//
+// A kernel is described by its iteration space, the graph nodes it must produce and the set of
+// nodes that are available in memory.  Everything between is folded into one expression per
+// lane: view, permute, broadcast, index/slice and concat arithmetic becomes integer index math
+// on the loads (the reference prints the same information as div/mod chains per operand,
+// src/kernel/indexing/matrix.rs:83-132, src/kernel/helper/shape.rs:13-76), element-wise
+// operations become register arithmetic (the reference stores every intermediate,
+// src/devices/opencl/kernels/fuse_elw.rs:3-21).
+#pragma once
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "graph.hpp"
+
+namespace adhip {
+
+struct GenBuffer {
+    Node* node;         // value held densely in memory
+    std::string param;  // parameter name in the kernel signature
+    bool written = false;
+    int64_t max_index = 0;
+};
+
+struct ElwKernelSpec {
+    std::vector<Node*> outputs;  // all with the same element count; written densely
+    std::string name;
+};
+
+struct ReduceKernelSpec {
+    Node* node = nullptr;  // Op::SUM, operand [V,R]
+    std::string name;
+};
+
+struct GeneratedKernel {
+    std::string source;
+    std::string entry;
+    std::string kind;
+    std::vector<Node*> buffer_args;  // in signature order (after guard); outputs included
+    std::vector<int64_t> int_args;   // trailing integer arguments
+    unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+    unsigned lds_bytes = 0;
+    double bytes = 0, flops = 0;
+    // reductions that need a second pass: partial sums [chunks][V] written to `out`, then summed
+    int64_t chunks = 1;
+};
+
+// `in_memory(n)` tells whether node n's value can be loaded from a buffer in this kernel.
+using InMemoryFn = bool (*)(const Node*, const void*);
+
+GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members);
+// Reduce over the last dim of a [V,R] operand.  If the result needs `chunks > 1`, the kernel writes
+// partial sums laid out [chunks][V]; the caller reduces those with gen_partial_sum_kernel.
+GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks = 0);
+GeneratedKernel gen_partial_sum_kernel(int64_t V, int64_t chunks, const std::string& name);
+
+// 2-D strided access description of a matmul operand, if the reference can be expressed that way.
+struct Affine2D {
+    Node* base = nullptr;
+    int64_t offset = 0, s0 = 0, s1 = 0;
+};
+bool tref_affine2d(const TRef& t, Affine2D& out);
+
+const char* kernel_prelude();
+
+}  // namespace adhip

@@ -1,0 +1,52 @@
+// Value graph of one straight-line region of the program.
+//
+// Every compute command of the IR becomes a Node whose operands are tensor references (views,
+// possibly piecewise) onto other nodes.  Nothing is computed or stored when a node is created:
+// the lowering later decides which nodes are written to memory ("roots", one kernel output each)
+// and which are folded into the kernels that consume them.  This replaces the reference's
+// one-kernel-per-command lowering followed by three peephole fusion passes
+// (reference src/kernel/to_kernel.rs:13-106, src/kernel/fusion/*.rs).
+#pragma once
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "view.hpp"
+
+namespace adhip {
+
+enum class Op : uint8_t {
+    // leaves
+    LIVEIN,   // contents of an id's home buffer at region entry
+    UPLOAD,   // contents of a CreateMat payload kept in a read-only device buffer
+    // element-wise
+    ADD, MUL, EXP2, LOG2, SIN, RECIP, SQRT, EQ0, GT0, LT0, COPY, FILL,
+    // kernels of their own
+    SUM,  // [V,R] -> [V]
+    DOT,  // [M,K] x [K,N] -> [M,N]
+};
+
+inline bool op_is_leaf(Op o) { return o == Op::LIVEIN || o == Op::UPLOAD; }
+inline bool op_is_elw(Op o) { return o >= Op::ADD && o <= Op::FILL; }
+inline bool op_is_transcendental(Op o) { return o == Op::EXP2 || o == Op::LOG2 || o == Op::SIN; }
+const char* op_name(Op o);
+
+struct Node {
+    int id = -1;
+    Op op = Op::COPY;
+    Shape shape;
+    std::vector<TRef> in;  // operands (resolved: no SYM/NESTED sources)
+    float cval = 0.f;      // FILL
+    std::string name;      // IR id this node was bound to when created (for diagnostics / home buffers)
+    double order = 0;      // program order (creation order; helper copies sit just before their consumer)
+
+    // filled in by the lowering
+    bool root = false;        // gets a buffer
+    bool force_root = false;  // Contigious, live-out, dot operand ...
+    int buffer = -1;          // plan buffer id holding this node's dense row-major value
+    int kernel = -1;          // index of the kernel (group) that produces it
+    int last_use_kernel = -1;
+    std::string key;          // structural key for common-subexpression merging
+};
+
+}  // namespace adhip

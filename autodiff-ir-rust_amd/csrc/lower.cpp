@@ -1,0 +1,1050 @@
+#include "lower.hpp"
+
+#include <algorithm>
+#include <cctype>
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <map>
+#include <unordered_map>
+
+#include "codegen.hpp"
+#include "graph.hpp"
+
+namespace adhip {
+
+const char* fixed_kernels_source() {
+    return R"(
+extern "C" __global__ __launch_bounds__(256) void adhip_copy(const int* __restrict__ guard, float* __restrict__ dst,
+                                                             const float* __restrict__ src, unsigned long long n) {
+    if (guard && *guard == 0) return;
+    unsigned long long i = (unsigned long long)blockIdx.x * 256u + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+// One thread per output element, k ascending, one accumulator: the reference's dot kernel
+// (src/devices/opencl/kernels/dotprod.rs:23-53).  Used for small products.
+extern "C" __global__ __launch_bounds__(256) void adhip_dot_naive(const int* __restrict__ guard, float* __restrict__ c,
+                                                                  const float* __restrict__ a, const float* __restrict__ b,
+                                                                  long long m, long long n, long long k,
+                                                                  long long a_off, long long a_sm, long long a_sk,
+                                                                  long long b_off, long long b_sk, long long b_sn) {
+    if (guard && *guard == 0) return;
+    long long g = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (g >= m * n) return;
+    long long row = g / n, col = g % n;
+    float acc = 0.0f;
+    const float* pa = a + a_off + row * a_sm;
+    const float* pb = b + b_off + col * b_sn;
+    for (long long kk = 0; kk < k; ++kk) acc = __builtin_fmaf(pa[kk * a_sk], pb[kk * b_sk], acc);
+    c[g] = acc;
+}
+)";
+}
+
+namespace {
+
+bool is_control(Tag t) { return t == T_WHILE || t == T_IF || t == T_EX; }
+bool is_view_op(Tag t) { return t == T_VIEW || t == T_INDEX || t == T_CONCAT || t == T_PERMUTE || t == T_BROADCAST; }
+
+struct Binding {
+    enum Kind { NONE, HOME, VAL, CONST, ALIAS } kind = NONE;
+    Node* node = nullptr;
+    float c = 0.f;
+    TRef alias;
+    Shape shape;
+};
+
+using IdSet = std::set<std::string>;
+using RegionKey = std::pair<const Proc*, size_t>;
+
+struct Group {
+    std::vector<Node*> members;
+    int64_t n = 0;
+    enum Kind { ELW, SUM, DOT } kind = ELW;
+};
+
+struct Lowerer {
+    const Proc& prog;
+    LowerOptions opt;
+    IdSet deps;
+    IdSet cond_ids;
+    std::unique_ptr<Plan> plan{new Plan()};
+    std::unordered_map<std::string, Binding> env;
+    std::map<std::string, int> home_buf;
+    std::map<std::string, IdSet> alias_srcs;
+    std::map<RegionKey, IdSet> region_live;
+    std::vector<std::unique_ptr<Node>> arena;
+    std::map<std::string, int> kernel_by_source;
+    int kernel_counter = 0;
+    int fixed_copy = -1, fixed_dot = -1;
+
+    // per region
+    std::vector<Node*> rnodes;
+    std::map<std::string, Node*> cse;
+    std::map<std::string, Node*> livein;
+
+    Lowerer(const Proc& p, const std::vector<std::string>& d, const LowerOptions& o) : prog(p), opt(o) {
+        for (auto& s : d) deps.insert(s);
+    }
+
+    // -----------------------------------------------------------------------------------
+    // liveness over the structured program
+    // -----------------------------------------------------------------------------------
+    void collect_alias_srcs(const Proc& p) {
+        for (const Cmd& c : p.cmds) {
+            if (is_view_op(c.tag)) {
+                alias_srcs[c.res].insert(c.a);
+                if (c.tag == T_CONCAT) alias_srcs[c.res].insert(c.b);
+            }
+            if (c.tag == T_WHILE) { cond_ids.insert(c.a); collect_alias_srcs(*c.block); }
+            if (c.tag == T_IF) {
+                for (auto& arm : c.conds) { cond_ids.insert(arm.first); collect_alias_srcs(*arm.second); }
+                if (c.else_block) collect_alias_srcs(*c.else_block);
+            }
+        }
+    }
+
+    void add_use(IdSet& live, const std::string& id) {
+        if (id.empty()) return;
+        if (!live.insert(id).second) return;
+        auto it = alias_srcs.find(id);
+        if (it != alias_srcs.end())
+            for (auto& s : it->second) add_use(live, s);
+    }
+
+    void transfer_cmd(const Cmd& c, IdSet& live) {
+        switch (c.tag) {
+        case T_CREATE_MAT: case T_CREATE_CONSTANT: live.erase(c.res); break;
+        case T_ELW_MULTIPLY: case T_ELW_ADD: case T_DOT_PRODUCT:
+            live.erase(c.res); add_use(live, c.a); add_use(live, c.b); break;
+        case T_ELW_MULTIPLY_EQ: case T_ELW_ADD_EQ:
+            add_use(live, c.a); add_use(live, c.b); break;
+        case T_CONCAT:
+            live.erase(c.res); add_use(live, c.a); add_use(live, c.b); break;
+        case T_HEADING: break;
+        default:
+            if (!is_control(c.tag)) { live.erase(c.res); add_use(live, c.a); }
+        }
+    }
+
+    // Returns the live-in set of the block; records the live-out set of every region.
+    IdSet live_block(const Proc& p, const IdSet& live_out) {
+        // segment boundaries
+        std::vector<size_t> ctrl;
+        for (size_t i = 0; i < p.cmds.size(); ++i)
+            if (is_control(p.cmds[i].tag)) ctrl.push_back(i);
+        IdSet live = live_out;
+        size_t end = p.cmds.size();
+        for (size_t ci = ctrl.size() + 1; ci-- > 0;) {
+            size_t start = ci == 0 ? 0 : ctrl[ci - 1] + 1;
+            // region [start, end)
+            IdSet& rec = region_live[{&p, start}];
+            rec.insert(live.begin(), live.end());
+            for (size_t i = end; i-- > start;) transfer_cmd(p.cmds[i], live);
+            if (ci == 0) break;
+            const Cmd& c = p.cmds[ctrl[ci - 1]];
+            if (c.tag == T_EX) {
+                live.clear();
+                for (auto& d : deps) add_use(live, d);
+            } else if (c.tag == T_WHILE) {
+                IdSet L = live;
+                add_use(L, c.a);
+                for (int it = 0; it < 8; ++it) {
+                    IdSet in = live_block(*c.block, L);
+                    size_t before = L.size();
+                    for (auto& s : in) add_use(L, s);
+                    if (L.size() == before) break;
+                }
+                live_block(*c.block, L);
+                live = L;
+            } else {  // If
+                IdSet L = live;
+                for (auto& arm : c.conds) {
+                    add_use(L, arm.first);
+                    IdSet in = live_block(*arm.second, live);
+                    for (auto& s : in) add_use(L, s);
+                }
+                if (c.else_block) {
+                    IdSet in = live_block(*c.else_block, live);
+                    for (auto& s : in) add_use(L, s);
+                }
+                live = L;
+            }
+            end = ctrl[ci - 1];
+        }
+        return live;
+    }
+
+    // -----------------------------------------------------------------------------------
+    // buffers
+    // -----------------------------------------------------------------------------------
+    int home(const std::string& id, int64_t elems) {
+        auto it = home_buf.find(id);
+        if (it == home_buf.end()) {
+            PlanBuffer b;
+            b.kind = PlanBuffer::HOME;
+            b.name = id;
+            b.elems = std::max<int64_t>(elems, 1);
+            plan->buffers.push_back(b);
+            home_buf[id] = (int)plan->buffers.size() - 1;
+            return home_buf[id];
+        }
+        PlanBuffer& b = plan->buffers[it->second];
+        b.elems = std::max<int64_t>(b.elems, elems);
+        return it->second;
+    }
+
+    std::vector<std::pair<int64_t, bool>> slots;  // (elems, in use)
+    int alloc_temp(int64_t elems, const std::string& name) {
+        elems = std::max<int64_t>(elems, 1);
+        int best = -1;
+        for (size_t i = 0; i < slots.size(); ++i) {
+            if (slots[i].second) continue;
+            if (best < 0) { best = (int)i; continue; }
+            const int64_t cur = slots[best].first, cand = slots[i].first;
+            const bool cur_fits = cur >= elems, cand_fits = cand >= elems;
+            if (cand_fits && (!cur_fits || cand < cur)) best = (int)i;
+            else if (!cand_fits && !cur_fits && cand > cur) best = (int)i;
+        }
+        if (best < 0) { slots.push_back({elems, true}); best = (int)slots.size() - 1; }
+        slots[best].first = std::max(slots[best].first, elems);
+        slots[best].second = true;
+        PlanBuffer b;
+        b.kind = PlanBuffer::TEMP;
+        b.name = name;
+        b.elems = elems;
+        b.slot = best;
+        plan->buffers.push_back(b);
+        return (int)plan->buffers.size() - 1;
+    }
+    void free_temp(int buf) {
+        const PlanBuffer& b = plan->buffers[buf];
+        if (b.kind == PlanBuffer::TEMP) slots[b.slot].second = false;
+    }
+
+    // -----------------------------------------------------------------------------------
+    // graph building
+    // -----------------------------------------------------------------------------------
+    Node* new_node(Op op, const Shape& shape, std::vector<TRef> in, const std::string& name, float cval = 0.f,
+                   bool allow_cse = true) {
+        std::string key = std::string(op_name(op)) + shape_str(shape) + "(";
+        for (auto& t : in) key += tref_str(t) + ";";
+        key += ")";
+        if (op == Op::FILL) key += strf("%a", cval);
+        if (allow_cse && op != Op::LIVEIN && op != Op::UPLOAD) {
+            auto it = cse.find(key);
+            if (it != cse.end()) return it->second;
+        }
+        arena.emplace_back(new Node());
+        Node* n = arena.back().get();
+        n->id = (int)arena.size() - 1;
+        n->order = (double)n->id;
+        n->op = op;
+        n->shape = shape;
+        n->in = std::move(in);
+        n->cval = cval;
+        n->name = name;
+        n->key = key;
+        rnodes.push_back(n);
+        if (allow_cse && op != Op::LIVEIN && op != Op::UPLOAD) cse[key] = n;
+        return n;
+    }
+
+    Node* get_livein(const std::string& id) {
+        auto it = livein.find(id);
+        if (it != livein.end()) return it->second;
+        Binding& b = env[id];
+        Node* n = new_node(Op::LIVEIN, b.shape, {}, id);
+        n->buffer = home(id, numel(b.shape));
+        livein[id] = n;
+        return n;
+    }
+
+    Binding& lookup(const std::string& id) {
+        auto it = env.find(id);
+        ADHIP_CHECK(it != env.end() && it->second.kind != Binding::NONE, "id '%s' is used before it is defined", id.c_str());
+        return it->second;
+    }
+
+    TRef resolve(const TRef& t) {
+        TRef o;
+        o.shape = t.shape;
+        for (const Piece& p : t.pieces) {
+            Piece q = p;
+            if (p.src.kind == Src::SYM) {
+                Binding& b = lookup(p.src.sym);
+                if (b.kind == Binding::CONST) { q.src = Src(); q.src.kind = Src::CONST; q.src.c = b.c; }
+                else if (b.kind == Binding::VAL) { q.src = Src(); q.src.kind = Src::NODE; q.src.node = b.node; }
+                else if (b.kind == Binding::HOME) { q.src = Src(); q.src.kind = Src::NODE; q.src.node = get_livein(p.src.sym); }
+                else {  // an alias that was (re)defined after this reference was made
+                    TRef inner = resolve(b.alias);
+                    Node* c = new_node(Op::COPY, inner.shape, {inner}, p.src.sym);
+                    q.src = Src(); q.src.kind = Src::NODE; q.src.node = c;
+                }
+            } else if (p.src.kind == Src::NESTED) {
+                TRef inner = resolve(*p.src.nested);
+                Node* c = new_node(Op::COPY, inner.shape, {inner}, "");
+                q.src = Src(); q.src.kind = Src::NODE; q.src.node = c;
+            }
+            o.pieces.push_back(std::move(q));
+        }
+        return o;
+    }
+
+    // symbolic reference to id (for building aliases)
+    TRef sym_ref(const std::string& id) {
+        Binding& b = lookup(id);
+        if (b.kind == Binding::ALIAS) return b.alias;
+        return tr_sym(id, b.shape);
+    }
+
+    // resolved operand of a compute command
+    TRef operand(const std::string& id, const Shape* want_shape = nullptr) {
+        Binding& b = lookup(id);
+        TRef t;
+        switch (b.kind) {
+        case Binding::CONST: t = tr_const(b.c, want_shape ? *want_shape : b.shape); break;
+        case Binding::VAL: t = tr_node(b.node, b.shape); break;
+        case Binding::HOME: t = tr_node(get_livein(id), b.shape); break;
+        case Binding::ALIAS: t = resolve(b.alias); break;
+        default: throw Error("unreachable");
+        }
+        if (want_shape && t.shape != *want_shape) {
+            ADHIP_CHECK(numel(t.shape) == numel(*want_shape), "operand '%s' of shape %s used where %s is expected", id.c_str(),
+                        shape_str(t.shape).c_str(), shape_str(*want_shape).c_str());
+            t = tr_reshape(t, *want_shape);
+            t = resolve(t);
+        }
+        return t;
+    }
+
+    void bind_val(const std::string& id, Node* n, const Shape& shape) {
+        Binding& b = env[id];
+        b.kind = Binding::VAL;
+        b.node = n;
+        b.shape = shape;
+        b.alias = TRef();
+    }
+
+    void build_cmd(const Cmd& c, bool once) {
+        switch (c.tag) {
+        case T_HEADING: return;
+        case T_CREATE_MAT: {
+            const int64_t ne = numel(c.dims);
+            if (once && !home_buf.count(c.res)) {
+                // executed exactly once: the payload is uploaded straight into the id's own buffer
+                int hb = home(c.res, ne);
+                plan->buffers[hb].host = c.host;
+                plan->buffers[hb].host_elems = ne;
+                Binding& b = env[c.res];
+                b = Binding();
+                b.kind = Binding::HOME;
+                b.shape = c.dims;
+                livein.erase(c.res);
+            } else {
+                // inside a loop or branch: keep the payload in a read-only buffer uploaded once
+                PlanBuffer pb;
+                pb.kind = PlanBuffer::CONSTPOOL;
+                pb.name = c.res + ".init";
+                pb.elems = std::max<int64_t>(ne, 1);
+                pb.host = c.host;
+                pb.host_elems = ne;
+                plan->buffers.push_back(pb);
+                Node* n = new_node(Op::UPLOAD, c.dims, {}, c.res);
+                n->buffer = (int)plan->buffers.size() - 1;
+                bind_val(c.res, n, c.dims);
+            }
+            return;
+        }
+        case T_CREATE_CONSTANT: {
+            Binding& b = env[c.res];
+            b = Binding();
+            b.kind = Binding::CONST;
+            b.c = c.f;
+            b.shape = c.dims;
+            return;
+        }
+        case T_ELW_MULTIPLY: case T_ELW_ADD: case T_ELW_MULTIPLY_EQ: case T_ELW_ADD_EQ: {
+            const bool mul = c.tag == T_ELW_MULTIPLY || c.tag == T_ELW_MULTIPLY_EQ;
+            Binding& ba = lookup(c.a);
+            Binding& bb = lookup(c.b);
+            if (ba.kind == Binding::CONST && bb.kind == Binding::CONST) {
+                // constant (x) constant folds on the host (reference src/kernel/trackers/constant.rs:26-56;
+                // its `+=` case multiplies, the evident intent -- add -- is followed here)
+                float r = mul ? ba.c * bb.c : ba.c + bb.c;
+                Shape sh = ba.shape;
+                Binding& br = env[c.res];
+                br = Binding();
+                br.kind = Binding::CONST;
+                br.c = r;
+                br.shape = sh;
+                return;
+            }
+            // result takes a's shape (reference src/kernel/trackers/shape.rs:31-34); a constant's
+            // shape is nominal, so the tensor operand decides then
+            Shape sh = ba.kind == Binding::CONST ? bb.shape : ba.shape;
+            TRef ta = operand(c.a, &sh), tb = operand(c.b, &sh);
+            Node* n = new_node(mul ? Op::MUL : Op::ADD, sh, {ta, tb}, c.res);
+            bind_val(c.res, n, sh);
+            return;
+        }
+        case T_EQUAL_ZERO: case T_MORE_ZERO: case T_LESS_ZERO: case T_EXP2: case T_LOG2: case T_SIN: case T_RECIP:
+        case T_SQRT: case T_CONTIGIOUS: {
+            Shape sh = lookup(c.a).shape;
+            TRef ta = operand(c.a);
+            Op op = Op::COPY;
+            switch (c.tag) {
+            case T_EQUAL_ZERO: op = Op::EQ0; break;
+            case T_MORE_ZERO: op = Op::GT0; break;
+            case T_LESS_ZERO: op = Op::LT0; break;
+            case T_EXP2: op = Op::EXP2; break;
+            case T_LOG2: op = Op::LOG2; break;
+            case T_SIN: op = Op::SIN; break;
+            case T_RECIP: op = Op::RECIP; break;
+            case T_SQRT: op = Op::SQRT; break;
+            default: break;
+            }
+            Node* n = new_node(op, sh, {ta}, c.res, 0.f, c.tag != T_CONTIGIOUS);
+            if (c.tag == T_CONTIGIOUS) n->force_root = true;
+            bind_val(c.res, n, sh);
+            return;
+        }
+        case T_SUM: {
+            TRef ta = operand(c.a);
+            ADHIP_CHECK(ta.shape.size() == 2, "Sum: operand '%s' has shape %s, expected 2-D", c.a.c_str(), shape_str(ta.shape).c_str());
+            Shape sh{ta.shape[0]};
+            Node* n = new_node(Op::SUM, sh, {ta}, c.res);
+            bind_val(c.res, n, sh);
+            return;
+        }
+        case T_DOT_PRODUCT: {
+            TRef ta = operand(c.a), tb = operand(c.b);
+            ADHIP_CHECK(ta.shape.size() == 2 && tb.shape.size() == 2, "DotProduct: operands must be 2-D");
+            ADHIP_CHECK(ta.shape[1] == tb.shape[0], "DotProduct: %s x %s", shape_str(ta.shape).c_str(), shape_str(tb.shape).c_str());
+            Shape sh{ta.shape[0], tb.shape[1]};
+            Node* n = new_node(Op::DOT, sh, {ta, tb}, c.res);
+            bind_val(c.res, n, sh);
+            return;
+        }
+        case T_VIEW: case T_INDEX: case T_PERMUTE: case T_BROADCAST: case T_CONCAT: {
+            TRef a = sym_ref(c.a);
+            TRef r;
+            if (c.tag == T_VIEW) r = tr_reshape(a, c.dims);
+            else if (c.tag == T_INDEX) r = tr_index(a, c.i0, c.i1);
+            else if (c.tag == T_PERMUTE) r = tr_permute(a, c.dims);
+            else if (c.tag == T_BROADCAST) r = tr_broadcast(a, c.i0, c.i1);
+            else r = tr_concat(a, sym_ref(c.b), c.i0);
+            Binding& b = env[c.res];
+            b = Binding();
+            b.kind = Binding::ALIAS;
+            b.shape = r.shape;
+            b.alias = std::move(r);
+            return;
+        }
+        default: throw Error(strf("internal: unexpected command %s in a region", tag_name(c.tag)));
+        }
+    }
+
+    // -----------------------------------------------------------------------------------
+    // region flush: choose roots, form kernels, assign buffers, emit launches
+    // -----------------------------------------------------------------------------------
+    static void for_each_src(const Node* n, const std::function<void(Node*, const Piece&, const TRef&)>& f) {
+        for (const TRef& t : n->in)
+            for (const Piece& p : t.pieces)
+                if (p.src.kind == Src::NODE) f(p.src.node, p, t);
+    }
+
+    static bool in_mem(const Node* n) { return op_is_leaf(n->op) || n->root; }
+
+    static bool identity_piece(const Piece& p, const TRef& t) {
+        if (!t.single_full()) return false;
+        for (const Stage& s : p.view.st)
+            if (!stage_is_identity(s)) return false;
+        return true;
+    }
+
+    // in-memory nodes a root reads (through folded nodes); value = every path is an identity view
+    void collect_reads(Node* r, std::map<Node*, bool>& reads) {
+        std::map<std::pair<Node*, bool>, bool> seen;
+        std::function<void(Node*, bool)> walk = [&](Node* n, bool ident) {
+            for_each_src(n, [&](Node* s, const Piece& p, const TRef& t) {
+                bool id2 = ident && identity_piece(p, t) && numel(s->shape) == numel(n->shape);
+                if (in_mem(s)) {
+                    auto it = reads.find(s);
+                    if (it == reads.end()) reads[s] = id2;
+                    else it->second = it->second && id2;
+                } else {
+                    if (seen.insert({{s, id2}, true}).second) walk(s, id2);
+                }
+            });
+        };
+        walk(r, true);
+    }
+
+    int add_kernel(const std::string& entry, const std::string& source, const std::string& kind) {
+        std::string key = entry + "\n" + source;
+        auto it = kernel_by_source.find(key);
+        if (it != kernel_by_source.end()) return it->second;
+        KernelDef d;
+        d.entry = entry;
+        d.source = source;
+        d.kind = kind;
+        plan->kernels.push_back(std::move(d));
+        kernel_by_source[key] = (int)plan->kernels.size() - 1;
+        return (int)plan->kernels.size() - 1;
+    }
+
+    void push_launch(std::vector<Step>& out, Launch l, const std::string& kind) {
+        KernelStat st;
+        st.label = l.label;
+        st.kind = kind;
+        st.kernel = l.kernel;
+        st.bytes = l.bytes;
+        st.flops = l.flops;
+        plan->stats.push_back(st);
+        l.stat = (int)plan->stats.size() - 1;
+        Step s;
+        s.kind = Step::LAUNCH;
+        s.launch = std::move(l);
+        out.push_back(std::move(s));
+    }
+
+    void emit_copy(std::vector<Step>& out, int dst, int src, int64_t n, const std::string& label) {
+        if (fixed_copy < 0) fixed_copy = add_kernel("adhip_copy", fixed_kernels_source(), "copy");
+        Launch l;
+        l.kernel = fixed_copy;
+        l.block[0] = 256;
+        l.grid[0] = (unsigned)((n + 255) / 256);
+        Arg a; a.kind = Arg::BUF; a.buf = dst; l.args.push_back(a);
+        a.buf = src; l.args.push_back(a);
+        Arg c; c.kind = Arg::I64; c.iv = n; l.args.push_back(c);
+        l.label = label;
+        l.bytes = 8.0 * (double)n;
+        push_launch(out, l, "copy");
+    }
+
+    void flush_region(const IdSet& live, bool final_region, std::vector<Step>& out) {
+        // ---- 1. what has to be in a home buffer when the region ends
+        std::vector<std::pair<std::string, Node*>> wanted;
+        std::set<Node*> wanted_nodes;
+        auto want = [&](const std::string& id, Node* n) {
+            if (numel(n->shape) == 0) return;
+            if (op_is_leaf(n->op) || wanted_nodes.count(n)) n = new_node(Op::COPY, n->shape, {tr_node(n, n->shape)}, id, 0.f, false);
+            wanted_nodes.insert(n);
+            wanted.push_back({id, n});
+        };
+        for (const std::string& id : live) {
+            auto it = env.find(id);
+            if (it == env.end()) continue;
+            Binding& b = it->second;
+            if (b.kind == Binding::VAL) {
+                if (b.node->op == Op::LIVEIN && b.node->name == id) continue;
+                want(id, b.node);
+            } else if ((b.kind == Binding::ALIAS || b.kind == Binding::CONST) &&
+                       ((final_region && deps.count(id)) || cond_ids.count(id))) {
+                if (numel(b.shape) == 0) continue;
+                Node* n;
+                if (b.kind == Binding::CONST) n = new_node(Op::FILL, b.shape, {}, id, b.c, false);
+                else {
+                    TRef r = resolve(b.alias);
+                    n = new_node(Op::COPY, r.shape, {r}, id, 0.f, false);
+                }
+                wanted_nodes.insert(n);
+                wanted.push_back({id, n});
+            }
+        }
+        // ---- 2. needed nodes in topological order
+        std::vector<Node*> topo;
+        {
+            std::set<Node*> seen;
+            std::function<void(Node*)> dfs = [&](Node* n) {
+                if (!seen.insert(n).second) return;
+                for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
+                topo.push_back(n);
+            };
+            for (auto& w : wanted) dfs(w.second);
+        }
+        if (topo.empty()) { end_region(wanted); return; }
+        // ---- 3. forced roots
+        for (auto& w : wanted) w.second->root = true;
+        for (size_t i = 0; i < topo.size(); ++i) {
+            Node* n = topo[i];
+            if (n->op == Op::SUM || n->op == Op::DOT || n->force_root) n->root = true;
+            if (!opt.fuse && op_is_elw(n->op)) n->root = true;
+            if (numel(n->shape) == 0) n->root = false;
+        }
+        // matmul operands must be strided 2-D views of memory
+        for (size_t i = 0; i < topo.size(); ++i) {
+            Node* n = topo[i];
+            if (n->op != Op::DOT) continue;
+            for (TRef& t : n->in) {
+                Affine2D a2;
+                if (tref_affine2d(t, a2) && (op_is_leaf(a2.base->op) || op_is_elw(a2.base->op) || a2.base->root)) {
+                    if (!op_is_leaf(a2.base->op)) a2.base->root = true;
+                    continue;
+                }
+                Node* c = new_node(Op::COPY, t.shape, {t}, n->name + ".operand", 0.f, false);
+                c->root = true;
+                c->order = n->order - 0.5;
+                t = tr_node(c, t.shape);
+            }
+        }
+        // recompute topo (copies were added)
+        topo.clear();
+        {
+            std::set<Node*> seen;
+            std::function<void(Node*)> dfs = [&](Node* n) {
+                if (!seen.insert(n).second) return;
+                for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
+                topo.push_back(n);
+            };
+            for (auto& w : wanted) dfs(w.second);
+        }
+        // ---- 4. folded nodes used by several kernels: keep in memory when recomputing costs more
+        {
+            std::map<Node*, std::set<std::string>> users;
+            std::map<Node*, std::set<Node*>> bigleaves;
+            for (Node* n : topo) {  // producers first
+                if (in_mem(n)) continue;
+                std::set<Node*>& bl = bigleaves[n];
+                for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                    if (in_mem(s)) { if (numel(s->shape) * 2 >= numel(n->shape)) bl.insert(s); }
+                    else bl.insert(bigleaves[s].begin(), bigleaves[s].end());
+                });
+            }
+            for (size_t i = topo.size(); i-- > 0;) {  // consumers first
+                Node* n = topo[i];
+                std::set<std::string> mine;
+                if (n->root) mine.insert(op_is_elw(n->op) ? "E" + std::to_string(numel(n->shape)) : "K" + std::to_string(n->id));
+                else mine = users[n];
+                if (!n->root && op_is_elw(n->op) && users[n].size() >= 2 && bigleaves[n].size() >= 3) {
+                    n->root = true;
+                    mine.clear();
+                    mine.insert("E" + std::to_string(numel(n->shape)));
+                }
+                for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                    if (!in_mem(s)) users[s].insert(mine.begin(), mine.end());
+                });
+            }
+        }
+        // ---- 5. group roots into kernels
+        // kernels run in program order: it is a valid topological order, and it keeps in-place updates
+        // after the reads of the old value that precede them in the program
+        std::vector<Node*> roots;
+        for (Node* n : topo)
+            if (n->root && !op_is_leaf(n->op)) roots.push_back(n);
+        std::stable_sort(roots.begin(), roots.end(), [](Node* a, Node* b) { return a->order < b->order; });
+        std::map<Node*, std::map<Node*, bool>> reads;
+        for (Node* r : roots) collect_reads(r, reads[r]);
+        std::vector<Group> groups;
+        std::map<Node*, int> group_of;
+        for (Node* r : roots) {
+            int chosen = -1;
+            if (op_is_elw(r->op) && opt.fuse) {
+                for (int g = (int)groups.size() - 1; g >= 0; --g) {
+                    if (groups[g].kind != Group::ELW || groups[g].n != numel(r->shape)) continue;
+                    bool ok = true;
+                    for (auto& rd : reads[r]) {
+                        if (op_is_leaf(rd.first->op)) continue;
+                        int gd = group_of[rd.first];
+                        if (gd == g) { if (!rd.second) { ok = false; break; } }
+                        else if (gd > g) { ok = false; break; }
+                    }
+                    if (ok) { chosen = g; break; }
+                }
+            }
+            if (chosen < 0) {
+                Group g;
+                g.n = numel(r->shape);
+                g.kind = r->op == Op::SUM ? Group::SUM : (r->op == Op::DOT ? Group::DOT : Group::ELW);
+                groups.push_back(g);
+                chosen = (int)groups.size() - 1;
+            }
+            groups[chosen].members.push_back(r);
+            group_of[r] = chosen;
+        }
+        // ---- 6. generate code per group (no buffers needed yet)
+        struct GK { GeneratedKernel k; std::vector<GeneratedKernel> extra; std::vector<Node*> extra_nodes; };
+        std::vector<GK> gks(groups.size());
+        // reads per group, with "identity only" flags, for hazard analysis
+        std::vector<std::map<Node*, bool>> greads(groups.size());
+        for (size_t g = 0; g < groups.size(); ++g) {
+            Group& G = groups[g];
+            std::set<const Node*> members(G.members.begin(), G.members.end());
+            for (Node* m : G.members)
+                for (auto& rd : reads[m]) {
+                    if (members.count(rd.first)) continue;
+                    auto it = greads[g].find(rd.first);
+                    if (it == greads[g].end()) greads[g][rd.first] = rd.second;
+                    else it->second = it->second && rd.second;
+                }
+            std::string name = strf("k%d_%s", kernel_counter++, G.members[0]->name.empty() ? "t" : G.members[0]->name.c_str());
+            for (char& ch : name) if (!isalnum((unsigned char)ch) && ch != '_') ch = '_';
+            if (G.kind == Group::ELW) {
+                ElwKernelSpec spec;
+                spec.outputs = G.members;
+                spec.name = name;
+                gks[g].k = gen_elw_kernel(spec, members);
+            } else if (G.kind == Group::SUM) {
+                ReduceKernelSpec spec;
+                spec.node = G.members[0];
+                spec.name = name;
+                gks[g].k = gen_reduce_kernel(spec);
+                if (gks[g].k.chunks > 1) {
+                    // second pass over the partial sums [chunks][V]
+                    Node* n = G.members[0];
+                    const int64_t V = n->shape[0], C = gks[g].k.chunks;
+                    Node* partial = new_node(Op::COPY, Shape{C, V}, {}, n->name + ".partial", 0.f, false);
+                    partial->root = true;
+                    Node* fin = new_node(Op::SUM, Shape{V}, {tr_permute(tr_node(partial, Shape{C, V}), Shape{1, 0})}, n->name, 0.f, false);
+                    fin->root = true;
+                    ReduceKernelSpec s2;
+                    s2.node = fin;
+                    s2.name = name + "_fin";
+                    gks[g].extra.push_back(gen_reduce_kernel(s2, 1));
+                    gks[g].extra_nodes = {partial, fin};
+                }
+            }
+        }
+        // ---- 7. buffers: homes, temporaries, in-place hazards
+        std::map<Node*, std::string> home_of;
+        for (auto& w : wanted) home_of[w.second] = w.first;
+        std::vector<int> last_use(arena.size() + 16, -1);
+        std::map<Node*, int> last_reader;
+        for (size_t g = 0; g < groups.size(); ++g)
+            for (auto& rd : greads[g]) last_reader[rd.first] = (int)g;
+        struct Commit { int dst, src; int64_t n; std::string id; };
+        std::vector<Commit> commits;
+        std::vector<std::vector<Node*>> free_after(groups.size());
+        for (size_t g = 0; g < groups.size(); ++g) {
+            for (Node* m : groups[g].members) {
+                auto ho = home_of.find(m);
+                bool direct = false;
+                if (ho != home_of.end()) {
+                    const std::string& id = ho->second;
+                    direct = true;
+                    auto li = livein.find(id);
+                    if (li != livein.end()) {
+                        Node* old = li->second;
+                        for (size_t g2 = 0; g2 < groups.size(); ++g2) {
+                            auto it = greads[g2].find(old);
+                            if (it == greads[g2].end()) continue;
+                            if (g2 > g) direct = false;
+                            if (g2 == g && !(it->second && groups[g].kind == Group::ELW)) direct = false;
+                        }
+                    }
+                    int hb = home(id, numel(m->shape));
+                    if (direct) m->buffer = hb;
+                    else {
+                        m->buffer = alloc_temp(numel(m->shape), id + ".new");
+                        commits.push_back({hb, m->buffer, numel(m->shape), id});
+                        // released after the commits
+                    }
+                } else {
+                    m->buffer = alloc_temp(numel(m->shape), m->name + ".tmp");
+                    auto lr = last_reader.find(m);
+                    int when = lr == last_reader.end() ? (int)g : std::max(lr->second, (int)g);
+                    free_after[when].push_back(m);
+                }
+            }
+            // partial-sum scratch of chunked reductions lives only inside this group
+            for (Node* e : gks[g].extra_nodes) {
+                if (e->op == Op::COPY) e->buffer = alloc_temp(numel(e->shape), e->name);
+            }
+            for (Node* e : gks[g].extra_nodes)
+                if (e->op == Op::COPY) free_temp(e->buffer);
+            for (Node* f : free_after[g]) free_temp(f->buffer);
+        }
+        // ---- 8. launches
+        auto buf_arg = [&](Node* n) {
+            ADHIP_CHECK(n->buffer >= 0, "internal: node %d (%s, %s) has no buffer", n->id, n->name.c_str(), op_name(n->op));
+            Arg a;
+            a.kind = Arg::BUF;
+            a.buf = n->buffer;
+            return a;
+        };
+        for (size_t g = 0; g < groups.size(); ++g) {
+            Group& G = groups[g];
+            if (G.kind == Group::DOT) {
+                emit_dot(G.members[0], out);
+                continue;
+            }
+            GeneratedKernel& k = gks[g].k;
+            Launch l;
+            l.kernel = add_kernel(k.entry, k.source, k.kind);
+            memcpy(l.grid, k.grid, sizeof l.grid);
+            memcpy(l.block, k.block, sizeof l.block);
+            l.lds_bytes = k.lds_bytes;
+            l.label = k.entry;
+            l.bytes = k.bytes;
+            l.flops = k.flops;
+            if (G.kind == Group::SUM && k.chunks > 1) {
+                Node* partial = gks[g].extra_nodes[0];
+                Node* fin = gks[g].extra_nodes[1];
+                fin->buffer = G.members[0]->buffer;
+                for (size_t i = 0; i < k.buffer_args.size(); ++i)
+                    l.args.push_back(buf_arg(i == 0 ? partial : k.buffer_args[i]));
+                push_launch(out, l, k.kind);
+                GeneratedKernel& k2 = gks[g].extra[0];
+                Launch l2;
+                l2.kernel = add_kernel(k2.entry, k2.source, k2.kind);
+                memcpy(l2.grid, k2.grid, sizeof l2.grid);
+                memcpy(l2.block, k2.block, sizeof l2.block);
+                l2.label = k2.entry;
+                l2.bytes = k2.bytes;
+                l2.flops = k2.flops;
+                for (Node* n : k2.buffer_args) l2.args.push_back(buf_arg(n));
+                push_launch(out, l2, k2.kind);
+            } else {
+                for (Node* n : k.buffer_args) l.args.push_back(buf_arg(n));
+                push_launch(out, l, k.kind);
+            }
+        }
+        for (auto& c : commits) emit_copy(out, c.dst, c.src, c.n, "commit_" + c.id);
+        for (auto& c : commits) free_temp(c.src);
+        end_region(wanted);
+    }
+
+    void emit_dot(Node* n, std::vector<Step>& out) {
+        Affine2D a, b;
+        ADHIP_CHECK(tref_affine2d(n->in[0], a) && tref_affine2d(n->in[1], b), "internal: matmul operand is not a strided view");
+        const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
+        if (fixed_dot < 0) fixed_dot = add_kernel("adhip_dot_naive", fixed_kernels_source(), "dot_naive");
+        Launch l;
+        l.kernel = fixed_dot;
+        l.block[0] = 256;
+        l.grid[0] = (unsigned)((M * N + 255) / 256);
+        auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: matmul operand without buffer"); q.buf = x->buffer; return q; };
+        auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
+        l.args = {B(n), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
+        l.label = strf("dot_%s_%lldx%lldx%lld", n->name.c_str(), (long long)M, (long long)N, (long long)K);
+        l.bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
+        l.flops = 2.0 * (double)M * (double)N * (double)K;
+        push_launch(out, l, "dot_naive");
+    }
+
+    void end_region(const std::vector<std::pair<std::string, Node*>>& wanted) {
+        std::set<std::string> homed;
+        for (auto& w : wanted) homed.insert(w.first);
+        for (auto& kv : env) {
+            Binding& b = kv.second;
+            if (b.kind == Binding::VAL) {
+                const bool is_own_livein = b.node->op == Op::LIVEIN && b.node->name == kv.first;
+                if (homed.count(kv.first) || is_own_livein || numel(b.shape) == 0) { b.kind = Binding::HOME; b.node = nullptr; }
+                else { b.kind = Binding::NONE; b.node = nullptr; }
+            }
+        }
+        rnodes.clear();
+        cse.clear();
+        livein.clear();
+    }
+
+    // -----------------------------------------------------------------------------------
+    // structured walk
+    // -----------------------------------------------------------------------------------
+    int cond_buffer(const std::string& id) {
+        Binding& b = lookup(id);
+        ADHIP_CHECK(numel(b.shape) == 1, "control predicate '%s' must have one element, has shape %s", id.c_str(), shape_str(b.shape).c_str());
+        return home(id, 1);
+    }
+
+    // Recognise `x += inc; t = x + add; cond = t < 0` at the top level of a loop body.
+    bool counted_loop(const Cmd& w, Step& step) {
+        const Proc& body = *w.block;
+        std::map<std::string, float> consts;
+        for (auto& kv : env)
+            if (kv.second.kind == Binding::CONST) consts[kv.first] = kv.second.c;
+        const Cmd* lt = nullptr;
+        const Cmd* add = nullptr;
+        const Cmd* inc = nullptr;
+        std::function<bool(const Proc&)> has_ex = [&](const Proc& p) {
+            for (const Cmd& c : p.cmds) {
+                if (c.tag == T_EX) return true;
+                if (c.tag == T_WHILE && has_ex(*c.block)) return true;
+                if (c.tag == T_IF) {
+                    for (auto& arm : c.conds) if (has_ex(*arm.second)) return true;
+                    if (c.else_block && has_ex(*c.else_block)) return true;
+                }
+            }
+            return false;
+        };
+        if (has_ex(body)) return false;
+        for (const Cmd& c : body.cmds) {
+            if (c.tag == T_CREATE_CONSTANT) consts[c.res] = c.f;
+            else if ((c.tag == T_ELW_MULTIPLY || c.tag == T_ELW_ADD) && consts.count(c.a) && consts.count(c.b))
+                consts[c.res] = c.tag == T_ELW_MULTIPLY ? consts[c.a] * consts[c.b] : consts[c.a] + consts[c.b];
+            else if (!c.res.empty()) consts.erase(c.res);
+            if (c.tag == T_LESS_ZERO && c.res == w.a) lt = &c;
+        }
+        if (!lt) return false;
+        for (const Cmd& c : body.cmds)
+            if (c.tag == T_ELW_ADD && c.res == lt->a) add = &c;
+        if (!add) return false;
+        std::string x, kadd;
+        if (consts.count(add->b) && !consts.count(add->a)) { x = add->a; kadd = add->b; }
+        else if (consts.count(add->a) && !consts.count(add->b)) { x = add->b; kadd = add->a; }
+        else return false;
+        auto bx = env.find(x);
+        if (bx == env.end() || numel(bx->second.shape) != 1 || bx->second.kind == Binding::ALIAS || bx->second.kind == Binding::CONST) return false;
+        // writes to x, t, cond: exactly the pattern, in this order, all at the top level
+        int pos_inc = -1, pos_add = -1, pos_lt = -1;
+        std::function<bool(const Proc&, bool)> scan = [&](const Proc& p, bool top) -> bool {
+            for (size_t i = 0; i < p.cmds.size(); ++i) {
+                const Cmd& c = p.cmds[i];
+                if (c.tag == T_WHILE) { if (!scan(*c.block, false)) return false; continue; }
+                if (c.tag == T_IF) {
+                    for (auto& arm : c.conds) if (!scan(*arm.second, false)) return false;
+                    if (c.else_block && !scan(*c.else_block, false)) return false;
+                    continue;
+                }
+                const bool writes = c.res == x || c.res == add->res || c.res == lt->res;
+                if (!writes) continue;
+                if (!top) return false;
+                if (c.res == x) {
+                    if (c.tag != T_ELW_ADD_EQ || !consts.count(c.b) || pos_inc >= 0) return false;
+                    inc = &c; pos_inc = (int)i;
+                } else if (c.res == add->res) {
+                    if (&c != add || pos_add >= 0) return false;
+                    pos_add = (int)i;
+                } else {
+                    if (&c != lt || pos_lt >= 0) return false;
+                    pos_lt = (int)i;
+                }
+            }
+            return true;
+        };
+        if (!scan(body, true)) return false;
+        if (!(pos_inc >= 0 && pos_inc < pos_add && pos_add < pos_lt)) return false;
+        // the constants must be the values in effect at those commands: both are defined by
+        // CreateConstant / folding only, checked by `consts` above
+        step.counter_buf = home(x, 1);
+        step.counter_inc = consts[inc->b];
+        step.counter_add = consts[kadd];
+        return true;
+    }
+
+    void lower_block(const Proc& p, std::vector<Step>& out, bool once) {
+        size_t i = 0;
+        const size_t n = p.cmds.size();
+        while (true) {
+            size_t j = i;
+            while (j < n && !is_control(p.cmds[j].tag)) ++j;
+            for (size_t k = i; k < j; ++k) build_cmd(p.cmds[k], once);
+            IdSet live = region_live[{&p, i}];
+            const bool final_region = (j == n && &p == &prog) || (j < n && p.cmds[j].tag == T_EX);
+            if (final_region)
+                for (auto& d : deps) add_use(live, d);
+            flush_region(live, final_region, out);
+            if (j == n) break;
+            const Cmd& c = p.cmds[j];
+            if (c.tag == T_EX) {
+                Step s;
+                s.kind = Step::EXIT;
+                out.push_back(std::move(s));
+                break;  // nothing after EX executes
+            } else if (c.tag == T_WHILE) {
+                Step s;
+                s.kind = Step::LOOP;
+                s.cond_buf = cond_buffer(c.a);
+                counted_loop(c, s);
+                lower_block(*c.block, s.body, false);
+                out.push_back(std::move(s));
+            } else {
+                Step s;
+                s.kind = Step::BRANCH;
+                for (auto& arm : c.conds) {
+                    std::vector<Step> body;
+                    int cb = cond_buffer(arm.first);
+                    lower_block(*arm.second, body, false);
+                    s.arms.emplace_back(cb, std::move(body));
+                }
+                if (c.else_block) lower_block(*c.else_block, s.else_body, false);
+                out.push_back(std::move(s));
+            }
+            i = j + 1;
+        }
+    }
+
+    std::unique_ptr<Plan> run() {
+        collect_alias_srcs(prog);
+        IdSet end_live;
+        for (auto& d : deps) add_use(end_live, d);
+        live_block(prog, end_live);
+        lower_block(prog, plan->steps, true);
+        // results
+        for (const std::string& d : deps) {
+            auto it = env.find(d);
+            if (it == env.end()) continue;
+            auto hb = home_buf.find(d);
+            if (hb == home_buf.end()) continue;
+            ResultDesc r;
+            r.buf = hb->second;
+            r.shape = it->second.shape;
+            plan->results[d] = r;
+        }
+        for (auto& s : slots) plan->slot_elems.push_back(s.first);
+        return std::move(plan);
+    }
+};
+
+void describe_steps(const std::vector<Step>& steps, const Plan& p, int indent, std::string& o) {
+    std::string pad((size_t)indent * 2, ' ');
+    for (const Step& s : steps) {
+        switch (s.kind) {
+        case Step::LAUNCH: {
+            const Launch& l = s.launch;
+            o += pad + strf("launch %s [%s] grid=(%u,%u,%u) block=%u bytes=%.0f flops=%.0f args:", l.label.c_str(),
+                            p.kernels[l.kernel].kind.c_str(), l.grid[0], l.grid[1], l.grid[2], l.block[0], l.bytes, l.flops);
+            for (const Arg& a : l.args) {
+                if (a.kind == Arg::BUF) o += " " + p.buffers[a.buf].name + "#" + std::to_string(a.buf);
+                else if (a.kind == Arg::F32) o += strf(" %g", a.fv);
+                else o += strf(" %lld", (long long)a.iv);
+            }
+            o += "\n";
+            break;
+        }
+        case Step::LOOP:
+            o += pad + strf("while %s#%d != 0", p.buffers[s.cond_buf].name.c_str(), s.cond_buf);
+            if (s.counter_buf >= 0) o += strf("   [counted: %s += %g; cond = (%s + %g) < 0]", p.buffers[s.counter_buf].name.c_str(), s.counter_inc, p.buffers[s.counter_buf].name.c_str(), s.counter_add);
+            o += " {\n";
+            describe_steps(s.body, p, indent + 1, o);
+            o += pad + "}\n";
+            break;
+        case Step::BRANCH:
+            for (size_t i = 0; i < s.arms.size(); ++i) {
+                o += pad + strf("%s %s#%d == 1 {\n", i ? "else if" : "if", p.buffers[s.arms[i].first].name.c_str(), s.arms[i].first);
+                describe_steps(s.arms[i].second, p, indent + 1, o);
+                o += pad + "}\n";
+            }
+            if (!s.else_body.empty()) {
+                o += pad + "else {\n";
+                describe_steps(s.else_body, p, indent + 1, o);
+                o += pad + "}\n";
+            }
+            break;
+        case Step::EXIT: o += pad + "exit\n"; break;
+        }
+    }
+}
+
+}  // namespace
+
+std::string Plan::describe() const {
+    std::string o;
+    o += strf("buffers: %zu (temp slots: %zu), kernels: %zu\n", buffers.size(), slot_elems.size(), kernels.size());
+    for (size_t i = 0; i < buffers.size(); ++i) {
+        const PlanBuffer& b = buffers[i];
+        o += strf("  #%zu %s %s elems=%lld%s%s\n", i, b.kind == PlanBuffer::HOME ? "home" : (b.kind == PlanBuffer::TEMP ? "temp" : "const"),
+                  b.name.c_str(), (long long)b.elems, b.kind == PlanBuffer::TEMP ? strf(" slot=%d", b.slot).c_str() : "", b.host ? " upload" : "");
+    }
+    describe_steps(steps, *this, 0, o);
+    return o;
+}
+
+std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids, const LowerOptions& opt) {
+    Lowerer l(prog, dep_ids, opt);
+    return l.run();
+}
+
+}  // namespace adhip

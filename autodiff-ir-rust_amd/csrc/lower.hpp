@@ -1,0 +1,25 @@
+// IR -> Plan.  Replaces the reference's `to_kernel` pipeline (reference
+// src/kernel/to_kernel.rs:34-106: per-command kernels, buffer renaming, proximity reordering,
+// alloc insertion, three fusion passes) with a value-graph lowering per straight-line region.
+#pragma once
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "ir.hpp"
+#include "plan.hpp"
+
+namespace adhip {
+
+struct LowerOptions {
+    bool fuse = true;  // false: one kernel per compute command (diagnostic mode)
+};
+
+std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids,
+                                    const LowerOptions& opt = LowerOptions());
+
+// Fixed (not generated) kernels
+const char* fixed_kernels_source();
+
+}  // namespace adhip

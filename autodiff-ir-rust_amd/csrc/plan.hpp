@@ -1,0 +1,87 @@
+// The lowered program: device buffers, generated kernels and a tree of launch / loop / branch steps.
+#pragma once
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+namespace adhip {
+
+struct PlanBuffer {
+    enum Kind { HOME, TEMP, CONSTPOOL } kind = TEMP;
+    int64_t elems = 0;
+    std::string name;
+    const float* host = nullptr;  // upload source (borrowed until upload)
+    int64_t host_elems = 0;
+    int slot = -1;                // TEMP: physical slot shared with other temporaries
+};
+
+struct KernelDef {
+    std::string entry;   // symbol name
+    std::string source;  // complete HIP C++ translation unit
+    std::string kind;    // "elw", "reduce_row", "reduce_col", "dot", ...
+};
+
+struct Arg {
+    enum Kind { BUF, I32, I64, F32 } kind = I32;
+    int buf = -1;
+    int64_t off = 0;  // BUF: element offset
+    int64_t iv = 0;
+    float fv = 0.f;
+};
+
+struct Launch {
+    int kernel = -1;  // index into Plan::kernels
+    unsigned grid[3] = {1, 1, 1};
+    unsigned block[3] = {1, 1, 1};
+    unsigned lds_bytes = 0;
+    std::vector<Arg> args;  // after the leading guard pointer
+    int guard = -1;         // flag slot or -1
+    std::string label;
+    double bytes = 0, flops = 0;  // algorithmic work of one launch
+    int stat = -1;                // index into Plan::stats
+};
+
+struct Step {
+    enum Kind { LAUNCH, LOOP, BRANCH, EXIT } kind = LAUNCH;
+    Launch launch;
+    // LOOP: while (cond[0] != 0) body; trip_count >= 0 when it is known on the host
+    int cond_buf = -1;
+    int64_t trip_count = -1;
+    // counted loop: the body's only effect on the predicate is `x += inc; cond = (x + add) < 0` on a
+    // one-element buffer x, so the trip count follows from x and cond at loop entry
+    int counter_buf = -1;
+    float counter_inc = 0.f, counter_add = 0.f;
+    std::vector<Step> body;
+    // BRANCH: first arm whose cond[0] == 1 runs, else else_body
+    std::vector<std::pair<int, std::vector<Step>>> arms;
+    std::vector<Step> else_body;
+};
+
+struct KernelStat {
+    std::string label;
+    std::string kind;
+    int kernel = -1;
+    double bytes = 0, flops = 0;
+    uint64_t launches = 0;
+    double total_ms = 0;
+};
+
+struct ResultDesc {
+    int buf = -1;
+    Shape shape;
+};
+
+struct Plan {
+    std::vector<PlanBuffer> buffers;
+    std::vector<KernelDef> kernels;
+    std::vector<Step> steps;
+    std::vector<KernelStat> stats;
+    std::map<std::string, ResultDesc> results;  // kept id -> where its value lives at exit
+    std::vector<int64_t> slot_elems;            // physical temp slots
+    int n_flags = 0;
+    std::string describe() const;
+};
+
+}  // namespace adhip

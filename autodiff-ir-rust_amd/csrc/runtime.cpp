@@ -1,0 +1,523 @@
+// HIP runtime side: context, hipRTC kernel cache, device buffers, plan executor, C ABI.
+//
+// What it replaces in the reference: src/devices/opencl/device.rs (execute / proc_exec / get_tensor)
+// and src/devices/opencl/context.rs (buffers, program build, kernel cache).  Differences that matter:
+// one stream and no wait after each kernel (the reference waits on every launch, e.g.
+// kernels/binary.rs:51); the program runs once (the reference runs it twice, device.rs:68-74);
+// CreateMat payloads are uploaded once, not on every execution of their Alloc (kernels/alloc.rs:5-12);
+// counted loops cost one host synchronisation in total, not one per iteration (device.rs:133).
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/adhip.h"
+#include "ir.hpp"
+#include "lower.hpp"
+#include "plan.hpp"
+
+using namespace adhip;
+
+namespace {
+
+thread_local std::string g_tls_error;
+
+#define HIP_OK(expr)                                                                                     \
+    do {                                                                                                 \
+        hipError_t e_ = (expr);                                                                          \
+        if (e_ != hipSuccess) throw Error(strf("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__)); \
+    } while (0)
+
+struct Module {
+    hipModule_t mod = nullptr;
+    std::map<std::string, hipFunction_t> fns;
+    ~Module() {
+        if (mod) (void)hipModuleUnload(mod);
+    }
+};
+
+struct HostResult {
+    std::vector<float> data;
+    std::vector<uint64_t> dims;
+};
+
+}  // namespace
+
+struct adhip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string arch;
+    std::string last_error;
+    std::map<std::string, std::shared_ptr<Module>> modules;  // by source text
+    std::map<std::string, HostResult> results;
+    float* pinned = nullptr;  // small pinned area for predicate read-back
+    double compile_ms = 0;
+};
+
+struct adhip_program {
+    adhip_ctx* ctx = nullptr;
+    std::unique_ptr<Proc> ir;
+    std::unique_ptr<Plan> plan;
+    std::vector<void*> buf_ptr;   // per plan buffer
+    std::vector<void*> owned;     // allocations to free
+    std::vector<hipFunction_t> fn;  // per plan kernel
+    std::vector<std::shared_ptr<Module>> mods;
+    bool profiling = false;
+    bool exited = false;
+    std::vector<std::pair<int, std::pair<hipEvent_t, hipEvent_t>>> pending;  // stat index, (start, stop)
+    std::vector<hipEvent_t> event_pool;
+    std::string description;
+};
+
+namespace {
+
+std::vector<char> compile_code_object(const std::string& source, const std::string& arch_name) {
+    hiprtcProgram prog;
+    if (hiprtcCreateProgram(&prog, source.c_str(), "adhip_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+        throw Error("hiprtcCreateProgram failed");
+    std::string arch = "--offload-arch=" + arch_name;
+    // Element-wise chains keep multiply and add separate (no contraction) so that they round like
+    // the unfused operations they replace; packed-FP32 code generation is switched off.
+    const char* opts[] = {arch.c_str(), "-O3", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt",
+                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    hiprtcResult r = hiprtcCompileProgram(prog, (int)(sizeof opts / sizeof opts[0]), opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t ls = 0;
+        hiprtcGetProgramLogSize(prog, &ls);
+        std::string log(ls, '\0');
+        if (ls) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        throw Error("hipRTC compilation failed:\n" + log + "\n--- source ---\n" + source);
+    }
+    size_t cs = 0;
+    hiprtcGetCodeSize(prog, &cs);
+    std::vector<char> code(cs);
+    hiprtcGetCode(prog, code.data());
+    hiprtcDestroyProgram(&prog);
+    return code;
+}
+
+std::shared_ptr<Module> compile_module(adhip_ctx* ctx, const std::string& source) {
+    auto it = ctx->modules.find(source);
+    if (it != ctx->modules.end()) return it->second;
+    std::vector<char> code = compile_code_object(source, ctx->arch);
+    auto m = std::make_shared<Module>();
+    HIP_OK(hipModuleLoadData(&m->mod, code.data()));
+    ctx->modules[source] = m;
+    return m;
+}
+
+hipFunction_t get_function(Module& m, const std::string& entry) {
+    auto it = m.fns.find(entry);
+    if (it != m.fns.end()) return it->second;
+    hipFunction_t f;
+    HIP_OK(hipModuleGetFunction(&f, m.mod, entry.c_str()));
+    m.fns[entry] = f;
+    return f;
+}
+
+void program_free(adhip_program* p) {
+    if (!p) return;
+    if (p->ctx) (void)hipSetDevice(p->ctx->device);
+    for (auto& pe : p->pending) { (void)hipEventDestroy(pe.second.first); (void)hipEventDestroy(pe.second.second); }
+    for (auto e : p->event_pool) (void)hipEventDestroy(e);
+    for (void* q : p->owned) (void)hipFree(q);
+    delete p;
+}
+
+std::vector<std::string> dep_vector(const char* const* dep_ids, size_t n) {
+    std::vector<std::string> d;
+    for (size_t i = 0; i < n; ++i)
+        if (dep_ids && dep_ids[i]) d.emplace_back(dep_ids[i]);
+    return d;
+}
+
+adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len, const char* const* dep_ids, size_t n) {
+    HIP_OK(hipSetDevice(ctx->device));
+    std::unique_ptr<adhip_program> p(new adhip_program());
+    p->ctx = ctx;
+    p->ir = parse_program(program, len);
+    p->plan = lower_program(*p->ir, dep_vector(dep_ids, n));
+    Plan& plan = *p->plan;
+    try {
+        // kernels
+        for (const KernelDef& k : plan.kernels) {
+            auto m = compile_module(ctx, k.source);
+            p->mods.push_back(m);
+            p->fn.push_back(get_function(*m, k.entry));
+        }
+        // buffers: one allocation per home / constant buffer, one per temp slot
+        std::vector<void*> slot_ptr(plan.slot_elems.size(), nullptr);
+        for (size_t s = 0; s < plan.slot_elems.size(); ++s) {
+            void* q = nullptr;
+            HIP_OK(hipMalloc(&q, (size_t)std::max<int64_t>(plan.slot_elems[s], 1) * sizeof(float)));
+            p->owned.push_back(q);
+            slot_ptr[s] = q;
+        }
+        p->buf_ptr.resize(plan.buffers.size(), nullptr);
+        for (size_t i = 0; i < plan.buffers.size(); ++i) {
+            const PlanBuffer& b = plan.buffers[i];
+            if (b.kind == PlanBuffer::TEMP) { p->buf_ptr[i] = slot_ptr[b.slot]; continue; }
+            void* q = nullptr;
+            HIP_OK(hipMalloc(&q, (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float)));
+            p->owned.push_back(q);
+            p->buf_ptr[i] = q;
+        }
+    } catch (...) {
+        program_free(p.release());
+        throw;
+    }
+    return p.release();
+}
+
+void program_upload(adhip_program* p) {
+    adhip_ctx* ctx = p->ctx;
+    HIP_OK(hipSetDevice(ctx->device));
+    Plan& plan = *p->plan;
+    for (size_t i = 0; i < plan.buffers.size(); ++i) {
+        const PlanBuffer& b = plan.buffers[i];
+        if (b.kind == PlanBuffer::TEMP) continue;
+        if (b.host && b.host_elems > 0) {
+            HIP_OK(hipMemcpyAsync(p->buf_ptr[i], b.host, (size_t)b.host_elems * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+        } else if (b.kind == PlanBuffer::HOME) {
+            HIP_OK(hipMemsetAsync(p->buf_ptr[i], 0, (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float), ctx->stream));
+        }
+    }
+    HIP_OK(hipStreamSynchronize(ctx->stream));
+}
+
+hipEvent_t get_event(adhip_program* p) {
+    if (!p->event_pool.empty()) {
+        hipEvent_t e = p->event_pool.back();
+        p->event_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e;
+    HIP_OK(hipEventCreate(&e));
+    return e;
+}
+
+void drain_events(adhip_program* p) {
+    for (auto& pe : p->pending) {
+        float ms = 0;
+        HIP_OK(hipEventSynchronize(pe.second.second));
+        HIP_OK(hipEventElapsedTime(&ms, pe.second.first, pe.second.second));
+        KernelStat& st = p->plan->stats[pe.first];
+        st.total_ms += ms;
+        p->event_pool.push_back(pe.second.first);
+        p->event_pool.push_back(pe.second.second);
+    }
+    p->pending.clear();
+}
+
+void launch(adhip_program* p, const Launch& l) {
+    adhip_ctx* ctx = p->ctx;
+    // argument block: guard pointer, then the plan's arguments
+    const void* guard = nullptr;
+    std::vector<void*> ptrs;
+    std::vector<std::unique_ptr<char[]>> store;
+    ptrs.reserve(l.args.size() + 1);
+    ptrs.push_back((void*)&guard);
+    std::vector<uint64_t> vals(l.args.size());
+    for (size_t i = 0; i < l.args.size(); ++i) {
+        const Arg& a = l.args[i];
+        switch (a.kind) {
+        case Arg::BUF: {
+            char* base = (char*)p->buf_ptr[a.buf];
+            void* q = base + a.off * (int64_t)sizeof(float);
+            memcpy(&vals[i], &q, sizeof q);
+            break;
+        }
+        case Arg::I32: { int v = (int)a.iv; memcpy(&vals[i], &v, sizeof v); break; }
+        case Arg::I64: { long long v = a.iv; memcpy(&vals[i], &v, sizeof v); break; }
+        case Arg::F32: { memcpy(&vals[i], &a.fv, sizeof a.fv); break; }
+        }
+        ptrs.push_back(&vals[i]);
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (p->profiling) {
+        e0 = get_event(p);
+        e1 = get_event(p);
+        HIP_OK(hipEventRecord(e0, ctx->stream));
+    }
+    HIP_OK(hipModuleLaunchKernel(p->fn[l.kernel], l.grid[0], l.grid[1], l.grid[2], l.block[0], l.block[1], l.block[2],
+                                 l.lds_bytes, ctx->stream, ptrs.data(), nullptr));
+    if (p->profiling) {
+        HIP_OK(hipEventRecord(e1, ctx->stream));
+        p->pending.push_back({l.stat, {e0, e1}});
+        if (p->pending.size() > 4096) drain_events(p);
+    }
+    p->plan->stats[l.stat].launches++;
+}
+
+float read_scalar(adhip_program* p, int buf, int slot) {
+    adhip_ctx* ctx = p->ctx;
+    HIP_OK(hipMemcpyAsync(ctx->pinned + slot, p->buf_ptr[buf], sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    return 0.f;
+}
+
+void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
+    adhip_ctx* ctx = p->ctx;
+    for (const Step& s : steps) {
+        if (p->exited) return;
+        switch (s.kind) {
+        case Step::LAUNCH: launch(p, s.launch); break;
+        case Step::EXIT: p->exited = true; return;
+        case Step::LOOP: {
+            if (s.counter_buf >= 0) {
+                // counted loop: one read of (cond, x) at entry decides the trip count
+                read_scalar(p, s.cond_buf, 0);
+                read_scalar(p, s.counter_buf, 1);
+                HIP_OK(hipStreamSynchronize(ctx->stream));
+                float cond = ctx->pinned[0], x = ctx->pinned[1];
+                int64_t n = 0;
+                while (cond != 0.0f) {
+                    ++n;
+                    x = x + s.counter_inc;
+                    float t = x + s.counter_add;
+                    cond = (t < 0.0f) ? 1.0f : 0.0f;
+                    if (n > (int64_t(1) << 40)) throw Error("counted loop does not terminate");
+                    if (x + s.counter_inc == x && cond != 0.0f) throw Error("counted loop does not terminate (counter saturated)");
+                }
+                for (int64_t i = 0; i < n && !p->exited; ++i) exec_steps(p, s.body);
+            } else {
+                while (!p->exited) {
+                    read_scalar(p, s.cond_buf, 0);
+                    HIP_OK(hipStreamSynchronize(ctx->stream));
+                    if (ctx->pinned[0] == 0.0f) break;
+                    exec_steps(p, s.body);
+                }
+            }
+            break;
+        }
+        case Step::BRANCH: {
+            for (size_t i = 0; i < s.arms.size() && i < 64; ++i) read_scalar(p, s.arms[i].first, (int)i);
+            HIP_OK(hipStreamSynchronize(ctx->stream));
+            bool ran = false;
+            for (size_t i = 0; i < s.arms.size(); ++i) {
+                float v = i < 64 ? ctx->pinned[i] : 0.f;
+                if (v == 1.0f) {
+                    exec_steps(p, s.arms[i].second);
+                    ran = true;
+                    break;
+                }
+            }
+            if (!ran) exec_steps(p, s.else_body);
+            break;
+        }
+        }
+    }
+}
+
+void program_run(adhip_program* p) {
+    adhip_ctx* ctx = p->ctx;
+    HIP_OK(hipSetDevice(ctx->device));
+    p->exited = false;
+    exec_steps(p, p->plan->steps);
+    HIP_OK(hipStreamSynchronize(ctx->stream));
+    if (p->profiling) drain_events(p);
+}
+
+void program_readback(adhip_program* p) {
+    adhip_ctx* ctx = p->ctx;
+    HIP_OK(hipSetDevice(ctx->device));
+    ctx->results.clear();
+    for (auto& kv : p->plan->results) {
+        HostResult r;
+        for (auto d : kv.second.shape) r.dims.push_back((uint64_t)d);
+        const int64_t ne = numel(kv.second.shape);
+        r.data.resize((size_t)ne);
+        if (ne > 0)
+            HIP_OK(hipMemcpyAsync(r.data.data(), p->buf_ptr[kv.second.buf], (size_t)ne * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+        ctx->results[kv.first] = std::move(r);
+    }
+    HIP_OK(hipStreamSynchronize(ctx->stream));
+}
+
+template <class F>
+int guarded(adhip_ctx* ctx, F&& f) {
+    try {
+        f();
+        return 0;
+    } catch (const std::exception& e) {
+        if (ctx) ctx->last_error = e.what();
+        g_tls_error = e.what();
+        return 2;
+    } catch (...) {
+        if (ctx) ctx->last_error = "unknown error";
+        g_tls_error = "unknown error";
+        return 2;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* adhip_version(void) { return "adhip 0.1 (gfx950)"; }
+
+int adhip_create(int device_ordinal, adhip_ctx** out) {
+    if (!out) return 2;
+    *out = nullptr;
+    return guarded(nullptr, [&] {
+        int n = 0;
+        HIP_OK(hipGetDeviceCount(&n));
+        ADHIP_CHECK(device_ordinal >= 0 && device_ordinal < n, "HIP device %d not available (%d devices)", device_ordinal, n);
+        HIP_OK(hipSetDevice(device_ordinal));
+        std::unique_ptr<adhip_ctx> ctx(new adhip_ctx());
+        ctx->device = device_ordinal;
+        hipDeviceProp_t prop;
+        HIP_OK(hipGetDeviceProperties(&prop, device_ordinal));
+        std::string arch = prop.gcnArchName;
+        size_t colon = arch.find(':');
+        if (colon != std::string::npos) arch = arch.substr(0, colon);
+        ctx->arch = arch;
+        HIP_OK(hipStreamCreate(&ctx->stream));
+        HIP_OK(hipHostMalloc((void**)&ctx->pinned, 64 * sizeof(float), hipHostMallocDefault));
+        *out = ctx.release();
+    });
+}
+
+void adhip_destroy(adhip_ctx* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    ctx->modules.clear();
+    if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+const char* adhip_last_error(adhip_ctx* ctx) { return ctx ? ctx->last_error.c_str() : g_tls_error.c_str(); }
+
+int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, const char* const* dep_ids, size_t n_dep_ids) {
+    if (!ctx) return 2;
+    return guarded(ctx, [&] {
+        ctx->results.clear();
+        adhip_program* p = program_create(ctx, program, program_len, dep_ids, n_dep_ids);
+        try {
+            program_upload(p);
+            program_run(p);
+            program_readback(p);
+        } catch (...) {
+            program_free(p);
+            throw;
+        }
+        program_free(p);
+    });
+}
+
+int adhip_get_tensor(adhip_ctx* ctx, const char* id, const float** data, const uint64_t** dims, size_t* ndim) {
+    if (!ctx || !id || !data || !dims || !ndim) return 2;
+    auto it = ctx->results.find(id);
+    if (it == ctx->results.end()) return 1;
+    *data = it->second.data.data();
+    *dims = it->second.dims.data();
+    *ndim = it->second.dims.size();
+    return 0;
+}
+
+int adhip_dot_prod_shape(const uint64_t* a_dims, size_t a_ndim, const uint64_t* b_dims, size_t b_ndim, uint64_t out[2]) {
+    if (!a_dims || !b_dims || !out || a_ndim == 0 || b_ndim == 0) return 2;
+    out[0] = a_dims[0];
+    out[1] = b_dims[b_ndim - 1];
+    return 0;
+}
+
+int adhip_program_create(adhip_ctx* ctx, const uint8_t* program, size_t program_len, const char* const* dep_ids,
+                         size_t n_dep_ids, adhip_program** out) {
+    if (!ctx || !out) return 2;
+    *out = nullptr;
+    return guarded(ctx, [&] { *out = program_create(ctx, program, program_len, dep_ids, n_dep_ids); });
+}
+
+int adhip_program_upload(adhip_program* p) {
+    if (!p) return 2;
+    return guarded(p->ctx, [&] { program_upload(p); });
+}
+
+int adhip_program_run(adhip_program* p) {
+    if (!p) return 2;
+    return guarded(p->ctx, [&] { program_run(p); });
+}
+
+int adhip_program_readback(adhip_program* p) {
+    if (!p) return 2;
+    return guarded(p->ctx, [&] { program_readback(p); });
+}
+
+void adhip_program_destroy(adhip_program* p) { program_free(p); }
+
+int adhip_program_set_profiling(adhip_program* p, int enabled) {
+    if (!p) return 2;
+    p->profiling = enabled != 0;
+    return 0;
+}
+
+int adhip_program_kernel_count(adhip_program* p) { return p ? (int)p->plan->stats.size() : 0; }
+
+int adhip_program_kernel_stat(adhip_program* p, int i, char* label, size_t label_cap, uint64_t* launches, double* total_ms,
+                              double* bytes_per_launch, double* flops_per_launch) {
+    if (!p || i < 0 || i >= (int)p->plan->stats.size()) return 2;
+    const KernelStat& s = p->plan->stats[i];
+    if (label && label_cap) {
+        std::string l = s.kind + ":" + s.label;
+        snprintf(label, label_cap, "%s", l.c_str());
+    }
+    if (launches) *launches = s.launches;
+    if (total_ms) *total_ms = s.total_ms;
+    if (bytes_per_launch) *bytes_per_launch = s.bytes;
+    if (flops_per_launch) *flops_per_launch = s.flops;
+    return 0;
+}
+
+const char* adhip_program_kernel_source(adhip_program* p, int i) {
+    if (!p || i < 0 || i >= (int)p->plan->stats.size()) return "";
+    return p->plan->kernels[p->plan->stats[i].kernel].source.c_str();
+}
+
+const char* adhip_program_describe(adhip_program* p) {
+    if (!p) return "";
+    p->description = p->plan->describe();
+    return p->description.c_str();
+}
+
+int adhip_lower_describe(const uint8_t* program, size_t program_len, const char* const* dep_ids, size_t n_dep_ids, char* out,
+                         size_t out_cap) {
+    if (!out || out_cap == 0) return 2;
+    std::string text;
+    int rc = guarded(nullptr, [&] {
+        auto ir = parse_program(program, program_len);
+        auto plan = lower_program(*ir, dep_vector(dep_ids, n_dep_ids));
+        text = plan->describe();
+        const char* dump = getenv("ADHIP_DUMP_SOURCE");
+        if (dump && *dump == '1')
+            for (auto& k : plan->kernels) text += "\n// ===== " + k.entry + " [" + k.kind + "] =====\n" + k.source;
+    });
+    if (rc != 0) text = g_tls_error;
+    snprintf(out, out_cap, "%s", text.c_str());
+    return rc;
+}
+
+int adhip_compile_check(const uint8_t* program, size_t program_len, const char* const* dep_ids, size_t n_dep_ids,
+                        const char* arch, char* out, size_t out_cap) {
+    if (!out || out_cap == 0) return 2;
+    std::string text;
+    int rc = guarded(nullptr, [&] {
+        auto ir = parse_program(program, program_len);
+        auto plan = lower_program(*ir, dep_vector(dep_ids, n_dep_ids));
+        size_t bytes = 0;
+        for (auto& k : plan->kernels) bytes += compile_code_object(k.source, arch && *arch ? arch : "gfx950").size();
+        text = strf("%zu kernels compiled, %zu bytes of code objects", plan->kernels.size(), bytes);
+    });
+    if (rc != 0) text = g_tls_error;
+    snprintf(out, out_cap, "%s", text.c_str());
+    return rc;
+}
+
+}  // extern "C"
