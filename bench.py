@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Benchmark of the device path on one MI355X.
+
+A step is one pass of the hot path (`adhip_program_run`: every kernel of the lowered program, to
+EX) over one batch of synthetic input that is already resident in HBM.  The headline workload is
+BASELINE.json configs[1]: fused element-wise + broadcast, forward and backward, 8192x8192 f32.
+The other configs are measured too (shorter) and reported under "extra".
+
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "autodiff-ir-rust_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
+
+
+def timed_runs(prog, steps, warmup):
+    for _ in range(warmup):
+        prog.run()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        prog.run()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps
+
+
+def profile(prog, runs):
+    """Per-kernel average durations from HIP events recorded on the stream the kernels run on."""
+    prog.set_profiling(True)
+    before = {i: (s.launches, s.total_ms) for i, s in enumerate(prog.kernel_stats())}
+    for _ in range(runs):
+        prog.run()
+    prog.set_profiling(False)
+    out = []
+    for i, s in enumerate(prog.kernel_stats()):
+        l0, ms0 = before[i]
+        n = s.launches - l0
+        if n:
+            out.append({"kernel": s.name, "launches_per_run": n / runs, "avg_ms": (s.total_ms - ms0) / n,
+                        "bytes": s.bytes_per_launch, "flops": s.flops_per_launch})
+    return out
+
+
+def compile_resident(dev, workload):
+    proc, deps = workload.finish()
+    prog = dev.compile(proc, deps)
+    prog.upload()
+    return prog
+
+
+def cpu_baseline_fused_elw(rows, cols):
+    """The oracle (a CPU restatement of the reference's per-kernel algorithms: one operation at a
+    time, every intermediate stored) on a bounded sample of the headline workload."""
+    from adhip import workloads as W
+    from oracle.interp import OracleDevice, c_kernels
+    wl = W.fused_elw(OracleDevice(), rows, cols, seed=0)
+    t0 = time.perf_counter()
+    wl.run()
+    dt = time.perf_counter() - t0
+    return {"value": wl.algorithmic_bytes / dt / 1e9, "unit": "GB/s", "cores": int(c_kernels().ref_num_threads()),
+            "kind": "port", "sample": f"fused_elw forward+backward on {rows}x{cols} f32 ({rows}/8192 of the rows), "
+            f"{dt:.2f} s wall", "seconds": dt}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--mlp-iters", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the device path is single-device (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    from adhip import HipDevice
+    from adhip import workloads as W
+
+    dev = HipDevice(0)
+    rows = cols = 8192
+    wl = W.fused_elw(dev, rows, cols, seed=0)
+    prog = compile_resident(dev, wl)
+    ms = timed_runs(prog, args.steps, args.warmup)
+    value = wl.algorithmic_bytes / (ms * 1e-3) / 1e9
+    kstats = profile(prog, 5)
+    dom = max(kstats, key=lambda k: k["avg_ms"] * k["launches_per_run"])
+    n = rows * cols
+    # algorithmic bytes of the dominant launch: a, b, c, bias read once; y, da, db, dc written once
+    dom_alg = 4.0 * (7 * n + cols) if dom["kernel"].startswith("elw") else dom["bytes"]
+    achieved = dom_alg / (dom["avg_ms"] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom["kernel"],
+                "avg_ms": dom["avg_ms"], "algorithmic_bytes": dom_alg}
+    prog.close()
+
+    extra = {"fused_elw_kernels": kstats}
+    if not args.skip_extra:
+        # config 3: reductions
+        wl3 = W.reductions(dev, 16384, 4096, seed=0)
+        p3 = compile_resident(dev, wl3)
+        ms3 = timed_runs(p3, max(5, args.steps // 2), 2)
+        extra["reductions"] = {"ms_per_step": ms3, "GBps": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
+                               "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}
+        p3.close()
+        # config 5: tensor manipulation + data-dependent loop
+        wl5 = W.manip_loop(dev)
+        p5 = compile_resident(dev, wl5)
+        t0 = time.perf_counter()
+        p5.run()
+        ms5 = (time.perf_counter() - t0) * 1e3
+        extra["manip_loop"] = {"ms_total": ms5, "kernels": profile_once(p5)}
+        p5.close()
+        # config 4: dense MLP training
+        wl4 = W.mlp_train(dev, 4096, (4096, 4096, 4096, 1024), args.mlp_iters, seed=0)
+        p4 = compile_resident(dev, wl4)
+        p4.run()      # warm-up: compiles nothing new, touches every buffer once
+        p4.upload()   # a run consumes the loop counter; restore the initial state (not timed)
+        t0 = time.perf_counter()
+        p4.run()
+        dt4 = time.perf_counter() - t0
+        k4 = profile_once(p4)
+        for k in k4:
+            k["launches_per_run"] = k.pop("launches")
+        dot_ms = sum(k["avg_ms"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
+        dot_fl = sum(k["flops"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
+        extra["mlp_train"] = {"steps_per_s": args.mlp_iters / dt4, "ms_per_train_step": dt4 * 1e3 / args.mlp_iters,
+                              "matmul_TFLOPs": dot_fl / (dot_ms * 1e-3) / 1e12 if dot_ms else None,
+                              "matmul_frac_of_fp32_mfma_peak": dot_fl / (dot_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS if dot_ms else None,
+                              "flops_per_train_step": wl4.flops / args.mlp_iters}
+        p4.close()
+
+    cpu = None
+    if not args.skip_cpu:
+        cpu = cpu_baseline_fused_elw(1024, 8192)
+
+    line = {
+        "metric": "fused-ELW & reduce GB/s (% HBM peak); fp32 MLP train steps/s, 1 MI355X",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: fused element-wise + broadcast, forward + backward, a,b,c f32 [8192,8192], bias [8192]",
+                   "algorithmic_bytes_per_step": wl.algorithmic_bytes, "frac_of_hbm_peak": value / HBM_PEAK_GBS},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+def profile_once(prog):
+    """Re-upload the inputs and profile one complete run (for programs whose run is not idempotent)."""
+    before = {i: (s.launches, s.total_ms) for i, s in enumerate(prog.kernel_stats())}
+    prog.set_profiling(True)
+    prog.upload()
+    prog.run()
+    prog.set_profiling(False)
+    out = []
+    for i, s in enumerate(prog.kernel_stats()):
+        n = s.launches - before[i][0]
+        if n:
+            out.append({"kernel": s.name, "launches": n, "avg_ms": (s.total_ms - before[i][1]) / n,
+                        "bytes": s.bytes_per_launch, "flops": s.flops_per_launch})
+    return out
+
+
+if __name__ == "__main__":
+    main()

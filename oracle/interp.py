@@ -116,6 +116,26 @@ _UNARY_OPS = {IR.T_EXP2: 0, IR.T_LOG2: 1, IR.T_SIN: 2, IR.T_RECIP: 4, IR.T_SQRT:
               IR.T_EQUAL_ZERO: 6, IR.T_MORE_ZERO: 7, IR.T_LESS_ZERO: 8}
 
 
+def ref_binary(mul: bool, a, b, shape) -> np.ndarray:
+    """res[g] = a[g] (+|*) b[g]; either operand may be an inline constant (binary.rs:3-14)."""
+    n = int(np.prod(shape)) if len(shape) else 1
+    out = np.empty(n, dtype=np.float32)
+    if n == 0:
+        return out
+
+    def prep(x):
+        if np.ndim(x) == 0:
+            return np.full(1, x, dtype=np.float32), 0
+        x = np.asarray(x, dtype=np.float32)
+        if x.size != n:
+            x = np.broadcast_to(x, shape)
+        return np.ascontiguousarray(x).reshape(-1), 1
+
+    (pa, sa), (pb, sb) = prep(a), prep(b)
+    c_kernels().ref_binary(1 if mul else 0, _ptr(pa), sa, _ptr(pb), sb, _ptr(out), n)
+    return out
+
+
 def ref_unary(tag: int, a: np.ndarray) -> np.ndarray:
     a = np.ascontiguousarray(a, dtype=np.float32)
     out = np.empty_like(a)
@@ -234,11 +254,7 @@ class OracleDevice(Device):
         elif t in (IR.T_ELW_MULTIPLY, IR.T_ELW_ADD):
             a, b = self._operand(cmd.a), self._operand(cmd.b)
             shape = self.shape[cmd.a]                     # shape.rs:31-32: result takes a's shape
-            r = (a * b) if t == IR.T_ELW_MULTIPLY else (a + b)
-            r = np.asarray(r, dtype=np.float32)
-            if r.size != int(np.prod(shape)):
-                r = np.broadcast_to(r, shape)
-            self._store(cmd.res, shape, r)
+            self._store(cmd.res, shape, ref_binary(t == IR.T_ELW_MULTIPLY, a, b, shape))
         elif t in (IR.T_ELW_MULTIPLY_EQ, IR.T_ELW_ADD_EQ):
             if cmd.s in self.const and cmd.o in self.const:   # folded, no kernel (elw.rs:41-43)
                 if t == IR.T_ELW_MULTIPLY_EQ:
@@ -248,11 +264,7 @@ class OracleDevice(Device):
                 return
             s, o = self._operand(cmd.s), self._operand(cmd.o)
             shape = self.shape[cmd.o] if cmd.s in self.const else self.shape[cmd.s]
-            r = (s * o) if t == IR.T_ELW_MULTIPLY_EQ else (s + o)
-            r = np.asarray(r, dtype=np.float32)
-            if r.size != int(np.prod(shape)):
-                r = np.broadcast_to(r, shape)
-            self._store(cmd.s, shape, r)
+            self._store(cmd.s, shape, ref_binary(t == IR.T_ELW_MULTIPLY_EQ, s, o, shape))
         elif t in _UNARY_OPS:
             a = self._value(cmd.a)
             self._store(cmd.res, self.shape[cmd.a], ref_unary(t, a))
