@@ -9,6 +9,7 @@
 #include <unordered_map>
 
 #include "codegen.hpp"
+#include "gemm.hpp"
 #include "graph.hpp"
 
 namespace adhip {
@@ -810,13 +811,33 @@ struct Lowerer {
         Affine2D a, b;
         ADHIP_CHECK(tref_affine2d(n->in[0], a) && tref_affine2d(n->in[1], b), "internal: matmul operand is not a strided view");
         const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
+        auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: matmul operand without buffer"); q.buf = x->buffer; return q; };
+        auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
+        const bool a_unit = a.s1 == 1 || a.s0 == 1, b_unit = b.s0 == 1 || b.s1 == 1;
+        if (M * N * K >= 64 * 64 * 64 && a_unit && b_unit) {
+            // matrix-core kernel; operands keep their strides (x^T, W^T are never copied)
+            GemmConfig cfg;
+            cfg.a_kcontig = a.s1 == 1;
+            cfg.b_kcontig = b.s0 == 1;
+            const int64_t a_ld = cfg.a_kcontig ? a.s0 : a.s1, b_ld = cfg.b_kcontig ? b.s1 : b.s0;
+            cfg.edge = (M % 128) || (N % 128) || (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
+            std::string entry = strf("adhip_gemm_%c%c%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.edge ? "_edge" : "");
+            Launch l;
+            l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
+            l.block[0] = 256;
+            l.grid[0] = (unsigned)(((M + 127) / 128) * ((N + 127) / 128));
+            l.args = {B(n), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
+            l.label = strf("dot_%s_%lldx%lldx%lld", n->name.c_str(), (long long)M, (long long)N, (long long)K);
+            l.bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
+            l.flops = 2.0 * (double)M * (double)N * (double)K;
+            push_launch(out, l, "dot_mfma");
+            return;
+        }
         if (fixed_dot < 0) fixed_dot = add_kernel("adhip_dot_naive", fixed_kernels_source(), "dot_naive");
         Launch l;
         l.kernel = fixed_dot;
         l.block[0] = 256;
         l.grid[0] = (unsigned)((M * N + 255) / 256);
-        auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: matmul operand without buffer"); q.buf = x->buffer; return q; };
-        auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
         l.args = {B(n), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
         l.label = strf("dot_%s_%lldx%lldx%lld", n->name.c_str(), (long long)M, (long long)N, (long long)K);
         l.bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);

@@ -88,3 +88,97 @@ def test_manip_loop_small(shape, hip_device):
     assert_exact(got["gathered"].data, expect.reshape(-1), "gathered vs numpy")
     assert_exact(got["i"].data, ref["i"].data, "i")
     assert_close(got["r"].data, ref["r"].data, RED_RTOL * math.sqrt(n1 + n3) * iters, "r")
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 128, 384), (100, 70, 90), (128, 16, 128), (512, 512, 512), (130, 33, 257),
+                                   (64, 64, 64), (1, 300, 5), (384, 1024, 128)])
+def test_dot_forward_backward(m, k, n, hip_device):
+    """C = A.B on the matrix cores, plus the two backward products that read W^T and x^T through
+    strides (no transposed copies)."""
+    print(f"[case] dot {m}x{k}x{n}", flush=True)
+    from adhip import autodiff, dot
+    rng = np.random.default_rng(7)
+    an = rng.standard_normal((m, k), dtype=np.float32)
+    bn = rng.standard_normal((k, n), dtype=np.float32)
+
+    def build(dev):
+        autodiff.set_device(dev)
+        a = autodiff.tensor(an, [m, k])
+        b = autodiff.tensor(bn, [k, n])
+        c = dot(a, b)
+        c.forward()
+        c.backward()
+        c.val().keep()
+        autodiff.execute()
+        return {"c": c.val().get(), "da": a.grad().get(), "db": b.grad().get()}
+
+    got, ref = build(hip_device), build(OracleDevice())
+    tol = RED_RTOL * math.sqrt(max(m, k, n))
+    compare_outputs(got, ref, {}, ("close", tol))
+    a64, b64 = an.astype(np.float64), bn.astype(np.float64)
+    ones = np.ones((m, n))
+    assert_close(got["c"].data, (a64 @ b64).reshape(-1), tol, "c vs f64")
+    assert_close(got["da"].data, (ones @ b64.T).reshape(-1), tol, "da vs f64")
+    assert_close(got["db"].data, (a64.T @ ones).reshape(-1), tol, "db vs f64")
+
+
+@pytest.mark.parametrize("chain", range(6))
+def test_data_movement_chains_bit_exact(chain, hip_device):
+    """View / permute / index / broadcast / concat chains (including a non-involutive permute and a
+    reshape across a permuted boundary) against brute-force index arithmetic."""
+    print(f"[case] chain {chain}", flush=True)
+    from adhip import ir as IR
+    from test_oracle_math import CHAINS, _brute, _to_ir
+    rng = np.random.default_rng(chain)
+    x = rng.standard_normal((2, 3, 4)).astype(np.float32)
+    z = rng.standard_normal((2, 4, 2)).astype(np.float32)
+    cmds = CHAINS[chain]
+    expect = _brute(cmds, {"x": x, "z": z})
+    last = cmds[-1][-1]
+    proc = IR.IRProcedure("main", [IR.CreateMat(x.reshape(-1), [2, 3, 4], "x"), IR.CreateMat(z.reshape(-1), [2, 4, 2], "z")]
+                          + _to_ir(cmds) + [IR.Contigious(a=last, res="out"), IR.EX()])
+    hip_device.execute(proc, {"out", last})
+    got = hip_device.get_tensor("out")
+    assert got.dim == list(expect.shape)
+    assert_exact(got.data, expect.reshape(-1), "contiguous copy")
+    # a kept id that is only a view has no buffer in the reference; here it is materialised
+    assert_exact(hip_device.get_tensor(last).data, expect.reshape(-1), "kept view id")
+
+
+def test_control_flow_and_late_bound_views(hip_device):
+    print("[case] control flow", flush=True)
+    from adhip import ir as IR
+    one = np.ones(4, np.float32)
+    proc = IR.IRProcedure("main", [
+        IR.CreateMat(np.arange(4, dtype=np.float32), [2, 2], "a"), IR.CreateMat(one, [2, 2], "o"),
+        IR.Permute(a="a", p=[1, 0], res="t"), IR.ElwAddEq(s="a", o="o"), IR.Contigious(a="t", res="u"), IR.EX()])
+    hip_device.execute(proc, {"u"})
+    assert_exact(hip_device.get_tensor("u").data, np.array([1, 3, 2, 4], np.float32), "view resolved at use")
+
+    body = IR.IRProcedure("b", [IR.CreateConstant(-1.0, "m", [1]), IR.ElwAddEq(s="c", o="m"),
+                                IR.CreateConstant(2.0, "two", [1]), IR.ElwMultiplyEq(s="y", o="two")])
+    skipped = IR.IRProcedure("s", [IR.CreateConstant(100.0, "h", [1]), IR.ElwAddEq(s="y", o="h")])
+    taken = IR.IRProcedure("t", [IR.CreateConstant(0.5, "q", [1]), IR.ElwAddEq(s="y", o="q")])
+    proc = IR.IRProcedure("main", [
+        IR.CreateMat(np.array([3.0], np.float32), [1], "c"), IR.CreateMat(np.array([1.0], np.float32), [1], "y"),
+        IR.CreateMat(np.array([2.0], np.float32), [1], "nt"), IR.CreateMat(np.array([1.0], np.float32), [1], "yes"),
+        IR.While(conditional_var="c", block=body),
+        IR.If(conditions=[("nt", skipped), ("yes", taken)], else_proc=skipped),
+        IR.EX(),
+        IR.ElwAddEq(s="y", o="yes"),
+    ])
+    hip_device.execute(proc, {"y", "c", "zz"})
+    assert hip_device.get_tensor("y").data[0] == 8.5
+    assert hip_device.get_tensor("c").data[0] == 0.0
+    assert hip_device.get_tensor("zz").is_none
+
+
+def test_errors_are_reported_not_fatal(hip_device):
+    from adhip import ir as IR
+    proc = IR.IRProcedure("main", [IR.ElwAdd(a="nope", b="nope", res="y"), IR.EX()])
+    with pytest.raises(RuntimeError, match="used before it is defined"):
+        hip_device.execute(proc, {"y"})
+    # the context stays usable
+    proc = IR.IRProcedure("main", [IR.CreateMat(np.ones(3, np.float32), [3], "a"), IR.ElwAdd(a="a", b="a", res="y"), IR.EX()])
+    hip_device.execute(proc, {"y"})
+    assert_exact(hip_device.get_tensor("y").data, np.full(3, 2.0, np.float32), "y")
