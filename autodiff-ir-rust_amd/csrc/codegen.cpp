@@ -519,6 +519,7 @@ namespace {
 struct ElwBody {
     Gen g;
     std::vector<std::string> out_exprs;
+    std::vector<std::string> cs_exprs;
     std::vector<int> dim_atoms;
     Shape iter_shape;
 };
@@ -547,17 +548,87 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
     }
     for (Node* out : spec.outputs) {
         // an output is computed from its operands even though it ends up in memory
-        std::vector<Val> a;
         ADHIP_CHECK(op_is_elw(out->op), "internal: element-wise kernel asked to produce %s", op_name(out->op));
         Val v = g.gen_node(out, lin, "");
         b.out_exprs.push_back(v.expr);
+    }
+    for (auto& cs : spec.colsums) {
+        Val v = g.gen_node(cs.value, lin, "");
+        b.cs_exprs.push_back(v.expr);
     }
     return b;
 }
 
 }  // namespace
 
+int64_t elw_colsum_tiles(int64_t rows, int64_t cols) {
+    const int64_t bx = (cols / 4 + 255) / 256;
+    int64_t tiles = (1024 + bx - 1) / bx;            // four blocks per CU on 256 CUs
+    tiles = std::min<int64_t>(tiles, std::max<int64_t>(rows / 8, 1));  // but at least 8 rows per tile
+    return std::max<int64_t>(tiles, 1);
+}
+
+// Element-wise pass over a [rows, cols] space that also accumulates column sums: a thread owns 4
+// adjacent columns and walks down a tile of rows, so the sums stay in registers; one partial row per
+// tile goes to memory and a small column reduction adds the tiles in a fixed order.
+static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members) {
+    const int64_t R = spec.rows, C = spec.cols, N = R * C;
+    ADHIP_CHECK(C % 4 == 0 && R > 0, "internal: column-sum fusion needs cols %% 4 == 0");
+    for (Node* o : spec.outputs) ADHIP_CHECK(numel(o->shape) == N, "internal: fused outputs differ in size");
+    std::vector<Node*> all = spec.outputs;
+    for (auto& cs : spec.colsums) all.push_back(cs.value);
+    const bool wide = needs_wide(all);
+    ElwBody b = elw_body(spec, members, Shape{R, C}, 4, wide);
+    Gen& g = b.g;
+    const int64_t tiles = elw_colsum_tiles(R, C);
+    const int64_t TR = (R + tiles - 1) / tiles;
+    GeneratedKernel k;
+    k.kind = "elw_colsum";
+    k.entry = spec.name;
+    std::string sig = "const int* __restrict__ guard";
+    std::vector<Node*> order;
+    const char* rq = spec.no_alias ? "__restrict__ " : "";
+    for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* %so%zu", rq, i); order.push_back(spec.outputs[i]); }
+    for (size_t i = 0; i < spec.colsums.size(); ++i) { sig += strf(", float* %sq%zu", rq, i); order.push_back(spec.colsums[i].partial); }
+    for (auto& gb : g.bufs) { sig += strf(", const float* %s%s", rq, gb.param.c_str()); order.push_back(gb.node); }
+    const char* it = g.idx_t();
+    const char* sfx = wide ? "ull" : "u";
+    std::string src = kernel_prelude();
+    src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+    src += "    if (guard && *guard == 0) return;\n";
+    src += strf("    const %s c1 = (%s)blockIdx.x * 256u + threadIdx.x;\n", it, it);
+    src += strf("    if (c1 >= %lld%s) return;\n", (long long)(C / 4), sfx);
+    src += strf("    const %s row0 = (%s)blockIdx.y * %lld%s;\n", it, it, (long long)TR, sfx);
+    src += strf("    const %s row1 = min(row0 + %lld%s, (%s)%lld%s);\n", it, (long long)TR, sfx, it, (long long)R, sfx);
+    for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("    float cs%zu[4] = {0.f, 0.f, 0.f, 0.f};\n", i);
+    src += strf("#pragma unroll 2\n    for (%s c0 = row0; c0 < row1; ++c0) {\n", it);
+    src += join(g.codeA, "        ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("        float w%zu[4];\n", i);
+    src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+    src += join(g.codeB, "            ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
+    for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("            cs%zu[j] += %s;\n", i, b.cs_exprs[i].c_str());
+    src += "        }\n";
+    for (size_t i = 0; i < spec.outputs.size(); ++i)
+        src += strf("        { float4_t q = {w%zu[0], w%zu[1], w%zu[2], w%zu[3]}; *(float4_t*)(o%zu + (c0 * %lld%s + c1 * 4u)) = q; }\n", i, i, i, i, i, (long long)C, sfx);
+    src += "    }\n";
+    for (size_t i = 0; i < spec.colsums.size(); ++i)
+        src += strf("    { float4_t q = {cs%zu[0], cs%zu[1], cs%zu[2], cs%zu[3]}; *(float4_t*)(q%zu + ((%s)blockIdx.y * %lld%s + c1 * 4u)) = q; }\n", i, i, i, i, i, it, (long long)C, sfx);
+    src += "}\n";
+    k.source = src;
+    k.buffer_args = order;
+    k.block[0] = 256;
+    k.grid[0] = (unsigned)((C / 4 + 255) / 256);
+    k.grid[1] = (unsigned)tiles;
+    k.chunks = tiles;
+    k.bytes = 4.0 * (double)N * (double)spec.outputs.size() + 4.0 * (double)tiles * C * spec.colsums.size();
+    for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), N);
+    k.flops = (g.flops + spec.colsums.size()) * (double)N;
+    return k;
+}
+
 GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members) {
+    if (!spec.colsums.empty()) return gen_elw_colsum_kernel(spec, members);
     ADHIP_CHECK(!spec.outputs.empty(), "internal: element-wise kernel without outputs");
     const int64_t N = numel(spec.outputs[0]->shape);
     for (Node* o : spec.outputs) ADHIP_CHECK(numel(o->shape) == N, "internal: fused outputs differ in size");
@@ -713,8 +784,9 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         RedBody b = red_body(n, layout, vec, wide);
         Gen& g = b.g;
         const int64_t RV = R / vec;
-        // threads per row
-        int T = RV <= 64 ? 64 : (RV <= 512 ? 64 : 256);
+        // threads per row: one wavefront per row (no barrier, no LDS) up to 8192 elements, a whole
+        // block beyond that
+        int T = RV <= 2048 ? 64 : 256;
         if (V < 64 && RV >= 4096) T = 256;
         const int rows_per_block = 256 / T;
         // split long rows over several blocks when there are too few rows to fill the GPU
@@ -736,8 +808,13 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += "    const unsigned chunk = blockIdx.y;\n";
         src += strf("    const bool row_ok = x < %lld%s;\n", (long long)V, wide ? "ull" : "u");
         src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = 0.0f;\n", vec, vec);
-        src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)RV);
-        src += strf("    if (row_ok) for (%s yv = (%s)chunk * %lldu + lane; yv < y_end; yv += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, T);
+        if (chunks == 1) {
+            // constant trip count: the loads of several iterations can be in flight together
+            src += strf("    if (row_ok)\n#pragma unroll 8\n    for (%s yv = lane; yv < %lldu; yv += %du) {\n", g.idx_t(), (long long)RV, T);
+        } else {
+            src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)RV);
+            src += strf("    if (row_ok)\n#pragma unroll 4\n    for (%s yv = (%s)chunk * %lldu + lane; yv < y_end; yv += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, T);
+        }
         src += join(g.codeA, "        ");
         if (vec > 1) src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
         else src += "        { const int j = 0;\n";
@@ -763,7 +840,8 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), V * R);
         k.flops = (g.flops + 1) * (double)V * (double)R;
     } else {
-        vec = (V % 4 == 0 && V >= 1024) ? 4 : 1;
+        // one column per thread when the problem is small (more blocks beat wider loads there)
+        vec = (V % 4 == 0 && V >= 1024 && V * R >= (int64_t(1) << 22)) ? 4 : 1;
         RedBody b = red_body(n, layout, vec, wide);
         Gen& g = b.g;
         const int64_t XV = V / vec;

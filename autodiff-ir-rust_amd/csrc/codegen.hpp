@@ -25,8 +25,17 @@ struct GenBuffer {
 };
 
 struct ElwKernelSpec {
-    std::vector<Node*> outputs;  // all with the same element count; written densely
+    std::vector<Node*> outputs;  // all with the same element count; written densely (may be empty with colsums)
     std::string name;
+    // Column sums produced by the same pass: the iteration space is viewed as [rows, cols]; for every
+    // entry the kernel also writes partial sums over a tile of rows of `value` (an element-wise node
+    // with rows*cols elements) to a [tiles][cols] buffer (`partial`).  The caller adds the partials.
+    struct ColSum { Node* value; Node* partial; };
+    std::vector<ColSum> colsums;
+    int64_t rows = 0, cols = 0;
+    // true when no output buffer can be one of the input buffers (no in-place update in this kernel):
+    // pointers are then declared __restrict__, which lets loads move ahead of earlier stores
+    bool no_alias = false;
 };
 
 struct ReduceKernelSpec {
@@ -44,6 +53,7 @@ struct GeneratedKernel {
     unsigned lds_bytes = 0;
     double bytes = 0, flops = 0;
     // reductions that need a second pass: partial sums [chunks][V] written to `out`, then summed
+    // (for element-wise kernels with column sums: the number of row tiles)
     int64_t chunks = 1;
 };
 
@@ -54,7 +64,8 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
 // Reduce over the last dim of a [V,R] operand.  If the result needs `chunks > 1`, the kernel writes
 // partial sums laid out [chunks][V]; the caller reduces those with gen_partial_sum_kernel.
 GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks = 0);
-GeneratedKernel gen_partial_sum_kernel(int64_t V, int64_t chunks, const std::string& name);
+// Number of row tiles an element-wise kernel with column sums over [rows, cols] will use.
+int64_t elw_colsum_tiles(int64_t rows, int64_t cols);
 
 // 2-D strided access description of a matmul operand, if the reference can be expressed that way.
 struct Affine2D {

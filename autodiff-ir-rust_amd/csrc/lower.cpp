@@ -23,6 +23,24 @@ extern "C" __global__ __launch_bounds__(256) void adhip_copy(const int* __restri
     if (i < n) dst[i] = src[i];
 }
 
+// Control-flow flags for device-predicated blocks (one thread).
+//   mode 0 (loop):  flags[slot] = parent && cond[0] != 0
+//   mode 1 (arm):   flags[slot] = parent && !flags[taken] && cond[0] == 1; sets flags[taken] when it fires
+//   mode 2 (else):  flags[slot] = parent && !flags[taken]
+//   mode 3 (clear): flags[slot] = 0
+extern "C" __global__ void adhip_flag(int* __restrict__ flags, int slot, int parent, const float* __restrict__ cond,
+                                      int mode, int taken) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const int p = parent < 0 ? 1 : flags[parent];
+    int v = 0;
+    if (mode == 0) v = p && (cond[0] != 0.0f);
+    else if (mode == 1) {
+        v = p && !flags[taken] && (cond[0] == 1.0f);
+        if (v) flags[taken] = 1;
+    } else if (mode == 2) v = p && !flags[taken];
+    flags[slot] = v;
+}
+
 // One thread per output element, k ascending, one accumulator: the reference's dot kernel
 // (src/devices/opencl/kernels/dotprod.rs:23-53).  Used for small products.
 extern "C" __global__ __launch_bounds__(256) void adhip_dot_naive(const int* __restrict__ guard, float* __restrict__ c,
@@ -63,6 +81,10 @@ struct Group {
     std::vector<Node*> members;
     int64_t n = 0;
     enum Kind { ELW, SUM, DOT } kind = ELW;
+    // column sums computed by this element-wise kernel: (value node, SUM node that wanted it)
+    std::vector<std::pair<Node*, Node*>> colsums;
+    int64_t cs_rows = 0, cs_cols = 0;
+    bool dead = false;  // its only member was absorbed by another group
 };
 
 struct Lowerer {
@@ -79,6 +101,7 @@ struct Lowerer {
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
     int fixed_copy = -1, fixed_dot = -1;
+    int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
 
     // per region
     std::vector<Node*> rnodes;
@@ -146,8 +169,10 @@ struct Lowerer {
             if (ci == 0) break;
             const Cmd& c = p.cmds[ctrl[ci - 1]];
             if (c.tag == T_EX) {
+                // kept views are materialised by the region that ends here; their sources need not
+                // outlive it, so no alias closure
                 live.clear();
-                for (auto& d : deps) add_use(live, d);
+                for (auto& d : deps) live.insert(d);
             } else if (c.tag == T_WHILE) {
                 IdSet L = live;
                 add_use(L, c.a);
@@ -465,8 +490,22 @@ struct Lowerer {
         return true;
     }
 
+    // A SUM whose operand is the transpose of an element-wise value E seen as [R, V] (a sum over the
+    // rows of E: `x.sum(0)`, bias gradients) can be produced by the pass that computes E.
+    static Node* colsum_source(const Node* s, int64_t& rows, int64_t& cols) {
+        if (s->op != Op::SUM) return nullptr;
+        Affine2D a;
+        if (!tref_affine2d(s->in[0], a)) return nullptr;
+        const int64_t V = s->in[0].shape[0], R = s->in[0].shape[1];
+        if (!op_is_elw(a.base->op) || a.offset != 0 || a.s0 != 1 || a.s1 != V) return nullptr;
+        if (numel(a.base->shape) != V * R || V % 4 != 0 || R < 16 || V * R < (int64_t(1) << 16)) return nullptr;
+        rows = R;
+        cols = V;
+        return a.base;
+    }
+
     // in-memory nodes a root reads (through folded nodes); value = every path is an identity view
-    void collect_reads(Node* r, std::map<Node*, bool>& reads) {
+    void collect_reads(Node* r, std::map<Node*, bool>& reads, std::set<Node*>* folded = nullptr) {
         std::map<std::pair<Node*, bool>, bool> seen;
         std::function<void(Node*, bool)> walk = [&](Node* n, bool ident) {
             for_each_src(n, [&](Node* s, const Piece& p, const TRef& t) {
@@ -476,6 +515,7 @@ struct Lowerer {
                     if (it == reads.end()) reads[s] = id2;
                     else it->second = it->second && id2;
                 } else {
+                    if (folded && id2) folded->insert(s);
                     if (seen.insert({{s, id2}, true}).second) walk(s, id2);
                 }
             });
@@ -505,6 +545,7 @@ struct Lowerer {
         st.flops = l.flops;
         plan->stats.push_back(st);
         l.stat = (int)plan->stats.size() - 1;
+        l.guard = cur_guard;
         Step s;
         s.kind = Step::LAUNCH;
         s.launch = std::move(l);
@@ -549,6 +590,23 @@ struct Lowerer {
                 if (b.kind == Binding::CONST) n = new_node(Op::FILL, b.shape, {}, id, b.c, false);
                 else {
                     TRef r = resolve(b.alias);
+                    // a kept view that is just another name for a whole computed value (same linear
+                    // layout) needs no copy: that value is written straight into this id's buffer
+                    if (r.single_full() && r.pieces[0].src.kind == Src::NODE && identity_piece(r.pieces[0], r) &&
+                        !op_is_leaf(r.pieces[0].src.node->op) && numel(r.pieces[0].src.node->shape) == numel(r.shape) &&
+                        !wanted_nodes.count(r.pieces[0].src.node)) {
+                        bool bound_elsewhere = false;  // ... unless the value must also live under its own id
+                        for (const std::string& other : live) {
+                            auto io = env.find(other);
+                            if (io != env.end() && io->second.kind == Binding::VAL && io->second.node == r.pieces[0].src.node) bound_elsewhere = true;
+                        }
+                        if (!bound_elsewhere) {
+                            n = r.pieces[0].src.node;
+                            wanted_nodes.insert(n);
+                            wanted.push_back({id, n});
+                            continue;
+                        }
+                    }
                     n = new_node(Op::COPY, r.shape, {r}, id, 0.f, false);
                 }
                 wanted_nodes.insert(n);
@@ -617,7 +675,9 @@ struct Lowerer {
             for (size_t i = topo.size(); i-- > 0;) {  // consumers first
                 Node* n = topo[i];
                 std::set<std::string> mine;
-                if (n->root) mine.insert(op_is_elw(n->op) ? "E" + std::to_string(numel(n->shape)) : "K" + std::to_string(n->id));
+                int64_t csr = 0, csc = 0;
+                if (n->root && opt.fuse && colsum_source(n, csr, csc)) mine.insert("E" + std::to_string(csr * csc));
+                else if (n->root) mine.insert(op_is_elw(n->op) ? "E" + std::to_string(numel(n->shape)) : "K" + std::to_string(n->id));
                 else mine = users[n];
                 if (!n->root && op_is_elw(n->op) && users[n].size() >= 2 && bigleaves[n].size() >= 3) {
                     n->root = true;
@@ -637,7 +697,8 @@ struct Lowerer {
             if (n->root && !op_is_leaf(n->op)) roots.push_back(n);
         std::stable_sort(roots.begin(), roots.end(), [](Node* a, Node* b) { return a->order < b->order; });
         std::map<Node*, std::map<Node*, bool>> reads;
-        for (Node* r : roots) collect_reads(r, reads[r]);
+        std::map<Node*, std::set<Node*>> folded_in;  // per root: folded nodes it evaluates at its own index
+        for (Node* r : roots) collect_reads(r, reads[r], &folded_in[r]);
         std::vector<Group> groups;
         std::map<Node*, int> group_of;
         for (Node* r : roots) {
@@ -665,13 +726,48 @@ struct Lowerer {
             groups[chosen].members.push_back(r);
             group_of[r] = chosen;
         }
+        // ---- 5b. column sums ride along with the element-wise pass that computes their operand
+        if (opt.fuse) {
+            for (size_t gs = 0; gs < groups.size(); ++gs) {
+                if (groups[gs].kind != Group::SUM) continue;
+                Node* S = groups[gs].members[0];
+                int64_t R = 0, C = 0;
+                Node* E = colsum_source(S, R, C);
+                if (!E) continue;
+                int target = -1;
+                for (size_t g = 0; g < groups.size() && target < 0; ++g) {
+                    Group& G = groups[g];
+                    if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
+                    if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
+                    for (Node* m : G.members)
+                        if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
+                }
+                if (target < 0) continue;
+                // everything that reads S must run after the pass that now produces it
+                bool ok = true;
+                for (size_t g = 0; g < groups.size(); ++g) {
+                    if (groups[g].dead) continue;
+                    for (Node* m : groups[g].members)
+                        if (reads[m].count(S) && (int)g <= target) ok = false;
+                }
+                if (!ok) continue;
+                groups[target].colsums.push_back({E, S});
+                groups[target].cs_rows = R;
+                groups[target].cs_cols = C;
+                groups[gs].dead = true;
+                group_of[S] = target;
+            }
+        }
         // ---- 6. generate code per group (no buffers needed yet)
+        std::map<Node*, std::string> home_of_early;
+        for (auto& w : wanted) home_of_early[w.second] = w.first;
         struct GK { GeneratedKernel k; std::vector<GeneratedKernel> extra; std::vector<Node*> extra_nodes; };
         std::vector<GK> gks(groups.size());
         // reads per group, with "identity only" flags, for hazard analysis
         std::vector<std::map<Node*, bool>> greads(groups.size());
         for (size_t g = 0; g < groups.size(); ++g) {
             Group& G = groups[g];
+            if (G.dead) continue;
             std::set<const Node*> members(G.members.begin(), G.members.end());
             for (Node* m : G.members)
                 for (auto& rd : reads[m]) {
@@ -686,6 +782,31 @@ struct Lowerer {
                 ElwKernelSpec spec;
                 spec.outputs = G.members;
                 spec.name = name;
+                spec.rows = G.cs_rows;
+                spec.cols = G.cs_cols;
+                // outputs can only share a buffer with an input through an in-place update of a live id
+                spec.no_alias = true;
+                for (Node* m : G.members) {
+                    auto ho = home_of_early.find(m);
+                    if (ho == home_of_early.end()) continue;
+                    auto li = livein.find(ho->second);
+                    if (li != livein.end() && greads[g].count(li->second)) spec.no_alias = false;
+                }
+                for (auto& cs : G.colsums) {
+                    const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
+                    Node* S = cs.second;
+                    Node* partial = new_node(Op::COPY, Shape{tiles, G.cs_cols}, {}, S->name + ".partial", 0.f, false);
+                    partial->root = true;
+                    Node* fin = new_node(Op::SUM, Shape{G.cs_cols}, {tr_permute(tr_node(partial, Shape{tiles, G.cs_cols}), Shape{1, 0})}, S->name, 0.f, false);
+                    fin->root = true;
+                    spec.colsums.push_back({cs.first, partial});
+                    ReduceKernelSpec s2;
+                    s2.node = fin;
+                    s2.name = name + "_cs" + std::to_string(gks[g].extra.size());
+                    gks[g].extra.push_back(gen_reduce_kernel(s2, 1));
+                    gks[g].extra_nodes.push_back(partial);
+                    gks[g].extra_nodes.push_back(fin);
+                }
                 gks[g].k = gen_elw_kernel(spec, members);
             } else if (G.kind == Group::SUM) {
                 ReduceKernelSpec spec;
@@ -714,12 +835,16 @@ struct Lowerer {
         std::vector<int> last_use(arena.size() + 16, -1);
         std::map<Node*, int> last_reader;
         for (size_t g = 0; g < groups.size(); ++g)
-            for (auto& rd : greads[g]) last_reader[rd.first] = (int)g;
+            if (!groups[g].dead)
+                for (auto& rd : greads[g]) last_reader[rd.first] = (int)g;
         struct Commit { int dst, src; int64_t n; std::string id; };
         std::vector<Commit> commits;
         std::vector<std::vector<Node*>> free_after(groups.size());
         for (size_t g = 0; g < groups.size(); ++g) {
-            for (Node* m : groups[g].members) {
+            if (groups[g].dead) continue;
+            std::vector<Node*> produced = groups[g].members;
+            for (auto& cs : groups[g].colsums) produced.push_back(cs.second);
+            for (Node* m : produced) {
                 auto ho = home_of.find(m);
                 bool direct = false;
                 if (ho != home_of.end()) {
@@ -728,11 +853,13 @@ struct Lowerer {
                     auto li = livein.find(id);
                     if (li != livein.end()) {
                         Node* old = li->second;
+                        const bool is_member = std::find(groups[g].members.begin(), groups[g].members.end(), m) != groups[g].members.end();
                         for (size_t g2 = 0; g2 < groups.size(); ++g2) {
+                            if (groups[g2].dead) continue;
                             auto it = greads[g2].find(old);
                             if (it == greads[g2].end()) continue;
                             if (g2 > g) direct = false;
-                            if (g2 == g && !(it->second && groups[g].kind == Group::ELW)) direct = false;
+                            if (g2 == g && !(it->second && groups[g].kind == Group::ELW && is_member)) direct = false;
                         }
                     }
                     int hb = home(id, numel(m->shape));
@@ -765,13 +892,35 @@ struct Lowerer {
             a.buf = n->buffer;
             return a;
         };
+        auto launch_generated = [&](GeneratedKernel& gk) {
+            Launch l2;
+            l2.kernel = add_kernel(gk.entry, gk.source, gk.kind);
+            memcpy(l2.grid, gk.grid, sizeof l2.grid);
+            memcpy(l2.block, gk.block, sizeof l2.block);
+            l2.lds_bytes = gk.lds_bytes;
+            l2.label = gk.entry;
+            l2.bytes = gk.bytes;
+            l2.flops = gk.flops;
+            for (Node* n : gk.buffer_args) l2.args.push_back(buf_arg(n));
+            push_launch(out, l2, gk.kind);
+        };
         for (size_t g = 0; g < groups.size(); ++g) {
             Group& G = groups[g];
+            if (G.dead) continue;
             if (G.kind == Group::DOT) {
                 emit_dot(G.members[0], out);
                 continue;
             }
             GeneratedKernel& k = gks[g].k;
+            if (G.kind == Group::ELW && !G.colsums.empty()) {
+                launch_generated(k);
+                for (size_t i = 0; i < G.colsums.size(); ++i) {
+                    Node* fin = gks[g].extra_nodes[2 * i + 1];
+                    fin->buffer = G.colsums[i].second->buffer;
+                    launch_generated(gks[g].extra[i]);
+                }
+                continue;
+            }
             Launch l;
             l.kernel = add_kernel(k.entry, k.source, k.kind);
             memcpy(l.grid, k.grid, sizeof l.grid);
@@ -945,6 +1094,18 @@ struct Lowerer {
         return true;
     }
 
+    static bool has_loop_or_exit(const Proc& p) {
+        for (const Cmd& c : p.cmds) {
+            if (c.tag == T_EX || c.tag == T_WHILE) return true;
+            if (c.tag == T_IF) {
+                for (auto& arm : c.conds)
+                    if (has_loop_or_exit(*arm.second)) return true;
+                if (c.else_block && has_loop_or_exit(*c.else_block)) return true;
+            }
+        }
+        return false;
+    }
+
     void lower_block(const Proc& p, std::vector<Step>& out, bool once) {
         size_t i = 0;
         const size_t n = p.cmds.size();
@@ -955,7 +1116,7 @@ struct Lowerer {
             IdSet live = region_live[{&p, i}];
             const bool final_region = (j == n && &p == &prog) || (j < n && p.cmds[j].tag == T_EX);
             if (final_region)
-                for (auto& d : deps) add_use(live, d);
+                for (auto& d : deps) live.insert(d);
             flush_region(live, final_region, out);
             if (j == n) break;
             const Cmd& c = p.cmds[j];
@@ -968,19 +1129,43 @@ struct Lowerer {
                 Step s;
                 s.kind = Step::LOOP;
                 s.cond_buf = cond_buffer(c.a);
-                counted_loop(c, s);
+                s.parent_guard = cur_guard;
+                const bool counted = counted_loop(c, s);
+                const int saved = cur_guard;
+                // a data-dependent loop whose body has no inner loop and no exit runs device-predicated
+                if (!counted && cur_guard < 0 && !has_loop_or_exit(*c.block)) {
+                    s.flag_slot = plan->n_flags++;
+                    cur_guard = s.flag_slot;
+                }
                 lower_block(*c.block, s.body, false);
+                cur_guard = saved;
                 out.push_back(std::move(s));
             } else {
                 Step s;
                 s.kind = Step::BRANCH;
+                s.parent_guard = cur_guard;
+                const int saved = cur_guard;
+                const bool predicated = cur_guard >= 0;  // inside a predicated loop the host cannot decide
+                if (predicated) s.taken_slot = plan->n_flags++;
                 for (auto& arm : c.conds) {
                     std::vector<Step> body;
                     int cb = cond_buffer(arm.first);
+                    if (predicated) {
+                        s.arm_slots.push_back(plan->n_flags++);
+                        cur_guard = s.arm_slots.back();
+                    }
                     lower_block(*arm.second, body, false);
+                    cur_guard = saved;
                     s.arms.emplace_back(cb, std::move(body));
                 }
-                if (c.else_block) lower_block(*c.else_block, s.else_body, false);
+                if (c.else_block) {
+                    if (predicated) {
+                        s.else_slot = plan->n_flags++;
+                        cur_guard = s.else_slot;
+                    }
+                    lower_block(*c.else_block, s.else_body, false);
+                    cur_guard = saved;
+                }
                 out.push_back(std::move(s));
             }
             i = j + 1;
@@ -990,7 +1175,7 @@ struct Lowerer {
     std::unique_ptr<Plan> run() {
         collect_alias_srcs(prog);
         IdSet end_live;
-        for (auto& d : deps) add_use(end_live, d);
+        for (auto& d : deps) end_live.insert(d);
         live_block(prog, end_live);
         lower_block(prog, plan->steps, true);
         // results
@@ -1027,6 +1212,7 @@ void describe_steps(const std::vector<Step>& steps, const Plan& p, int indent, s
         }
         case Step::LOOP:
             o += pad + strf("while %s#%d != 0", p.buffers[s.cond_buf].name.c_str(), s.cond_buf);
+            if (s.flag_slot >= 0) o += strf("   [device-predicated, flag %d]", s.flag_slot);
             if (s.counter_buf >= 0) o += strf("   [counted: %s += %g; cond = (%s + %g) < 0]", p.buffers[s.counter_buf].name.c_str(), s.counter_inc, p.buffers[s.counter_buf].name.c_str(), s.counter_add);
             o += " {\n";
             describe_steps(s.body, p, indent + 1, o);

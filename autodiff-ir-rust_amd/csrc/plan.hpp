@@ -57,6 +57,14 @@ struct Step {
     // BRANCH: first arm whose cond[0] == 1 runs, else else_body
     std::vector<std::pair<int, std::vector<Step>>> arms;
     std::vector<Step> else_body;
+    // Device-predicated execution.  A data-dependent LOOP with flag_slot >= 0 is enqueued several
+    // iterations ahead: a one-thread kernel latches `parent && cond != 0` into flags[flag_slot] at the
+    // top of every iteration and every kernel of the body returns at once when its flag is 0, so
+    // iterations enqueued past the end of the loop change nothing.  A BRANCH inside such a loop cannot
+    // be decided on the host either: each arm gets a flag (arm_slots / else_slot, `taken_slot` records
+    // that an earlier arm ran).  parent_guard is the flag of the enclosing predicated block or -1.
+    int flag_slot = -1, parent_guard = -1, taken_slot = -1, else_slot = -1;
+    std::vector<int> arm_slots;
 };
 
 struct KernelStat {

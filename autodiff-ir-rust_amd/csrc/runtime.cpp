@@ -70,6 +70,9 @@ struct adhip_program {
     std::vector<std::shared_ptr<Module>> mods;
     bool profiling = false;
     bool exited = false;
+    int* flags = nullptr;            // device flags of predicated blocks
+    hipFunction_t flag_fn = nullptr;
+    uint64_t flag_launches = 0;
     std::vector<std::pair<int, std::pair<hipEvent_t, hipEvent_t>>> pending;  // stat index, (start, stop)
     std::vector<hipEvent_t> event_pool;
     std::string description;
@@ -160,6 +163,15 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
             p->owned.push_back(q);
             slot_ptr[s] = q;
         }
+        if (plan.n_flags > 0) {
+            void* q = nullptr;
+            HIP_OK(hipMalloc(&q, (size_t)plan.n_flags * sizeof(int)));
+            p->owned.push_back(q);
+            p->flags = (int*)q;
+            auto m = compile_module(ctx, fixed_kernels_source());
+            p->mods.push_back(m);
+            p->flag_fn = get_function(*m, "adhip_flag");
+        }
         p->buf_ptr.resize(plan.buffers.size(), nullptr);
         for (size_t i = 0; i < plan.buffers.size(); ++i) {
             const PlanBuffer& b = plan.buffers[i];
@@ -219,7 +231,7 @@ void drain_events(adhip_program* p) {
 void launch(adhip_program* p, const Launch& l) {
     adhip_ctx* ctx = p->ctx;
     // argument block: guard pointer, then the plan's arguments
-    const void* guard = nullptr;
+    const void* guard = l.guard >= 0 ? (const void*)(p->flags + l.guard) : nullptr;
     std::vector<void*> ptrs;
     std::vector<std::unique_ptr<char[]>> store;
     ptrs.reserve(l.args.size() + 1);
@@ -256,6 +268,14 @@ void launch(adhip_program* p, const Launch& l) {
     p->plan->stats[l.stat].launches++;
 }
 
+void launch_flag(adhip_program* p, int slot, int parent, int cond_buf, int mode, int taken) {
+    int* flags = p->flags;
+    const float* cond = cond_buf >= 0 ? (const float*)p->buf_ptr[cond_buf] : nullptr;
+    void* args[] = {&flags, &slot, &parent, &cond, &mode, &taken};
+    HIP_OK(hipModuleLaunchKernel(p->flag_fn, 1, 1, 1, 64, 1, 1, 0, p->ctx->stream, args, nullptr));
+    p->flag_launches++;
+}
+
 float read_scalar(adhip_program* p, int buf, int slot) {
     adhip_ctx* ctx = p->ctx;
     HIP_OK(hipMemcpyAsync(ctx->pinned + slot, p->buf_ptr[buf], sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
@@ -286,6 +306,22 @@ void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
                     if (x + s.counter_inc == x && cond != 0.0f) throw Error("counted loop does not terminate (counter saturated)");
                 }
                 for (int64_t i = 0; i < n && !p->exited; ++i) exec_steps(p, s.body);
+            } else if (s.flag_slot >= 0) {
+                // device-predicated: enqueue a batch of iterations, then look at the predicate once
+                int batch = 4;
+                while (true) {
+                    for (int b = 0; b < batch; ++b) {
+                        launch_flag(p, s.flag_slot, s.parent_guard, s.cond_buf, 0, -1);
+                        exec_steps(p, s.body);
+                    }
+                    read_scalar(p, s.cond_buf, 0);
+                    HIP_OK(hipMemcpyAsync(ctx->pinned + 1, p->flags + s.flag_slot, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+                    HIP_OK(hipStreamSynchronize(ctx->stream));
+                    int flag;
+                    memcpy(&flag, ctx->pinned + 1, sizeof flag);
+                    if (flag == 0 || ctx->pinned[0] == 0.0f) break;
+                    if (batch < 32) batch *= 2;
+                }
             } else {
                 while (!p->exited) {
                     read_scalar(p, s.cond_buf, 0);
@@ -297,6 +333,19 @@ void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
             break;
         }
         case Step::BRANCH: {
+            if (s.taken_slot >= 0) {
+                // inside a predicated loop: every arm is enqueued under its own device flag
+                launch_flag(p, s.taken_slot, -1, -1, 3, -1);
+                for (size_t i = 0; i < s.arms.size(); ++i) {
+                    launch_flag(p, s.arm_slots[i], s.parent_guard, s.arms[i].first, 1, s.taken_slot);
+                    exec_steps(p, s.arms[i].second);
+                }
+                if (s.else_slot >= 0) {
+                    launch_flag(p, s.else_slot, s.parent_guard, -1, 2, s.taken_slot);
+                    exec_steps(p, s.else_body);
+                }
+                break;
+            }
             for (size_t i = 0; i < s.arms.size() && i < 64; ++i) read_scalar(p, s.arms[i].first, (int)i);
             HIP_OK(hipStreamSynchronize(ctx->stream));
             bool ran = false;
@@ -512,7 +561,16 @@ int adhip_compile_check(const uint8_t* program, size_t program_len, const char* 
         auto ir = parse_program(program, program_len);
         auto plan = lower_program(*ir, dep_vector(dep_ids, n_dep_ids));
         size_t bytes = 0;
-        for (auto& k : plan->kernels) bytes += compile_code_object(k.source, arch && *arch ? arch : "gfx950").size();
+        const char* dump_dir = getenv("ADHIP_DUMP_CODE_DIR");
+        for (auto& k : plan->kernels) {
+            std::vector<char> code = compile_code_object(k.source, arch && *arch ? arch : "gfx950");
+            bytes += code.size();
+            if (dump_dir && *dump_dir) {
+                std::string base = std::string(dump_dir) + "/" + k.entry;
+                if (FILE* f = fopen((base + ".hsaco").c_str(), "wb")) { fwrite(code.data(), 1, code.size(), f); fclose(f); }
+                if (FILE* f = fopen((base + ".hip").c_str(), "wb")) { fwrite(k.source.data(), 1, k.source.size(), f); fclose(f); }
+            }
+        }
         text = strf("%zu kernels compiled, %zu bytes of code objects", plan->kernels.size(), bytes);
     });
     if (rc != 0) text = g_tls_error;

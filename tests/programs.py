@@ -280,3 +280,36 @@ def check_golden(name, out):
                 f"{name}.{key}[{idx}]: {got[idx]} vs {exp[idx]}"
             got[idx] = exp[idx]
         assert np.array_equal(got, exp), f"{name}.{key}: {got} != {exp}"
+
+
+def predicated_loop_program(dev):
+    """A data-dependent while loop (its predicate is a product of two comparisons, so it is not the
+    counted `ir_for` shape) with an if/else and a nested if in the body.
+    i = 0..6: i < 2 -> y += 10; else { if i > 3 -> z *= 2; y += 1 }.  Result: y = 25, z = 8, i = 7."""
+    autodiff.set_device(dev)
+    i = autodiff.scalar(0.0)
+    y = autodiff.scalar(0.0)
+    z = autodiff.scalar(1.0)
+    pred = i.less_than(constant(7.0, [1])) * i.less_than(constant(100.0, [1]))
+
+    def body():
+        nonlocal i
+
+        def then():
+            y.__iadd__(10.0)
+            y.forward()
+
+        def other():
+            def inner():
+                z.__imul__(2.0)
+                z.forward()
+            autodiff.ir_if(lambda: i.more_than(autodiff.scalar(3.0)), inner)
+            y.__iadd__(1.0)
+            y.forward()
+
+        autodiff.ir_if_else(lambda: i.less_than(autodiff.scalar(2.0)), then, other)
+        i += 1.0
+
+    autodiff.ir_while(pred, body)
+    autodiff.execute()
+    return {"y": y.val().get(), "z": z.val().get(), "i": i.val().get()}

@@ -113,3 +113,13 @@ def test_range_select_collapses_to_two_pieces():
         os.environ["ADHIP_DUMP_SOURCE"] = "0"
     gather = [k for k in text.split("// =====") if "[elw]" in k][0]
     assert gather.count("?") <= 8, gather
+
+
+def test_data_dependent_loop_is_device_predicated():
+    from programs import predicated_loop_program
+    dev = Capture()
+    predicated_loop_program(dev)
+    text = lower_describe(dev.proc, dev.deps)
+    assert "[device-predicated" in text
+    rc, msg = _compile_check(dev.proc, dev.deps)
+    assert rc == 0, msg

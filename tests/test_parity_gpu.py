@@ -182,3 +182,15 @@ def test_errors_are_reported_not_fatal(hip_device):
     proc = IR.IRProcedure("main", [IR.CreateMat(np.ones(3, np.float32), [3], "a"), IR.ElwAdd(a="a", b="a", res="y"), IR.EX()])
     hip_device.execute(proc, {"y"})
     assert_exact(hip_device.get_tensor("y").data, np.full(3, 2.0, np.float32), "y")
+
+
+def test_predicated_loop_with_branches(hip_device):
+    """Data-dependent loop run device-predicated (iterations enqueued ahead, flags on the device),
+    including an if/else and a nested if whose arms are predicated too."""
+    print("[case] predicated loop", flush=True)
+    from programs import predicated_loop_program
+    got = predicated_loop_program(hip_device)
+    ref = predicated_loop_program(OracleDevice())
+    assert [ref["y"].data[0], ref["z"].data[0], ref["i"].data[0]] == [25.0, 8.0, 7.0]
+    for k in ref:
+        assert_exact(got[k].data, ref[k].data, k)
