@@ -20,6 +20,9 @@ for p in (ROOT, os.path.join(ROOT, "autodiff-ir-rust_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+# HBM bytes per launch of the fused forward+backward kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
+# plain copy kernel (profiles/fused_elw_8192x8192.hbm_traffic_pmc.txt).  Valid for the 8192x8192 workload only.
+FUSED_ELW_TRAFFIC_BYTES = 805784371 + 1082130944
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 
 
@@ -79,6 +82,9 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
+    ap.add_argument("--workload", default="all", choices=["all", "copy"],
+                    help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
+                         "the known-size reference that hardware byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the device path is single-device (run with --gpus 1)", file=sys.stderr)
@@ -89,6 +95,21 @@ def main():
 
     dev = HipDevice(0)
     rows = cols = 8192
+    if args.workload == "copy":
+        import numpy as np
+        from adhip import autodiff
+        autodiff.set_device(dev)
+        src = autodiff.tensor(np.zeros(rows * cols, dtype=np.float32), [rows, cols])
+        dst = src.contigious()
+        dst.forward()
+        dst.val().keep()
+        wlc = W.Workload("copy", {"dst": dst.val()}, {}, algorithmic_bytes=8.0 * rows * cols)
+        pc = compile_resident(dev, wlc)
+        msc = timed_runs(pc, args.steps, args.warmup)
+        print(json.dumps({"metric": "plain copy", "value": wlc.algorithmic_bytes / (msc * 1e-3) / 1e9, "unit": "GB/s",
+                          "ms_per_step": msc, "bytes_read": 4.0 * rows * cols, "bytes_written": 4.0 * rows * cols,
+                          "kernels": profile(pc, 3)}))
+        return
     wl = W.fused_elw(dev, rows, cols, seed=0)
     prog = compile_resident(dev, wl)
     ms = timed_runs(prog, args.steps, args.warmup)
@@ -100,7 +121,9 @@ def main():
     dom_alg = 4.0 * (7 * n + cols) if dom["kernel"].startswith("elw") else dom["bytes"]
     achieved = dom_alg / (dom["avg_ms"] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom["kernel"],
+                "frac": achieved / HBM_PEAK_GBS,
+                "traffic": FUSED_ELW_TRAFFIC_BYTES if dom["kernel"].startswith("elw_colsum") else None,
+                "kernel": dom["kernel"],
                 "avg_ms": dom["avg_ms"], "algorithmic_bytes": dom_alg}
     prog.close()
 
@@ -142,7 +165,7 @@ def main():
 
     cpu = None
     if not args.skip_cpu:
-        cpu = cpu_baseline_fused_elw(1024, 8192)
+        cpu = cpu_baseline_fused_elw(4096, 8192)
 
     line = {
         "metric": "fused-ELW & reduce GB/s (% HBM peak); fp32 MLP train steps/s, 1 MI355X",
