@@ -715,16 +715,18 @@ enum class RedLayout { ROW, COL };
 
 struct RedBody {
     Gen g;
+    std::vector<std::string> side_exprs;
     std::string value;  // per-lane value expression
     bool value_lane = false;
 };
 
 // atoms: ROW: x, yv (+ lane j along y); COL: xv, y (+ lane j along x)
-RedBody red_body(const Node* n, RedLayout layout, int vec, bool wide) {
+RedBody red_body(const Node* n, RedLayout layout, int vec, bool wide, const std::vector<Node*>& side = {}) {
     RedBody b;
     Gen& g = b.g;
     g.vec = vec;
     g.wide = wide;
+    for (Node* s : side) g.members.insert(s);
     const TRef& t = n->in[0];
     const int64_t V = t.shape[0], R = t.shape[1];
     Aff lin;
@@ -744,6 +746,7 @@ RedBody red_body(const Node* n, RedLayout layout, int vec, bool wide) {
     Val v = g.gen_tref(t, lin, "");
     b.value = v.expr;
     b.value_lane = v.lane;
+    for (Node* s : side) b.side_exprs.push_back(g.gen_node(s, lin, "").expr);
     return b;
 }
 
@@ -781,8 +784,10 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
     std::string src = kernel_prelude();
     if (layout == RedLayout::ROW) {
         vec = (R % 4 == 0 && R >= 256) ? 4 : 1;
-        RedBody b = red_body(n, layout, vec, wide);
+        const bool side = !spec.side_outputs.empty() && vec == 4;
+        RedBody b = red_body(n, layout, vec, wide, side ? spec.side_outputs : std::vector<Node*>());
         Gen& g = b.g;
+        k.side_done = side;
         const int64_t RV = R / vec;
         // threads per row: one wavefront per row (no barrier, no LDS) up to 8192 elements, a whole
         // block beyond that
@@ -792,15 +797,18 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         // split long rows over several blocks when there are too few rows to fill the GPU
         int64_t chunks = 1;
         if (force_chunks > 0) chunks = force_chunks;
-        else if (V * T < 131072 && RV >= (int64_t)T * 32) {
+        else if (V * T < 131072 && RV >= (int64_t)T * 128) {
             chunks = std::min<int64_t>((131072 + V * T - 1) / (V * T), RV / ((int64_t)T * 8));
             chunks = std::max<int64_t>(chunks, 1);
         }
         const int64_t CH = (RV + chunks - 1) / chunks;  // vector elements per chunk
-        k.kind = "reduce_row";
-        std::string sig = "const int* __restrict__ guard, float* __restrict__ out";
+        k.kind = side ? "reduce_row_store" : "reduce_row";
+        std::string sig = side ? "const int* __restrict__ guard, float* out" : "const int* __restrict__ guard, float* __restrict__ out";
         std::vector<Node*> order{const_cast<Node*>(n)};
-        for (auto& gb : g.bufs) { sig += ", const float* __restrict__ " + gb.param; order.push_back(gb.node); }
+        if (side)
+            for (size_t i = 0; i < spec.side_outputs.size(); ++i) { sig += strf(", float* w%zu", i); order.push_back(spec.side_outputs[i]); }
+        // a stored value may update one of the inputs in place, so nothing is restrict-qualified then
+        for (auto& gb : g.bufs) { sig += std::string(", const float* ") + (side ? "" : "__restrict__ ") + gb.param; order.push_back(gb.node); }
         src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
         src += strf("    const unsigned lane = threadIdx.x %% %du;\n", T);
@@ -816,10 +824,18 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
             src += strf("    if (row_ok)\n#pragma unroll 4\n    for (%s yv = (%s)chunk * %lldu + lane; yv < y_end; yv += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, T);
         }
         src += join(g.codeA, "        ");
+        if (side)
+            for (size_t i = 0; i < b.side_exprs.size(); ++i) src += strf("        float sv%zu[4];\n", i);
         if (vec > 1) src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
         else src += "        { const int j = 0;\n";
         src += join(g.codeB, "            ");
-        src += strf("            acc[j] += %s;\n        }\n    }\n", b.value.c_str());
+        if (side)
+            for (size_t i = 0; i < b.side_exprs.size(); ++i) src += strf("            sv%zu[j] = %s;\n", i, b.side_exprs[i].c_str());
+        src += strf("            acc[j] += %s;\n        }\n", b.value.c_str());
+        if (side)
+            for (size_t i = 0; i < b.side_exprs.size(); ++i)
+                src += strf("        { float4_t q = {sv%zu[0], sv%zu[1], sv%zu[2], sv%zu[3]}; *(float4_t*)(w%zu + (%lldu * x + 4u * yv)) = q; }\n", i, i, i, i, i, (long long)R);
+        src += "    }\n";
         if (vec == 4) src += "    float s = (acc[0] + acc[1]) + (acc[2] + acc[3]);\n";
         else src += "    float s = acc[0];\n";
         if (T == 64) {
@@ -837,6 +853,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         k.grid[1] = (unsigned)chunks;
         k.chunks = chunks;
         k.bytes = 4.0 * (double)V * (double)chunks;
+        if (side) k.bytes += 4.0 * (double)V * (double)R * (double)spec.side_outputs.size();
         for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), V * R);
         k.flops = (g.flops + 1) * (double)V * (double)R;
     } else {

@@ -41,6 +41,9 @@ struct ElwKernelSpec {
 struct ReduceKernelSpec {
     Node* node = nullptr;  // Op::SUM, operand [V,R]
     std::string name;
+    // Element-wise values with V*R elements that this kernel also stores (row layout only): the
+    // reduction's own operand chain is evaluated once, stored and summed in the same pass.
+    std::vector<Node*> side_outputs;
 };
 
 struct GeneratedKernel {
@@ -55,6 +58,7 @@ struct GeneratedKernel {
     // reductions that need a second pass: partial sums [chunks][V] written to `out`, then summed
     // (for element-wise kernels with column sums: the number of row tiles)
     int64_t chunks = 1;
+    bool side_done = false;  // the reduction stored its side outputs
 };
 
 // `in_memory(n)` tells whether node n's value can be loaded from a buffer in this kernel.

@@ -43,6 +43,8 @@ struct Node {
     // filled in by the lowering
     bool root = false;        // gets a buffer
     bool force_root = false;  // Contigious, live-out, dot operand ...
+    bool transpose = false;   // dense copy of a strided view, produced by the LDS-tiled transposing kernel
+    int transpose_u = -1;     // the dim of `shape` that is contiguous in the source
     int buffer = -1;          // plan buffer id holding this node's dense row-major value
     int kernel = -1;          // index of the kernel (group) that produces it
     int last_use_kernel = -1;

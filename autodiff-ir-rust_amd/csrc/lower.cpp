@@ -23,6 +23,71 @@ extern "C" __global__ __launch_bounds__(256) void adhip_copy(const int* __restri
     if (i < n) dst[i] = src[i];
 }
 
+// Dense copy of a strided view whose contiguous source dim (u) is not the innermost dim of the result (v):
+// a 64x64 tile goes through LDS so that both the reads (along u) and the writes (along v) are coalesced.
+// Up to three further dims are batch dims, given by extent and by source / result strides.
+extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy(
+    const int* __restrict__ guard, float* __restrict__ out, const float* __restrict__ in, long long in_off,
+    long long nb0, long long nb1, long long nb2, long long ib0, long long ib1, long long ib2, long long ob0, long long ob1,
+    long long ob2, long long U, long long V, long long in_sv, long long out_su) {
+    if (guard && *guard == 0) return;
+    __shared__ float tile[64][65];
+    long long b = blockIdx.z;
+    const long long b2 = b % nb2; b /= nb2;
+    const long long b1 = b % nb1; b /= nb1;
+    const long long b0 = b;
+    const float* src = in + in_off + b0 * ib0 + b1 * ib1 + b2 * ib2;
+    float* dst = out + b0 * ob0 + b1 * ob1 + b2 * ob2;
+    const unsigned tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;
+    const long long u0 = (long long)blockIdx.x * 64, v0 = (long long)blockIdx.y * 64;
+#pragma unroll 4
+    for (unsigned r = ty; r < 64u; r += 4u) {
+        const long long u = u0 + tx, v = v0 + r;
+        if (u < U && v < V) tile[r][tx] = src[v * in_sv + u];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (unsigned r = ty; r < 64u; r += 4u) {
+        const long long u = u0 + r, v = v0 + tx;
+        if (u < U && v < V) dst[u * out_su + v] = tile[tx][r];
+    }
+}
+
+// Same, 128-bit accesses: U, V, all strides and offsets are multiples of 4 elements.
+extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy4(
+    const int* __restrict__ guard, float* __restrict__ out, const float* __restrict__ in, long long in_off,
+    long long nb0, long long nb1, long long nb2, long long ib0, long long ib1, long long ib2, long long ob0, long long ob1,
+    long long ob2, long long U, long long V, long long in_sv, long long out_su) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    if (guard && *guard == 0) return;
+    __shared__ float tile[64][65];
+    long long b = blockIdx.z;
+    const long long b2 = b % nb2; b /= nb2;
+    const long long b1 = b % nb1; b /= nb1;
+    const long long b0 = b;
+    const float* src = in + in_off + b0 * ib0 + b1 * ib1 + b2 * ib2;
+    float* dst = out + b0 * ob0 + b1 * ob1 + b2 * ob2;
+    const unsigned c4 = threadIdx.x & 15u, rr = threadIdx.x >> 4;
+    const long long u0 = (long long)blockIdx.x * 64, v0 = (long long)blockIdx.y * 64;
+#pragma unroll
+    for (unsigned r = rr; r < 64u; r += 16u) {
+        const long long u = u0 + 4 * c4, v = v0 + r;
+        if (u < U && v < V) {
+            const f4 q = *(const f4*)(src + v * in_sv + u);
+            tile[r][4 * c4 + 0] = q.x; tile[r][4 * c4 + 1] = q.y; tile[r][4 * c4 + 2] = q.z; tile[r][4 * c4 + 3] = q.w;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (unsigned r = rr; r < 64u; r += 16u) {
+        const long long u = u0 + r, v = v0 + 4 * c4;
+        if (u < U && v < V) {
+            f4 q = {tile[4 * c4 + 0][r], tile[4 * c4 + 1][r], tile[4 * c4 + 2][r], tile[4 * c4 + 3][r]};
+            *(f4*)(dst + u * out_su + v) = q;
+        }
+    }
+}
+
 // Control-flow flags for device-predicated blocks (one thread).
 //   mode 0 (loop):  flags[slot] = parent && cond[0] != 0
 //   mode 1 (arm):   flags[slot] = parent && !flags[taken] && cond[0] == 1; sets flags[taken] when it fires
@@ -80,10 +145,12 @@ using RegionKey = std::pair<const Proc*, size_t>;
 struct Group {
     std::vector<Node*> members;
     int64_t n = 0;
-    enum Kind { ELW, SUM, DOT } kind = ELW;
+    enum Kind { ELW, SUM, DOT, TRANSPOSE } kind = ELW;
     // column sums computed by this element-wise kernel: (value node, SUM node that wanted it)
     std::vector<std::pair<Node*, Node*>> colsums;
     int64_t cs_rows = 0, cs_cols = 0;
+    // element-wise values a row reduction stores while it sums them
+    std::vector<Node*> side;
     bool dead = false;  // its only member was absorbed by another group
 };
 
@@ -100,7 +167,7 @@ struct Lowerer {
     std::vector<std::unique_ptr<Node>> arena;
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
-    int fixed_copy = -1, fixed_dot = -1;
+    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
 
     // per region
@@ -660,6 +727,61 @@ struct Lowerer {
             };
             for (auto& w : wanted) dfs(w.second);
         }
+        // ---- 3b. large operands read against the grain (unit stride on a dim that is not the innermost one
+        // of the consumer) are first copied densely by the tiled transposing kernel
+        if (opt.fuse) {
+            std::vector<Node*> work = topo;
+            bool added = false;
+            for (Node* n : work) {
+                if (!op_is_elw(n->op) || n->transpose) continue;
+                for (TRef& t : n->in) {
+                    for (Piece& pc : t.pieces) {
+                        if (pc.src.kind != Src::NODE || !in_mem(pc.src.node) || pc.view.st.empty()) continue;
+                        // the last stage is the one that addresses the buffer; earlier stages only
+                        // produce a row-major index into its shape, which a dense copy keeps valid
+                        const Stage st = pc.view.st.back();
+                        int last = -1, u = -1, nbatch = 0;
+                        for (int d = (int)st.shape.size() - 1; d >= 0; --d)
+                            if (st.shape[d] > 1) { last = d; break; }
+                        if (last < 0 || st.stride[last] <= 1) continue;
+                        for (int d = 0; d < last; ++d)
+                            if (st.shape[d] > 1 && st.stride[d] == 1) u = d;
+                        if (u < 0 || st.shape[u] < 16 || st.shape[last] < 16 || numel(st.shape) < (int64_t(1) << 18)) continue;
+                        for (int d = 0; d < last; ++d)
+                            if (d != u && st.shape[d] > 1) ++nbatch;
+                        if (nbatch > 3) continue;
+                        TRef region;
+                        region.shape = st.shape;
+                        Piece whole;
+                        whole.lo.assign(st.shape.size(), 0);
+                        whole.hi = st.shape;
+                        whole.view.st = {st};
+                        whole.src = pc.src;
+                        region.pieces.push_back(whole);
+                        Node* T = new_node(Op::COPY, st.shape, {region}, pc.src.node->name + ".t", 0.f, true);
+                        T->root = true;
+                        T->transpose = true;
+                        T->transpose_u = u;
+                        T->order = std::min(T->order, n->order - 0.25);
+                        pc.view.st.back() = contiguous_stage(st.shape);
+                        pc.src = Src();
+                        pc.src.kind = Src::NODE;
+                        pc.src.node = T;
+                        added = true;
+                    }
+                }
+            }
+            if (added) {
+                topo.clear();
+                std::set<Node*> seen;
+                std::function<void(Node*)> dfs = [&](Node* n) {
+                    if (!seen.insert(n).second) return;
+                    for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
+                    topo.push_back(n);
+                };
+                for (auto& w : wanted) dfs(w.second);
+            }
+        }
         // ---- 4. folded nodes used by several kernels: keep in memory when recomputing costs more
         {
             std::map<Node*, std::set<std::string>> users;
@@ -703,7 +825,7 @@ struct Lowerer {
         std::map<Node*, int> group_of;
         for (Node* r : roots) {
             int chosen = -1;
-            if (op_is_elw(r->op) && opt.fuse) {
+            if (op_is_elw(r->op) && opt.fuse && !r->transpose) {
                 for (int g = (int)groups.size() - 1; g >= 0; --g) {
                     if (groups[g].kind != Group::ELW || groups[g].n != numel(r->shape)) continue;
                     bool ok = true;
@@ -719,7 +841,7 @@ struct Lowerer {
             if (chosen < 0) {
                 Group g;
                 g.n = numel(r->shape);
-                g.kind = r->op == Op::SUM ? Group::SUM : (r->op == Op::DOT ? Group::DOT : Group::ELW);
+                g.kind = r->op == Op::SUM ? Group::SUM : (r->op == Op::DOT ? Group::DOT : (r->transpose ? Group::TRANSPOSE : Group::ELW));
                 groups.push_back(g);
                 chosen = (int)groups.size() - 1;
             }
@@ -758,6 +880,29 @@ struct Lowerer {
                 group_of[S] = target;
             }
         }
+        // ---- 5c. a row sum over an element-wise value produced by the kernel just before it: the
+        // reduction computes, stores and sums that value in one pass
+        if (opt.fuse) {
+            for (size_t gs = 1; gs < groups.size(); ++gs) {
+                Group& GS = groups[gs];
+                if (GS.dead || GS.kind != Group::SUM) continue;
+                Node* S = GS.members[0];
+                const TRef& t = S->in[0];
+                if (!t.single_full() || t.pieces[0].src.kind != Src::NODE) continue;
+                Node* E = t.pieces[0].src.node;
+                if (!E->root || !op_is_elw(E->op) || E->transpose || !identity_piece(t.pieces[0], t)) continue;
+                if (numel(E->shape) != numel(t.shape) || t.shape[1] % 4 != 0 || t.shape[1] < 256) continue;
+                int ge = group_of[E];
+                int prev = (int)gs - 1;
+                while (prev >= 0 && groups[prev].dead) --prev;
+                if (ge != prev) continue;
+                Group& GE = groups[ge];
+                if (GE.kind != Group::ELW || GE.members.size() != 1 || !GE.colsums.empty()) continue;
+                GS.side.push_back(E);
+                GE.dead = true;
+                group_of[E] = (int)gs;
+            }
+        }
         // ---- 6. generate code per group (no buffers needed yet)
         std::map<Node*, std::string> home_of_early;
         for (auto& w : wanted) home_of_early[w.second] = w.first;
@@ -769,7 +914,9 @@ struct Lowerer {
             Group& G = groups[g];
             if (G.dead) continue;
             std::set<const Node*> members(G.members.begin(), G.members.end());
-            for (Node* m : G.members)
+            std::vector<Node*> readers = G.members;
+            for (Node* sd : G.side) { members.insert(sd); readers.push_back(sd); }
+            for (Node* m : readers)
                 for (auto& rd : reads[m]) {
                     if (members.count(rd.first)) continue;
                     auto it = greads[g].find(rd.first);
@@ -812,7 +959,9 @@ struct Lowerer {
                 ReduceKernelSpec spec;
                 spec.node = G.members[0];
                 spec.name = name;
+                spec.side_outputs = G.side;
                 gks[g].k = gen_reduce_kernel(spec);
+                ADHIP_CHECK(G.side.empty() || gks[g].k.side_done, "internal: row reduction did not take over its operand's store");
                 if (gks[g].k.chunks > 1) {
                     // second pass over the partial sums [chunks][V]
                     Node* n = G.members[0];
@@ -844,6 +993,7 @@ struct Lowerer {
             if (groups[g].dead) continue;
             std::vector<Node*> produced = groups[g].members;
             for (auto& cs : groups[g].colsums) produced.push_back(cs.second);
+            for (Node* sd : groups[g].side) produced.push_back(sd);
             for (Node* m : produced) {
                 auto ho = home_of.find(m);
                 bool direct = false;
@@ -853,13 +1003,15 @@ struct Lowerer {
                     auto li = livein.find(id);
                     if (li != livein.end()) {
                         Node* old = li->second;
-                        const bool is_member = std::find(groups[g].members.begin(), groups[g].members.end(), m) != groups[g].members.end();
+                        const bool is_side = std::find(groups[g].side.begin(), groups[g].side.end(), m) != groups[g].side.end();
+                        const bool is_member = is_side || (groups[g].kind == Group::ELW &&
+                            std::find(groups[g].members.begin(), groups[g].members.end(), m) != groups[g].members.end());
                         for (size_t g2 = 0; g2 < groups.size(); ++g2) {
                             if (groups[g2].dead) continue;
                             auto it = greads[g2].find(old);
                             if (it == greads[g2].end()) continue;
                             if (g2 > g) direct = false;
-                            if (g2 == g && !(it->second && groups[g].kind == Group::ELW && is_member)) direct = false;
+                            if (g2 == g && !(it->second && is_member)) direct = false;
                         }
                     }
                     int hb = home(id, numel(m->shape));
@@ -911,6 +1063,10 @@ struct Lowerer {
                 emit_dot(G.members[0], out);
                 continue;
             }
+            if (G.kind == Group::TRANSPOSE) {
+                emit_transpose(G.members[0], out);
+                continue;
+            }
             GeneratedKernel& k = gks[g].k;
             if (G.kind == Group::ELW && !G.colsums.empty()) {
                 launch_generated(k);
@@ -954,6 +1110,45 @@ struct Lowerer {
         for (auto& c : commits) emit_copy(out, c.dst, c.src, c.n, "commit_" + c.id);
         for (auto& c : commits) free_temp(c.src);
         end_region(wanted);
+    }
+
+    void emit_transpose(Node* n, std::vector<Step>& out) {
+        const Piece& pc = n->in[0].pieces[0];
+        const Stage& st = pc.view.st[0];
+        const int nd = (int)st.shape.size();
+        int last = -1;
+        for (int d = nd - 1; d >= 0; --d)
+            if (st.shape[d] > 1) { last = d; break; }
+        const int u = n->transpose_u;
+        Shape dense = row_major_strides(st.shape);
+        int64_t nb[3] = {1, 1, 1}, ib[3] = {0, 0, 0}, ob[3] = {0, 0, 0};
+        int k = 0;
+        for (int d = 0; d < last; ++d)
+            if (d != u && st.shape[d] > 1) { nb[k] = st.shape[d]; ib[k] = st.stride[d]; ob[k] = dense[d]; ++k; }
+        const int64_t U = st.shape[u], V = st.shape[last];
+        const int64_t batches = nb[0] * nb[1] * nb[2];
+        ADHIP_CHECK(batches <= 65535 && (V + 63) / 64 <= 65535, "internal: transpose grid too large");
+        // the source region must lie inside the source buffer
+        int64_t hi = st.offset;
+        for (int d = 0; d < nd; ++d) hi += (st.shape[d] - 1) * st.stride[d];
+        ADHIP_CHECK(st.offset >= 0 && hi < numel(pc.src.node->shape), "internal: transposing copy reads outside its source");
+        bool v4 = (U % 4 == 0) && (V % 4 == 0) && (st.offset % 4 == 0) && (st.stride[last] % 4 == 0) && (dense[u] % 4 == 0);
+        for (int q = 0; q < 3; ++q) v4 = v4 && (ib[q] % 4 == 0) && (ob[q] % 4 == 0);
+        if (fixed_transpose < 0) fixed_transpose = add_kernel("adhip_transpose_copy", fixed_kernels_source(), "transpose");
+        if (fixed_transpose4 < 0) fixed_transpose4 = add_kernel("adhip_transpose_copy4", fixed_kernels_source(), "transpose");
+        Launch l;
+        l.kernel = v4 ? fixed_transpose4 : fixed_transpose;
+        l.block[0] = 256;
+        l.grid[0] = (unsigned)((U + 63) / 64);
+        l.grid[1] = (unsigned)((V + 63) / 64);
+        l.grid[2] = (unsigned)batches;
+        auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: transpose operand without buffer"); q.buf = x->buffer; return q; };
+        auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
+        l.args = {B(n), B(pc.src.node), I(st.offset), I(nb[0]), I(nb[1]), I(nb[2]), I(ib[0]), I(ib[1]), I(ib[2]),
+                  I(ob[0]), I(ob[1]), I(ob[2]), I(U), I(V), I(st.stride[last]), I(dense[u])};
+        l.label = "transpose_" + n->name;
+        l.bytes = 8.0 * (double)numel(st.shape);
+        push_launch(out, l, "transpose");
     }
 
     void emit_dot(Node* n, std::vector<Step>& out) {
