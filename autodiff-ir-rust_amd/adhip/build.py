@@ -25,5 +25,18 @@ def build_library(verbose: bool = False) -> str:
     return out
 
 
+def build_cxx_smoke(verbose: bool = False) -> str:
+    """Compile tests/cxx/cabi_smoke.cpp (plain C++ against include/adhip.h) and link it with the library."""
+    root = os.path.dirname(os.path.dirname(_PKG_DIR))
+    src = os.path.join(root, "tests", "cxx", "cabi_smoke.cpp")
+    out = os.path.join(root, "tests", "cxx", "cabi_smoke")
+    cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-o", out, src, "-L" + CSRC, "-ladhip", "-Wl,-rpath," + CSRC,
+           "-Wl,-rpath,/opt/rocm/lib"]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))

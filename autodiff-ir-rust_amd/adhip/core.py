@@ -927,7 +927,11 @@ class BroadcastNode(Node):
         return p_dim
 
     def backward(self, grad: Value):
-        self.parent.n.backward(grad.to_node().sum(self._dim).forward())
+        # The reference hands the parent the summed gradient with the broadcast dim dropped
+        # (broadcast.rs:28-32), which only works when the parent is the left-padding view.  The dim is
+        # put back (a free view) so any parent sees a gradient of its own shape.
+        g = grad.to_node().sum(self._dim).view(self.parent.dim())
+        self.parent.n.backward(g.forward())
 
     def val(self):
         if self.parent.val() is None:

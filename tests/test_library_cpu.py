@@ -123,3 +123,15 @@ def test_data_dependent_loop_is_device_predicated():
     assert "[device-predicated" in text
     rc, msg = _compile_check(dev.proc, dev.deps)
     assert rc == 0, msg
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_programs_lower_and_compile(seed):
+    from fuzz_programs import random_program
+    dev = Capture()
+    random_program(dev, seed)
+    rc, msg = _compile_check(dev.proc, dev.deps)
+    assert rc == 0, msg
+    from oracle.interp import OracleDevice
+    out = random_program(OracleDevice(), seed)
+    assert not out["target"].is_none
