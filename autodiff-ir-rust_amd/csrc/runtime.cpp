@@ -9,6 +9,10 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cerrno>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -80,7 +84,65 @@ struct adhip_program {
 
 namespace {
 
+// Code objects are cached on disk, keyed by a hash of (arch, options, source), so that a process that
+// runs a program it has seen before does not pay for hipRTC again.  ADHIP_CACHE_DIR overrides the
+// location; ADHIP_CACHE_DIR=off disables the cache.
+const char* kCompileOptionsTag = "O3;fp-contract=off;correctly-rounded-divide-sqrt;no-packed-fp32;v1";
+
+uint64_t fnv1a(const std::string& s, uint64_t h = 1469598103934665603ull) {
+    for (unsigned char c : s) { h ^= c; h *= 1099511628211ull; }
+    return h;
+}
+
+std::string cache_path(const std::string& source, const std::string& arch_name) {
+    const char* dir = getenv("ADHIP_CACHE_DIR");
+    std::string d;
+    if (dir && *dir) {
+        if (std::string(dir) == "off") return "";
+        d = dir;
+    } else {
+        const char* home = getenv("HOME");
+        d = std::string(home && *home ? home : "/tmp") + "/.cache/adhip";
+    }
+    std::string cmd_dir = d;
+    // create the directory (two levels at most); failures just disable the cache
+    for (size_t i = 1; i <= cmd_dir.size(); ++i)
+        if (i == cmd_dir.size() || cmd_dir[i] == '/') {
+            std::string sub = cmd_dir.substr(0, i);
+            if (mkdir(sub.c_str(), 0755) != 0 && errno != EEXIST) { /* keep going: a parent may be read-only but exist */ }
+        }
+    uint64_t h = fnv1a(source, fnv1a(arch_name + ";" + kCompileOptionsTag));
+    return d + "/" + strf("%016llx_%zu.hsaco", (unsigned long long)h, source.size());
+}
+
+std::vector<char> compile_code_object_uncached(const std::string& source, const std::string& arch_name);
+
 std::vector<char> compile_code_object(const std::string& source, const std::string& arch_name) {
+    const std::string path = cache_path(source, arch_name);
+    if (!path.empty()) {
+        if (FILE* f = fopen(path.c_str(), "rb")) {
+            std::vector<char> code;
+            char buf[65536];
+            size_t n;
+            while ((n = fread(buf, 1, sizeof buf, f)) > 0) code.insert(code.end(), buf, buf + n);
+            fclose(f);
+            if (code.size() > 64) return code;
+        }
+    }
+    std::vector<char> code = compile_code_object_uncached(source, arch_name);
+    if (!path.empty()) {
+        std::string tmp = path + strf(".tmp%d", (int)getpid());
+        if (FILE* f = fopen(tmp.c_str(), "wb")) {
+            const bool ok = fwrite(code.data(), 1, code.size(), f) == code.size();
+            fclose(f);
+            if (ok) rename(tmp.c_str(), path.c_str());
+            else remove(tmp.c_str());
+        }
+    }
+    return code;
+}
+
+std::vector<char> compile_code_object_uncached(const std::string& source, const std::string& arch_name) {
     hiprtcProgram prog;
     if (hiprtcCreateProgram(&prog, source.c_str(), "adhip_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
         throw Error("hiprtcCreateProgram failed");

@@ -129,6 +129,24 @@ def main():
 
     extra = {"fused_elw_kernels": kstats}
     if not args.skip_extra:
+        # config 1: README MLP, a latency case: complete adhip_execute calls (parse, lower, upload, run, read back)
+        wl1 = W.readme_mlp(dev, seed=0)
+        proc1, deps1 = wl1.finish()
+        dev.execute(proc1, deps1)  # first call compiles the kernels
+        t0 = time.perf_counter()
+        for _ in range(20):
+            dev.execute(proc1, deps1)
+        us_exec = (time.perf_counter() - t0) / 20 * 1e6
+        p1 = dev.compile(proc1, deps1)
+        p1.upload()
+        p1.run()
+        t0 = time.perf_counter()
+        for _ in range(50):
+            p1.run()
+        us_run = (time.perf_counter() - t0) / 50 * 1e6
+        extra["readme_mlp"] = {"us_per_execute_call": us_exec, "us_per_resident_run": us_run,
+                               "kernels_per_run": sum(1 for s_ in p1.kernel_stats())}
+        p1.close()
         # config 3: reductions
         wl3 = W.reductions(dev, 16384, 4096, seed=0)
         p3 = compile_resident(dev, wl3)
@@ -165,7 +183,7 @@ def main():
 
     cpu = None
     if not args.skip_cpu:
-        cpu = cpu_baseline_fused_elw(4096, 8192)
+        cpu = cpu_baseline_fused_elw(8192, 8192)
 
     line = {
         "metric": "fused-ELW & reduce GB/s (% HBM peak); fp32 MLP train steps/s, 1 MI355X",
