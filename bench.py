@@ -82,7 +82,7 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "mlp"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by")
     args = ap.parse_args()
@@ -109,6 +109,15 @@ def main():
         print(json.dumps({"metric": "plain copy", "value": wlc.algorithmic_bytes / (msc * 1e-3) / 1e9, "unit": "GB/s",
                           "ms_per_step": msc, "bytes_read": 4.0 * rows * cols, "bytes_written": 4.0 * rows * cols,
                           "kernels": profile(pc, 3)}))
+        return
+    if args.workload == "mlp":
+        wl4 = W.mlp_train(dev, 4096, (4096, 4096, 4096, 1024), args.mlp_iters, seed=0)
+        p4 = compile_resident(dev, wl4)
+        t0 = time.perf_counter()
+        p4.run()
+        dt4 = time.perf_counter() - t0
+        print(json.dumps({"metric": "fp32 MLP train steps/s", "value": args.mlp_iters / dt4, "unit": "steps/s",
+                          "ms_per_train_step": dt4 * 1e3 / args.mlp_iters}))
         return
     wl = W.fused_elw(dev, rows, cols, seed=0)
     prog = compile_resident(dev, wl)

@@ -220,3 +220,61 @@ def test_random_programs_match_oracle(seed, hip_device):
     for k, rv in ref.items():
         assert got[k].dim == rv.dim, f"{k}: dim {got[k].dim} vs {rv.dim}"
         assert_close(got[k].data, rv.data, 2e-4, f"seed {seed} {k}")
+
+
+def _run_ir(dev, cmds, keep):
+    from adhip import ir as IR
+    proc = IR.IRProcedure("main", list(cmds) + [IR.EX()])
+    dev.execute(proc, set(keep))
+    return {k: dev.get_tensor(k) for k in keep}
+
+
+def test_edge_shapes(hip_device):
+    """Empty tensors, single elements, degenerate matmuls and reductions, high rank."""
+    print("[case] edge shapes", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal(2 * 3 * 2 * 2 * 5).astype(np.float32)
+    cmds = [
+        IR.CreateMat(np.zeros(0, np.float32), [0, 4], "e"), IR.CreateMat(np.arange(8, dtype=np.float32), [2, 4], "a"),
+        IR.Concat(a="e", b="a", dim=0, res="ea"), IR.Concat(a="a", b="e", dim=0, res="ae"),   # empty pieces vanish
+        IR.Contigious(a="ea", res="c1"), IR.Contigious(a="ae", res="c2"),
+        IR.CreateMat(np.array([3.0], np.float32), [1, 1], "one"), IR.DotProduct(a="one", b="one", res="d11"),
+        IR.CreateMat(np.arange(6, dtype=np.float32), [6, 1], "col"), IR.Sum(a="col", res="s1"),           # R = 1
+        IR.Permute(a="col", p=[1, 0], res="row"), IR.Sum(a="row", res="s6"),                           # V = 1
+        IR.DotProduct(a="col", b="row", res="outer"),                                                     # K = 1
+        IR.CreateMat(x, [2, 3, 2, 2, 5], "x5"), IR.Permute(a="x5", p=[4, 2, 0, 3, 1], res="p5"),
+        IR.View(a="p5", target_dim=[10, 12], res="v5"), IR.Sum(a="v5", res="s5"),
+        IR.Index(a="a", index=1, dim=0, res="a1"), IR.Index(a="a1", index=2, dim=0, res="a12"),          # rank 0
+        IR.View(a="a12", target_dim=[1], res="a12v"), IR.Contigious(a="a12v", res="scalar"),
+    ]
+    out = _run_ir(hip_device, cmds, ["c1", "c2", "d11", "s1", "s6", "outer", "s5", "scalar", "e"])
+    assert out["c1"].dim == [2, 4] and out["c2"].dim == [2, 4]
+    assert_exact(out["c1"].data, np.arange(8, dtype=np.float32), "empty ++ a")
+    assert_exact(out["c2"].data, np.arange(8, dtype=np.float32), "a ++ empty")
+    assert out["d11"].data[0] == 9.0
+    assert_exact(out["s1"].data, np.arange(6, dtype=np.float32), "sum over one element")
+    assert_exact(out["s6"].data, np.array([15.0], np.float32), "sum of one row")
+    assert_exact(out["outer"].data, np.outer(np.arange(6), np.arange(6)).astype(np.float32).reshape(-1), "outer product")
+    ref5 = x.reshape(2, 3, 2, 2, 5).transpose(4, 2, 0, 3, 1).reshape(10, 12).astype(np.float64).sum(1)
+    assert_close(out["s5"].data, ref5, RED_RTOL * math.sqrt(12), "5-D permute + view + sum")
+    assert out["scalar"].data[0] == 6.0 and out["scalar"].dim == [1]
+    assert out["e"].dim == [0, 4] and out["e"].data.size == 0
+
+
+def test_shape_errors_are_reported(hip_device):
+    from adhip import ir as IR
+    a = IR.CreateMat(np.zeros(6, np.float32), [2, 3], "a")
+    b = IR.CreateMat(np.zeros(8, np.float32), [2, 4], "b")
+    for bad, msg in [
+        ([a, b, IR.DotProduct(a="a", b="b", res="c")], "DotProduct"),
+        ([a, IR.View(a="a", target_dim=[4, 2], res="v")], "cannot be viewed"),
+        ([a, IR.Permute(a="a", p=[0, 0], res="p")], "not a permutation"),
+        ([a, IR.Index(a="a", index=5, dim=0, res="i")], "out of range"),
+        ([a, b, IR.Concat(a="a", b="b", dim=0, res="c")], "Concat"),
+        ([a, IR.Broadcast(a="a", dim=1, r=7, res="r")], "Broadcast"),
+        ([a, IR.Sum(a="a", res="s"), IR.Sum(a="s", res="t")], "expected 2-D"),
+    ]:
+        proc = IR.IRProcedure("main", bad + [IR.EX()])
+        with pytest.raises(RuntimeError, match=msg):
+            hip_device.execute(proc, {"a"})
