@@ -3,9 +3,9 @@
 // The reference multiplies with one work-item per output element, a sequential k loop and two
 // global loads per multiply-add (reference src/devices/opencl/kernels/dotprod.rs:23-53); transposed
 // operands are folded into its index expressions.  Here both operands are described by strides
-// (so x^T and W^T of the backward pass need no copy), staged through LDS in 128x128x16 tiles with
-// register prefetch of the next tile, and each of the four wavefronts of a block owns a 64x64
-// sub-tile = 2x2 MFMA blocks of 32x32.
+// (so x^T and W^T of the backward pass need no copy), staged through LDS in 128x128x16 or 256x128x16
+// tiles with register prefetch of the next tile, and each of the four (eight) wavefronts of a block
+// owns a 64x64 sub-tile = 2x2 MFMA blocks of 32x32.
 #include "gemm.hpp"
 
 #include "common.hpp"
@@ -16,12 +16,14 @@ std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry) 
     std::string s;
     s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n", cfg.a_kcontig ? 1 : 0, cfg.b_kcontig ? 1 : 0,
               cfg.edge ? 1 : 0);
-    s += strf("#define KERNEL_NAME %s\n", entry.c_str());
+    s += strf("#define KERNEL_NAME %s\n#define BM %d\n", entry.c_str(), cfg.bm);
     s += R"(
-#define BM 128
 #define BN 128
 #define BK 16
 #define LDA (BM + 4)
+#define LDB (BN + 4)
+#define NT (BM * 2)            /* threads: one wave per 64x64 sub-tile */
+#define B_LOADS (512 / NT)     /* float4 loads of the B tile per thread */
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
@@ -29,13 +31,13 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 // A_KCONTIG: a_sk == 1 (else a_sm == 1).  B_KCONTIG: b_sk == 1 (else b_sn == 1).
 // EDGE: M, N or K is not a multiple of the tile, or an operand is not 16-byte aligned; every
 // access is then bounds-checked and scalar.
-extern "C" __global__ __launch_bounds__(256) void KERNEL_NAME(
+extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     const int* __restrict__ guard, float* __restrict__ C, const float* __restrict__ A, const float* __restrict__ B,
     long long M, long long N, long long K, long long a_off, long long a_sm, long long a_sk, long long b_off,
     long long b_sk, long long b_sn) {
     if (guard && *guard == 0) return;
     __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDB];
 
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u, wave = tid >> 6;
@@ -69,13 +71,13 @@ extern "C" __global__ __launch_bounds__(256) void KERNEL_NAME(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    float4_t ra[2], rb[2];
+    float4_t ra0[2], rb0[B_LOADS];
 
-    auto load_a = [&](long long k0) {
+    auto load_a = [&](long long k0, float4_t* ra) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #if A_KCONTIG
-            const unsigned kq = tid & 3u, mr = (tid >> 2) + 64u * i;
+            const unsigned kq = tid & 3u, mr = (tid >> 2) + (NT / 4) * i;
             const long long m = bm + mr, k = k0 + 4 * kq;
 #if EDGE
             float4_t v = {0.f, 0.f, 0.f, 0.f};
@@ -89,7 +91,7 @@ extern "C" __global__ __launch_bounds__(256) void KERNEL_NAME(
             ra[i] = *(const float4_t*)(A + m * a_sm + k);
 #endif
 #else
-            const unsigned mq = tid & 31u, kr = (tid >> 5) + 8u * i;
+            const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + 8u * i;
             const long long m = bm + 4 * mq, k = k0 + kr;
 #if EDGE
             float4_t v = {0.f, 0.f, 0.f, 0.f};
@@ -105,11 +107,11 @@ extern "C" __global__ __launch_bounds__(256) void KERNEL_NAME(
 #endif
         }
     };
-    auto load_b = [&](long long k0) {
+    auto load_b = [&](long long k0, float4_t* rb) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < B_LOADS; ++i) {
 #if B_KCONTIG
-            const unsigned kq = tid & 3u, nr = (tid >> 2) + 64u * i;
+            const unsigned kq = tid & 3u, nr = (tid >> 2) + (NT / 4) * i;
             const long long n = bn + nr, k = k0 + 4 * kq;
 #if EDGE
             float4_t v = {0.f, 0.f, 0.f, 0.f};
@@ -123,7 +125,7 @@ extern "C" __global__ __launch_bounds__(256) void KERNEL_NAME(
             rb[i] = *(const float4_t*)(B + n * b_sn + k);
 #endif
 #else
-            const unsigned nq = tid & 31u, kr = (tid >> 5) + 8u * i;
+            const unsigned nq = tid & 31u, kr = (tid >> 5) + (NT / 32) * i;
             const long long n = bn + 4 * nq, k = k0 + kr;
 #if EDGE
             float4_t v = {0.f, 0.f, 0.f, 0.f};
@@ -139,61 +141,72 @@ extern "C" __global__ __launch_bounds__(256) void KERNEL_NAME(
 #endif
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_tiles = [&](int buf, const float4_t* ra, const float4_t* rb) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #if A_KCONTIG
-            {
-                const unsigned kq = tid & 3u, mr = (tid >> 2) + 64u * i;
+            const unsigned kq = tid & 3u, mr = (tid >> 2) + (NT / 4) * i;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) As[buf][4 * kq + j][mr] = ra[i][j];
-            }
+            for (int j = 0; j < 4; ++j) As[buf][4 * kq + j][mr] = ra[i][j];
 #else
-            {
-                const unsigned mq = tid & 31u, kr = (tid >> 5) + 8u * i;
-                *(float4_t*)&As[buf][kr][4 * mq] = ra[i];
-            }
+            const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + 8u * i;
+            *(float4_t*)&As[buf][kr][4 * mq] = ra[i];
 #endif
-#if B_KCONTIG
-            {
-                const unsigned kq = tid & 3u, nr = (tid >> 2) + 64u * i;
+        }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) Bs[buf][4 * kq + j][nr] = rb[i][j];
-            }
+        for (int i = 0; i < B_LOADS; ++i) {
+#if B_KCONTIG
+            const unsigned kq = tid & 3u, nr = (tid >> 2) + (NT / 4) * i;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) Bs[buf][4 * kq + j][nr] = rb[i][j];
 #else
-            {
-                const unsigned nq = tid & 31u, kr = (tid >> 5) + 8u * i;
-                *(float4_t*)&Bs[buf][kr][4 * nq] = rb[i];
-            }
+            const unsigned nq = tid & 31u, kr = (tid >> 5) + (NT / 32) * i;
+            *(float4_t*)&Bs[buf][kr][4 * nq] = rb[i];
 #endif
         }
     };
 
+    // One k-tile: 8 MFMA steps from LDS buffer `cur`; the operands of step ks+1 are fetched from LDS before the
+    // four MFMAs of step ks are issued, and half way through the tile that was prefetched into registers (sa, sb)
+    // is parked in the other LDS buffer, which nobody reads during this iteration.
+    auto compute = [&](int cur, bool park, const float4_t* sa, const float4_t* sb) {
+        float fa0[2], fa1[2], fb0[2], fb1[2];
+        fa0[0] = As[cur][lh][wm * 64 + li];
+        fa1[0] = As[cur][lh][wm * 64 + 32 + li];
+        fb0[0] = Bs[cur][lh][wn * 64 + li];
+        fb1[0] = Bs[cur][lh][wn * 64 + 32 + li];
+#pragma unroll
+        for (int ks = 0; ks < BK / 2; ++ks) {
+            const int c = ks & 1, nx = c ^ 1;
+            if (ks + 1 < BK / 2) {
+                fa0[nx] = As[cur][2 * (ks + 1) + lh][wm * 64 + li];
+                fa1[nx] = As[cur][2 * (ks + 1) + lh][wm * 64 + 32 + li];
+                fb0[nx] = Bs[cur][2 * (ks + 1) + lh][wn * 64 + li];
+                fb1[nx] = Bs[cur][2 * (ks + 1) + lh][wn * 64 + 32 + li];
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads ahead of the MFMAs that hide their latency
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0[c], fb0[c], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0[c], fb1[c], acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1[c], fb0[c], acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1[c], fb1[c], acc[1][1], 0, 0, 0);
+            if (ks == BK / 4 - 1 && park) store_tiles(cur ^ 1, sa, sb);
+        }
+    };
+
+    // The next tile's global loads are issued before the current tile is multiplied (one tile ahead).
     const long long KT = (K + BK - 1) / BK;
-    load_a(0);
-    load_b(0);
-    store_tiles(0);
+    load_a(0, ra0);
+    load_b(0, rb0);
+    store_tiles(0, ra0, rb0);
     __syncthreads();
 
     for (long long kt = 0; kt < KT; ++kt) {
-        const int cur = (int)(kt & 1);
         const bool more = kt + 1 < KT;
         if (more) {
-            load_a((kt + 1) * BK);
-            load_b((kt + 1) * BK);
+            load_a((kt + 1) * BK, ra0);
+            load_b((kt + 1) * BK, rb0);
         }
-#pragma unroll
-        for (int ks = 0; ks < BK / 2; ++ks) {
-            const float a0 = As[cur][2 * ks + lh][wm * 64 + li];
-            const float a1 = As[cur][2 * ks + lh][wm * 64 + 32 + li];
-            const float b0 = Bs[cur][2 * ks + lh][wn * 64 + li];
-            const float b1 = Bs[cur][2 * ks + lh][wn * 64 + 32 + li];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-        }
-        if (more) store_tiles(cur ^ 1);
+        compute((int)(kt & 1), more, ra0, rb0);
         __syncthreads();
     }
 

@@ -1165,11 +1165,13 @@ struct Lowerer {
             cfg.b_kcontig = b.s0 == 1;
             const int64_t a_ld = cfg.a_kcontig ? a.s0 : a.s1, b_ld = cfg.b_kcontig ? b.s1 : b.s0;
             cfg.edge = (M % 128) || (N % 128) || (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
-            std::string entry = strf("adhip_gemm_%c%c%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.edge ? "_edge" : "");
+            // 256-row tiles (8 waves) when that still leaves two blocks per CU; else 128-row tiles
+            cfg.bm = (!cfg.edge && M % 256 == 0 && (M / 256) * (N / 128) >= 512) ? 256 : 128;
+            std::string entry = strf("adhip_gemm_%c%c_%d%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm, cfg.edge ? "_edge" : "");
             Launch l;
             l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
-            l.block[0] = 256;
-            l.grid[0] = (unsigned)(((M + 127) / 128) * ((N + 127) / 128));
+            l.block[0] = (unsigned)(cfg.bm * 2);
+            l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + 127) / 128));
             l.args = {B(n), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
             l.label = strf("dot_%s_%lldx%lldx%lld", n->name.c_str(), (long long)M, (long long)N, (long long)K);
             l.bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);

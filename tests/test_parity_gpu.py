@@ -278,3 +278,9 @@ def test_shape_errors_are_reported(hip_device):
         proc = IR.IRProcedure("main", bad + [IR.EX()])
         with pytest.raises(RuntimeError, match=msg):
             hip_device.execute(proc, {"a"})
+
+
+@pytest.mark.parametrize("m,k,n", [(2048, 256, 4096), (1024, 64, 8192)])
+def test_dot_large_tile_variant(m, k, n, hip_device):
+    """Shapes that select the 256-row block tile (8 waves) of the MFMA kernel, all three operand layouts."""
+    test_dot_forward_backward(m, k, n, hip_device)
