@@ -74,6 +74,10 @@ struct adhip_program {
     std::vector<std::shared_ptr<Module>> mods;
     bool profiling = false;
     bool exited = false;
+    // runs of consecutive launches replayed as one hipGraph: key = (step list, index of the first launch)
+    std::map<std::pair<const void*, size_t>, hipGraphExec_t> graphs;
+    std::vector<hipGraph_t> graph_objs;
+    bool use_graphs = true;
     int* flags = nullptr;            // device flags of predicated blocks
     hipFunction_t flag_fn = nullptr;
     uint64_t flag_launches = 0;
@@ -192,6 +196,8 @@ void program_free(adhip_program* p) {
     if (p->ctx) (void)hipSetDevice(p->ctx->device);
     for (auto& pe : p->pending) { (void)hipEventDestroy(pe.second.first); (void)hipEventDestroy(pe.second.second); }
     for (auto e : p->event_pool) (void)hipEventDestroy(e);
+    for (auto& g : p->graphs) (void)hipGraphExecDestroy(g.second);
+    for (auto g : p->graph_objs) (void)hipGraphDestroy(g);
     for (void* q : p->owned) (void)hipFree(q);
     delete p;
 }
@@ -207,6 +213,8 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
     HIP_OK(hipSetDevice(ctx->device));
     std::unique_ptr<adhip_program> p(new adhip_program());
     p->ctx = ctx;
+    const char* genv = getenv("ADHIP_GRAPHS");
+    if (genv && *genv == '0') p->use_graphs = false;
     p->ir = parse_program(program, len);
     p->plan = lower_program(*p->ir, dep_vector(dep_ids, n));
     Plan& plan = *p->plan;
@@ -344,12 +352,49 @@ float read_scalar(adhip_program* p, int buf, int slot) {
     return 0.f;
 }
 
+// A run of at least eight consecutive kernel launches is captured once into a hipGraph and replayed with a
+// single submission afterwards (kernel arguments are fixed device pointers and constants, so the captured
+// nodes never need updating).  Per-kernel profiling and ADHIP_GRAPHS=0 bypass this.
+bool replay_run(adhip_program* p, const std::vector<Step>& steps, size_t first, size_t last) {
+    if (!p->use_graphs || p->profiling || last - first < 8) return false;
+    adhip_ctx* ctx = p->ctx;
+    auto key = std::make_pair((const void*)&steps, first);
+    auto it = p->graphs.find(key);
+    if (it == p->graphs.end()) {
+        hipGraph_t graph = nullptr;
+        HIP_OK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+        try {
+            for (size_t i = first; i < last; ++i) launch(p, steps[i].launch);
+        } catch (...) {
+            (void)hipStreamEndCapture(ctx->stream, &graph);
+            if (graph) (void)hipGraphDestroy(graph);
+            throw;
+        }
+        HIP_OK(hipStreamEndCapture(ctx->stream, &graph));
+        hipGraphExec_t exec = nullptr;
+        HIP_OK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        p->graph_objs.push_back(graph);
+        it = p->graphs.emplace(key, exec).first;
+    } else {
+        for (size_t i = first; i < last; ++i) p->plan->stats[steps[i].launch.stat].launches++;
+    }
+    HIP_OK(hipGraphLaunch(it->second, ctx->stream));
+    return true;
+}
+
 void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
     adhip_ctx* ctx = p->ctx;
-    for (const Step& s : steps) {
+    for (size_t si = 0; si < steps.size(); ++si) {
+        const Step& s = steps[si];
         if (p->exited) return;
         switch (s.kind) {
-        case Step::LAUNCH: launch(p, s.launch); break;
+        case Step::LAUNCH: {
+            size_t last = si;
+            while (last < steps.size() && steps[last].kind == Step::LAUNCH) ++last;
+            if (replay_run(p, steps, si, last)) si = last - 1;
+            else launch(p, s.launch);
+            break;
+        }
         case Step::EXIT: p->exited = true; return;
         case Step::LOOP: {
             if (s.counter_buf >= 0) {
