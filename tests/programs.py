@@ -13,45 +13,14 @@ from adhip import autodiff, nn
 from adhip.core import concat, constant, dot
 
 
-# ---- golden vectors asserted by the reference's tests -----------------------------------
-GOLDEN = {
-    # src/tests/nn.rs:73-99 (round 4)
-    "nn": {
-        "y": ([2, 2], [-1.6599, -1.5678, -1.6662, -1.5736]),
-        "l1_w": ([5, 3], [0.0461, 0.0349, 0.025, 0.0599, 0.0683, 0.0815, 0.0358, 0.1238, 0.094,
-                          0.0487, 0.0365, 0.1067, 0.0639, 0.0428, 0.0729]),
-        "l1_b": ([3], [0.4715, 0.4172, 0.4423]),
-        "l2_w": ([3, 2], [-1.0534, -1.0594, -1.0530, -0.9670, -1.0603, -0.9833]),
-    },
-    # src/tests/grd.rs:36,40 (exact)
-    "grd": {"a": ([2, 2], [5.0, 7.0, 3.0, 4.0]), "a_grad": ([2, 2], [4.0, 10.0, 4.0, 2.0])},
-    # src/tests/eq.rs:55-67 (exact)
-    "eq": {"res": ([6], [0.0, 0.0, 27.0, 0.0, 0.0, 27.0]), "x_grad": ([6], [0.0, 0.0, 18.0, 0.0, 0.0, 18.0]),
-           "all_no": ([1], [0.0]), "all_yes": ([1], [1.0])},
-    # src/tests/ctrl.rs:31,64,68,86,122,126 (exact)
-    "if_ctrl": {"y": ([1], [10.0])},
-    "if_else_ctrl": {"y": ([1], [7.0]), "y_two": ([1], [13.0])},
-    "for_ctrl": {"y": ([1], [14.0])},
-    "evrty_ctrl": {"y": ([1], [-18.0]), "y_two": ([1], [72.0])},
-    # src/tests/ct.rs:39-58 (round 4)
-    "ct": {
-        "res": ([2, 4], [8.5169, 4.1459, -0.9816, 783.6786, 5.6071, -4.9606, -15.6413, 5.6242]),
-        "x_grad": ([2, 4], [-41.4012, 6.4684, 3.5990, -353566.88, 4.4253, 9.1042, -117.8715, 1.7871]),
-        "y_grad": ([2, 4], [0.2070, 0.1600, 0.5591, 0.1442, 0.0983, 0.1327, 0.1162, 0.0899]),
-    },
-    # src/tests/norm.rs:25-28,49-52 (round 4)
-    "rmsnorm": {"res": ([2, 4], [0.3651, 0.7303, 1.0954, 1.4606, 0.7581, 0.9097, 1.0613, 1.213])},
-    "layernorm": {"res": ([2, 4], [-1.3416, -0.4472, 0.4472, 1.3416, -1.1832, -0.5071, 0.169, 1.5213])},
-    # src/tests/evryt.rs:47-67 (exact; ignored upstream because its device cannot run Concat)
-    "everything": {
-        "result": ([3, 2], [1518.0, 3.0, 1518.0, 12.0, 1518.0, 48.0]),
-        "x_grad": ([2, 4], [134.0, 36.0, 108.0, 72.0, 134.0, 36.0, 108.0, 72.0]),
-        "y_grad": ([2, 4], [84.0, 112.0, 140.0, 168.0, 24.0, 32.0, 40.0, 48.0]),
-        "z_grad": ([2, 1], [332.0, 356.0]),
-        "v_grad": ([3, 1], [6.0, 12.0, 0.0]),
-    },
-}
-ROUNDED = {"nn", "ct", "rmsnorm", "layernorm"}
+# ---- golden vectors asserted by the reference's tests: tests/golden/reference_kats.json ------------
+import json as _json
+import os as _os
+
+with open(_os.path.join(_os.path.dirname(_os.path.abspath(__file__)), "golden", "reference_kats.json")) as _f:
+    _KATS_JSON = _json.load(_f)["tests"]
+GOLDEN = {name: {k: (v["dim"], v["data"]) for k, v in t["expected"].items()} for name, t in _KATS_JSON.items()}
+ROUNDED = {name for name, t in _KATS_JSON.items() if t["rounded"]}
 # ct.x_grad[3] = -353566.88 sits where cos(2x+3) ~ 0 (the reference's file calls the test "not the
 # most stable", src/tests/ct.rs:2); its last digit depends on the sin() of the runtime that produced
 # it.  That one element is compared to 4e-6 relative instead of digit-for-digit.

@@ -284,3 +284,37 @@ def test_shape_errors_are_reported(hip_device):
 def test_dot_large_tile_variant(m, k, n, hip_device):
     """Shapes that select the 256-row block tile (8 waves) of the MFMA kernel, all three operand layouts."""
     test_dot_forward_backward(m, k, n, hip_device)
+
+
+def test_single_ops_per_element(hip_device):
+    """Every element-wise command on its own (nothing to fuse), compared element by element: add, multiply, the
+    in-place forms, reciprocal, square root and the comparisons bit-exactly (both sides round correctly once);
+    exp2, log2 and sin within 1e-6 relative per element (two different libm implementations)."""
+    print("[case] single ops", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(17)
+    n = 64 * 1024
+    xa = (rng.uniform(-8.0, 8.0, n)).astype(np.float32)
+    xb = (rng.uniform(-8.0, 8.0, n)).astype(np.float32)
+    xp = (rng.uniform(1e-3, 100.0, n)).astype(np.float32)
+    xz = xa.copy()
+    xz[::7] = 0.0
+    cmds = [
+        IR.CreateMat(xa, [64, 1024], "a"), IR.CreateMat(xb, [64, 1024], "b"), IR.CreateMat(xp, [64, 1024], "p"),
+        IR.CreateMat(xz, [64, 1024], "z"), IR.CreateMat(xa.copy(), [64, 1024], "ia"), IR.CreateMat(xa.copy(), [64, 1024], "im"),
+        IR.ElwAdd(a="a", b="b", res="add"), IR.ElwMultiply(a="a", b="b", res="mul"),
+        IR.ElwAddEq(s="ia", o="b"), IR.ElwMultiplyEq(s="im", o="b"),
+        IR.Recip(a="a", res="rcp"), IR.Sqrt(a="p", res="sqrt"),
+        IR.EqualZero(a="z", res="eq"), IR.MoreZero(a="z", res="gt"), IR.LessZero(a="z", res="lt"),
+        IR.Exp2(a="a", res="exp2"), IR.Log2(a="p", res="log2"), IR.Sin(a="a", res="sin"),
+    ]
+    keep = ["add", "mul", "ia", "im", "rcp", "sqrt", "eq", "gt", "lt", "exp2", "log2", "sin"]
+    got = _run_ir(hip_device, cmds, keep)
+    ref = _run_ir(OracleDevice(), cmds, keep)
+    for k in ["add", "mul", "ia", "im", "rcp", "sqrt", "eq", "gt", "lt"]:
+        assert_exact(got[k].data, ref[k].data, k)
+    for k in ["exp2", "log2", "sin"]:
+        g = got[k].data.astype(np.float64)
+        r = ref[k].data.astype(np.float64)
+        rel = np.abs(g - r) / np.maximum(np.abs(r), 1e-30)
+        assert rel.max() <= ELW_RTOL, f"{k}: worst per-element relative error {rel.max():.3e}"
