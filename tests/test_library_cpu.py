@@ -135,3 +135,47 @@ def test_random_programs_lower_and_compile(seed):
     from oracle.interp import OracleDevice
     out = random_program(OracleDevice(), seed)
     assert not out["target"].is_none
+
+
+def test_generated_sine_is_accurate_on_the_host(tmp_path, monkeypatch):
+    """The sine the generated kernels use is plain float arithmetic (fma, rint, a polynomial), so the very text the
+    device compiles can be built for the host and compared with float64 sin: at most 2.5 ulp everywhere, including
+    the floats next to multiples of pi (where a sloppy range reduction loses all relative accuracy), tiny arguments,
+    and arguments beyond the fast range, which go to the library routine."""
+    import subprocess
+    import numpy as np
+    monkeypatch.setenv("ADHIP_DUMP_SOURCE", "1")
+    proc = IR.IRProcedure("main", [IR.CreateMat(np.zeros(8, np.float32), [2, 4], "a"), IR.Sin(a="a", res="s"), IR.EX()])
+    text = lower_describe(proc, {"s"})
+    m = re.search(r"static __device__ __forceinline__ float adhip_sinf\(float x\) \{.*?\n\}\n", text, re.S)
+    assert m, "the generated source no longer defines adhip_sinf"
+    assert "adhip_sinf(" in text[m.end():], "the Sin command does not call adhip_sinf"
+    body = m.group(0).replace("static __device__ __forceinline__", "static inline")
+    src = tmp_path / "sine.cpp"
+    src.write_text("#include <math.h>\n" + body +
+                   'extern "C" void apply(const float* x, float* y, long n) { for (long i = 0; i < n; ++i) y[i] = adhip_sinf(x[i]); }\n')
+    so = tmp_path / "sine.so"
+    subprocess.run(["g++", "-O2", "-std=c++20", "-ffp-contract=off", "-mfma", "-shared", "-fPIC", "-o", str(so), str(src)], check=True)
+    lib = ctypes.CDLL(str(so))
+    lib.apply.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    rng = np.random.default_rng(5)
+    k = np.arange(1, 10400, dtype=np.float64)
+    near = (k * np.pi).astype(np.float32)
+    near_half = ((k - 0.5) * np.pi).astype(np.float32)
+    xs = np.concatenate([
+        rng.uniform(-8, 8, 2_000_000), rng.uniform(-32768, 32768, 2_000_000), 10.0 ** rng.uniform(-30, 0, 200_000),
+        near, np.nextafter(near, np.float32(0)), np.nextafter(near, np.float32(1e9)), -near, near_half, -near_half,
+        rng.uniform(32768, 1e9, 100_000), [0.0, 32768.0, -32768.0, np.nextafter(np.float32(32768), np.float32(1e9))],
+    ]).astype(np.float32)
+    ys = np.empty_like(xs)
+    lib.apply(xs.ctypes.data, ys.ctypes.data, xs.size)
+    ref = np.sin(xs.astype(np.float64))
+    ulp = np.spacing(np.abs(ref).astype(np.float32)).astype(np.float64)
+    err = np.abs(ys.astype(np.float64) - ref) / np.maximum(ulp, np.finfo(np.float32).tiny)
+    worst = int(np.argmax(err))
+    assert err[worst] <= 2.5, f"sin({xs[worst]!r}) = {ys[worst]!r}, {err[worst]:.2f} ulp from {ref[worst]!r}"
+    lib.apply.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    special = np.array([np.nan, np.inf, -np.inf], dtype=np.float32)
+    out = np.empty_like(special)
+    lib.apply(special.ctypes.data, out.ctypes.data, 3)
+    assert np.isnan(out).all()
