@@ -8,6 +8,8 @@ namespace {
 struct Reader {
     const uint8_t* p;
     const uint8_t* end;
+    const uint8_t* base = nullptr;
+    std::vector<size_t>* payload_offsets = nullptr;
     void need(size_t n) { ADHIP_CHECK((size_t)(end - p) >= n, "program stream truncated"); }
     uint8_t u8() { need(1); return *p++; }
     uint32_t u32() { need(4); uint32_t v; memcpy(&v, p, 4); p += 4; return v; }
@@ -44,6 +46,7 @@ std::unique_ptr<Proc> parse_proc(Reader& r, int depth) {
         case T_CREATE_MAT: {
             c.res = r.str();
             c.dims = r.dims();
+            if (r.payload_offsets) r.payload_offsets->push_back((size_t)(r.p - r.base));
             c.host = (const float*)(uintptr_t)r.u64();
             c.count = r.u64();
             ADHIP_CHECK((int64_t)c.count == numel(c.dims), "CreateMat %s: %llu values for dim %s", c.res.c_str(),
@@ -108,10 +111,10 @@ std::unique_ptr<Proc> parse_proc(Reader& r, int depth) {
 }
 }  // namespace
 
-std::unique_ptr<Proc> parse_program(const uint8_t* data, size_t len) {
+std::unique_ptr<Proc> parse_program(const uint8_t* data, size_t len, std::vector<size_t>* payload_offsets) {
     ADHIP_CHECK(data != nullptr && len >= 8, "program stream too short");
     ADHIP_CHECK(memcmp(data, "ADIR", 4) == 0, "bad program magic");
-    Reader r{data + 4, data + len};
+    Reader r{data + 4, data + len, data, payload_offsets};
     uint32_t ver = r.u32();
     ADHIP_CHECK(ver == 1, "unsupported program version %u", ver);
     auto p = parse_proc(r, 0);

@@ -38,7 +38,8 @@ struct Proc {
 };
 
 // Parses the byte stream produced by the host-side serialiser.  Throws Error on malformed input.
-std::unique_ptr<Proc> parse_program(const uint8_t* data, size_t len);
+// `payload_offsets`, when given, receives the byte offset of every CreateMat host-pointer field in stream order.
+std::unique_ptr<Proc> parse_program(const uint8_t* data, size_t len, std::vector<size_t>* payload_offsets = nullptr);
 
 const char* tag_name(Tag t);
 

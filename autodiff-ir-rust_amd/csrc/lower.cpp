@@ -1415,8 +1415,15 @@ struct Lowerer {
         collect_alias_srcs(prog);
         IdSet end_live;
         for (auto& d : deps) end_live.insert(d);
-        live_block(prog, end_live);
+        const IdSet start_live = live_block(prog, end_live);
         lower_block(prog, plan->steps, true);
+        // an id that is live when the program starts can be read before it is written (defined only on some paths,
+        // or only inside a loop that may run zero times): its buffer starts as zeros.  Every other buffer is fully
+        // written by a kernel or an upload before its first read and needs no clearing.
+        for (const std::string& id : start_live) {
+            auto hb = home_buf.find(id);
+            if (hb != home_buf.end()) plan->buffers[hb->second].zero_init = true;
+        }
         // results
         for (const std::string& d : deps) {
             auto it = env.find(d);

@@ -15,6 +15,7 @@ struct PlanBuffer {
     const float* host = nullptr;  // upload source (borrowed until upload)
     int64_t host_elems = 0;
     int slot = -1;                // TEMP: physical slot shared with other temporaries
+    bool zero_init = false;       // HOME: may be read before any kernel has written it; cleared at upload
 };
 
 struct KernelDef {

@@ -16,6 +16,7 @@
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <set>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -61,8 +62,17 @@ struct adhip_ctx {
     std::map<std::string, std::shared_ptr<Module>> modules;  // by source text
     std::map<std::string, HostResult> results;
     float* pinned = nullptr;  // small pinned area for predicate read-back
+    char* stage = nullptr;    // pinned staging area for small uploads and read-backs
     double compile_ms = 0;
+    // Programs kept from earlier adhip_execute calls, most recently used first: a caller that executes the same
+    // program again (a training loop) skips lowering, module loading and allocation.
+    struct CachedExec { std::string key; adhip_program* prog; size_t bytes; };
+    std::vector<CachedExec> exec_cache;
 };
+constexpr size_t kStageBytes = 1 << 20;        // pinned staging area
+constexpr size_t kStageMaxItem = 64 << 10;     // larger transfers go directly
+constexpr size_t kExecCacheEntries = 4;        // programs kept per context
+constexpr size_t kExecCacheBytes = size_t(4) << 30;  // device memory the kept programs may hold together
 
 struct adhip_program {
     adhip_ctx* ctx = nullptr;
@@ -78,6 +88,10 @@ struct adhip_program {
     std::map<std::pair<const void*, size_t>, hipGraphExec_t> graphs;
     std::vector<hipGraph_t> graph_objs;
     bool use_graphs = true;
+    std::set<std::pair<const void*, size_t>> seen_runs;  // launch runs executed once already
+    std::vector<const float*> payloads;  // CreateMat host pointers in stream order (programs made by adhip_execute)
+    std::vector<int> payload_of;         // per plan buffer: index into `payloads`, -1 if none
+    size_t device_bytes = 0;
     int* flags = nullptr;            // device flags of predicated blocks
     hipFunction_t flag_fn = nullptr;
     uint64_t flag_launches = 0;
@@ -209,13 +223,14 @@ std::vector<std::string> dep_vector(const char* const* dep_ids, size_t n) {
     return d;
 }
 
-adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len, const char* const* dep_ids, size_t n) {
+adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len, const char* const* dep_ids, size_t n,
+                              std::vector<size_t>* payload_offsets = nullptr) {
     HIP_OK(hipSetDevice(ctx->device));
     std::unique_ptr<adhip_program> p(new adhip_program());
     p->ctx = ctx;
     const char* genv = getenv("ADHIP_GRAPHS");
     if (genv && *genv == '0') p->use_graphs = false;
-    p->ir = parse_program(program, len);
+    p->ir = parse_program(program, len, payload_offsets);
     p->plan = lower_program(*p->ir, dep_vector(dep_ids, n));
     Plan& plan = *p->plan;
     try {
@@ -231,6 +246,7 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
             void* q = nullptr;
             HIP_OK(hipMalloc(&q, (size_t)std::max<int64_t>(plan.slot_elems[s], 1) * sizeof(float)));
             p->owned.push_back(q);
+            p->device_bytes += (size_t)std::max<int64_t>(plan.slot_elems[s], 1) * sizeof(float);
             slot_ptr[s] = q;
         }
         if (plan.n_flags > 0) {
@@ -249,6 +265,7 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
             void* q = nullptr;
             HIP_OK(hipMalloc(&q, (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float)));
             p->owned.push_back(q);
+            p->device_bytes += (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float);
             p->buf_ptr[i] = q;
         }
     } catch (...) {
@@ -262,12 +279,25 @@ void program_upload(adhip_program* p) {
     adhip_ctx* ctx = p->ctx;
     HIP_OK(hipSetDevice(ctx->device));
     Plan& plan = *p->plan;
+    size_t staged = 0;
     for (size_t i = 0; i < plan.buffers.size(); ++i) {
         const PlanBuffer& b = plan.buffers[i];
         if (b.kind == PlanBuffer::TEMP) continue;
         if (b.host && b.host_elems > 0) {
-            HIP_OK(hipMemcpyAsync(p->buf_ptr[i], b.host, (size_t)b.host_elems * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
-        } else if (b.kind == PlanBuffer::HOME) {
+            const size_t nb = (size_t)b.host_elems * sizeof(float);
+            const void* src = b.host;
+            if (nb <= kStageMaxItem) {
+                // small payloads go through pinned memory, so that the copies queue up instead of each one waiting
+                if (staged + nb > kStageBytes) {
+                    HIP_OK(hipStreamSynchronize(ctx->stream));
+                    staged = 0;
+                }
+                memcpy(ctx->stage + staged, b.host, nb);
+                src = ctx->stage + staged;
+                staged += (nb + 255) & ~size_t(255);
+            }
+            HIP_OK(hipMemcpyAsync(p->buf_ptr[i], src, nb, hipMemcpyHostToDevice, ctx->stream));
+        } else if (b.kind == PlanBuffer::HOME && b.zero_init) {
             HIP_OK(hipMemsetAsync(p->buf_ptr[i], 0, (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float), ctx->stream));
         }
     }
@@ -360,6 +390,8 @@ bool replay_run(adhip_program* p, const std::vector<Step>& steps, size_t first, 
     adhip_ctx* ctx = p->ctx;
     auto key = std::make_pair((const void*)&steps, first);
     auto it = p->graphs.find(key);
+    // the first time a run is met it is launched directly: a program that runs once never pays for a capture
+    if (it == p->graphs.end() && p->seen_runs.insert(key).second) return false;
     if (it == p->graphs.end()) {
         hipGraph_t graph = nullptr;
         HIP_OK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
@@ -484,16 +516,32 @@ void program_readback(adhip_program* p) {
     adhip_ctx* ctx = p->ctx;
     HIP_OK(hipSetDevice(ctx->device));
     ctx->results.clear();
+    struct Staged { HostResult* r; size_t off, nb; };
+    std::vector<Staged> staged;
+    size_t used = 0;
+    auto drain = [&] {
+        HIP_OK(hipStreamSynchronize(ctx->stream));
+        for (auto& st : staged) memcpy(st.r->data.data(), ctx->stage + st.off, st.nb);
+        staged.clear();
+        used = 0;
+    };
     for (auto& kv : p->plan->results) {
-        HostResult r;
+        HostResult& r = ctx->results[kv.first];
         for (auto d : kv.second.shape) r.dims.push_back((uint64_t)d);
         const int64_t ne = numel(kv.second.shape);
         r.data.resize((size_t)ne);
-        if (ne > 0)
-            HIP_OK(hipMemcpyAsync(r.data.data(), p->buf_ptr[kv.second.buf], (size_t)ne * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
-        ctx->results[kv.first] = std::move(r);
+        if (ne <= 0) continue;
+        const size_t nb = (size_t)ne * sizeof(float);
+        if (nb <= kStageMaxItem) {
+            if (used + nb > kStageBytes) drain();
+            HIP_OK(hipMemcpyAsync(ctx->stage + used, p->buf_ptr[kv.second.buf], nb, hipMemcpyDeviceToHost, ctx->stream));
+            staged.push_back({&r, used, nb});
+            used += (nb + 255) & ~size_t(255);
+        } else {
+            HIP_OK(hipMemcpyAsync(r.data.data(), p->buf_ptr[kv.second.buf], nb, hipMemcpyDeviceToHost, ctx->stream));
+        }
     }
-    HIP_OK(hipStreamSynchronize(ctx->stream));
+    drain();
 }
 
 template <class F>
@@ -536,6 +584,7 @@ int adhip_create(int device_ordinal, adhip_ctx** out) {
         ctx->arch = arch;
         HIP_OK(hipStreamCreate(&ctx->stream));
         HIP_OK(hipHostMalloc((void**)&ctx->pinned, 64 * sizeof(float), hipHostMallocDefault));
+        HIP_OK(hipHostMalloc((void**)&ctx->stage, kStageBytes, hipHostMallocDefault));
         *out = ctx.release();
     });
 }
@@ -543,8 +592,11 @@ int adhip_create(int device_ordinal, adhip_ctx** out) {
 void adhip_destroy(adhip_ctx* ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
+    for (auto& e : ctx->exec_cache) program_free(e.prog);
+    ctx->exec_cache.clear();
     ctx->modules.clear();
     if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+    if (ctx->stage) (void)hipHostFree(ctx->stage);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -555,16 +607,87 @@ int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, co
     if (!ctx) return 2;
     return guarded(ctx, [&] {
         ctx->results.clear();
-        adhip_program* p = program_create(ctx, program, program_len, dep_ids, n_dep_ids);
+        const char* cenv = getenv("ADHIP_EXEC_CACHE");
+        const bool caching = !(cenv && *cenv == '0');
+        adhip_program* p = nullptr;
+        std::string key;
+        std::vector<size_t> offs;
+        std::vector<const float*> ptrs;
+        if (caching && program && program_len >= 8) {
+            // key: the stream with every payload pointer blanked, plus the keep list
+            parse_program(program, program_len, &offs);
+            key.assign((const char*)program, program_len);
+            for (size_t o : offs) {
+                uint64_t v;
+                memcpy(&v, program + o, 8);
+                ptrs.push_back((const float*)(uintptr_t)v);
+                memset(&key[o], 0, 8);
+            }
+            for (const std::string& d : dep_vector(dep_ids, n_dep_ids)) { key.push_back('\0'); key += d; }
+            for (size_t i = 0; i < ctx->exec_cache.size(); ++i) {
+                if (ctx->exec_cache[i].key != key) continue;
+                adhip_program* q = ctx->exec_cache[i].prog;
+                // the kept program can be re-bound if payloads that shared a pointer before still share one
+                bool ok = q->payloads.size() == ptrs.size();
+                for (size_t a = 0; ok && a < ptrs.size(); ++a)
+                    for (size_t b = a + 1; ok && b < ptrs.size(); ++b)
+                        if (q->payloads[a] == q->payloads[b] && ptrs[a] != ptrs[b]) ok = false;
+                auto entry = ctx->exec_cache[i];
+                ctx->exec_cache.erase(ctx->exec_cache.begin() + (long)i);
+                if (ok) {
+                    for (size_t bi = 0; bi < q->plan->buffers.size(); ++bi)
+                        if (q->payload_of[bi] >= 0) q->plan->buffers[bi].host = ptrs[(size_t)q->payload_of[bi]];
+                    q->payloads = ptrs;
+                    ctx->exec_cache.insert(ctx->exec_cache.begin(), entry);
+                    p = q;
+                } else {
+                    program_free(q);
+                }
+                break;
+            }
+        }
+        const bool reused = p != nullptr;
+        if (!p) {
+            offs.clear();
+            p = program_create(ctx, program, program_len, dep_ids, n_dep_ids, &offs);
+        }
+        bool keep = reused;
         try {
+            if (!reused && caching && p->device_bytes <= kExecCacheBytes) {
+                p->payloads = ptrs;
+                p->payload_of.assign(p->plan->buffers.size(), -1);
+                keep = true;
+                for (size_t bi = 0; bi < p->plan->buffers.size() && keep; ++bi) {
+                    const float* h = p->plan->buffers[bi].host;
+                    if (!h) continue;
+                    for (size_t a = 0; a < ptrs.size(); ++a)
+                        if (ptrs[a] == h) { p->payload_of[bi] = (int)a; break; }
+                    if (p->payload_of[bi] < 0) keep = false;  // a payload the stream does not name: cannot be re-bound
+                }
+                if (keep) {
+                    ctx->exec_cache.insert(ctx->exec_cache.begin(), {key, p, p->device_bytes});
+                    size_t total = 0, n_keep = 0;
+                    for (; n_keep < ctx->exec_cache.size() && n_keep < kExecCacheEntries; ++n_keep) {
+                        if (total + ctx->exec_cache[n_keep].bytes > kExecCacheBytes && n_keep > 0) break;
+                        total += ctx->exec_cache[n_keep].bytes;
+                    }
+                    while (ctx->exec_cache.size() > n_keep) {
+                        program_free(ctx->exec_cache.back().prog);
+                        ctx->exec_cache.pop_back();
+                    }
+                }
+            }
             program_upload(p);
             program_run(p);
             program_readback(p);
         } catch (...) {
+            // a program that failed is not kept
+            for (size_t i = 0; i < ctx->exec_cache.size(); ++i)
+                if (ctx->exec_cache[i].prog == p) { ctx->exec_cache.erase(ctx->exec_cache.begin() + (long)i); break; }
             program_free(p);
             throw;
         }
-        program_free(p);
+        if (!keep) program_free(p);
     });
 }
 

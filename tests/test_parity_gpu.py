@@ -318,3 +318,40 @@ def test_single_ops_per_element(hip_device):
         r = ref[k].data.astype(np.float64)
         rel = np.abs(g - r) / np.maximum(np.abs(r), 1e-30)
         assert rel.max() <= ELW_RTOL, f"{k}: worst per-element relative error {rel.max():.3e}"
+
+
+def test_repeated_execute_rebinds_payloads(hip_device):
+    """A program executed again (same commands, new CreateMat contents) reuses the kept plan and buffers but must see
+    the new contents, start from fresh device state, and honour a different keep list; more distinct programs than
+    the context keeps must still all be right."""
+    print("[case] repeated execute", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(23)
+
+    def prog(x, w, n_iter):
+        body = IR.IRProcedure("body", [IR.ElwAddEq(s="acc", o="x"), IR.ElwAddEq(s="i", o="one"),
+                                       IR.ElwAdd(a="i", b="lim", res="t"), IR.LessZero(a="t", res="c")])
+        return [IR.CreateMat(x, [4, 8], "x"), IR.CreateMat(w, [8, 3], "w"), IR.CreateMat(np.zeros(32, np.float32), [4, 8], "acc"),
+                IR.CreateMat(np.zeros(1, np.float32), [1], "i"), IR.CreateMat(np.ones(1, np.float32), [1], "one"),
+                IR.CreateMat(np.array([-float(n_iter)], np.float32), [1], "lim"),
+                IR.ElwAdd(a="i", b="lim", res="t"), IR.LessZero(a="t", res="c"),
+                IR.While(conditional_var="c", block=body), IR.DotProduct(a="acc", b="w", res="y")]
+
+    for trial in range(4):
+        x = rng.standard_normal(32).astype(np.float32)
+        w = rng.standard_normal(24).astype(np.float32)
+        n_iter = 2 + trial          # same stream, different payload: the trip count is read on the device
+        keep = ["y", "acc"] if trial != 2 else ["y"]
+        out = _run_ir(hip_device, prog(x, w, n_iter), keep)
+        acc = np.zeros(32, np.float32)
+        for _ in range(n_iter):
+            acc = acc + x
+        assert_exact(out["acc"].data, acc, f"trial {trial} acc") if "acc" in keep else None
+        assert_close(out["y"].data, (acc.reshape(4, 8).astype(np.float64) @ w.reshape(8, 3)).reshape(-1), RED_RTOL * math.sqrt(8), f"trial {trial} y")
+        if trial == 2:
+            assert hip_device.get_tensor("acc").is_none
+    # more distinct programs than the context keeps, then the first one again
+    for width in (4, 8, 12, 16, 20, 24, 4):
+        v = rng.standard_normal(2 * width).astype(np.float32)
+        out = _run_ir(hip_device, [IR.CreateMat(v, [2, width], "v"), IR.Sum(a="v", res="s")], ["s"])
+        assert_close(out["s"].data, v.reshape(2, width).astype(np.float64).sum(1), RED_RTOL * math.sqrt(width), f"width {width}")
