@@ -583,7 +583,7 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
 int64_t elw_colsum_tiles(int64_t rows, int64_t cols) {
     const int64_t bx = (cols / 4 + 255) / 256;
     int64_t tiles = (1024 + bx - 1) / bx;            // four blocks per CU on 256 CUs
-    tiles = std::min<int64_t>(tiles, 128);                             // the partials are summed by few blocks
+    tiles = std::min<int64_t>(tiles, 256);                             // bounds the partial sums the second pass reads
     tiles = std::min<int64_t>(tiles, std::max<int64_t>(rows / 8, 1));  // and at least 8 rows per tile
     return std::max<int64_t>(tiles, 1);
 }

@@ -593,7 +593,7 @@ struct Lowerer {
         Affine2D a;
         if (!tref_affine2d(s->in[0], a)) return nullptr;
         const int64_t V = s->in[0].shape[0], R = s->in[0].shape[1];
-        if (!op_is_elw(a.base->op) || a.offset != 0 || a.s0 != 1 || a.s1 != V) return nullptr;
+        if (!(op_is_elw(a.base->op) || in_mem(a.base)) || a.offset != 0 || a.s0 != 1 || a.s1 != V) return nullptr;
         if (numel(a.base->shape) != V * R || V % 4 != 0 || R < 16 || V * R < (int64_t(1) << 16)) return nullptr;
         rows = R;
         cols = V;
@@ -892,6 +892,30 @@ struct Lowerer {
                     if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
                     for (Node* m : G.members)
                         if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
+                }
+                if (target < 0) {
+                    // no pass computes E itself; one that already loads, element for element, everything E is made
+                    // of can still produce the sum without reading anything more (x.sum(0) next to dx = f(x))
+                    std::map<Node*, bool> er;
+                    if (in_mem(E)) er[E] = true;
+                    else collect_reads(E, er);
+                    bool ident = !er.empty();
+                    for (auto& kv : er) ident = ident && kv.second;
+                    for (size_t g = 0; ident && g < groups.size() && target < 0; ++g) {
+                        Group& G = groups[g];
+                        if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
+                        if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
+                        bool all = true;
+                        for (auto& kv : er) {
+                            bool found = false;
+                            for (Node* m : G.members) {
+                                auto it = reads[m].find(kv.first);
+                                if (it != reads[m].end() && it->second) { found = true; break; }
+                            }
+                            all = all && found;
+                        }
+                        if (all) target = (int)g;
+                    }
                 }
                 if (target < 0) continue;
                 // everything that reads S must run after the pass that now produces it

@@ -1,0 +1,207 @@
+"""Random IR programs with nested control flow, written directly as commands (not through the graph front end), for
+differential testing of the device against the oracle.
+
+What they stress: ids redefined inside loops and branches, in-place updates next to reads of the old value, views
+taken before a loop and used inside it (late binding), sums and matmuls inside loop bodies, values that are only
+conditionally rewritten, counted loops, data-dependent loops and branches.
+
+Two families of tensors keep the comparison meaningful:
+  * integer-valued ones (names k*): only additions, negations and multiplications by small integers, so every
+    device computes them exactly; all predicates are derived from these, so both sides take the same path;
+  * real-valued ones (names f*): contractive arithmetic (scaled sums, sines, exp2 of bounded arguments), compared
+    with a tolerance.
+Every id is created at the top level before any control flow, blocks only redefine existing ids, so no path reads an
+undefined id."""
+import numpy as np
+
+from adhip import ir as IR
+
+SHAPES = [[4, 6], [6, 4], [6], [4], [1]]
+
+
+class _Gen:
+    def __init__(self, seed):
+        self.rng = np.random.default_rng(seed)
+        self.n = 0
+        self.counters = 0
+        self.ints = {}    # id -> shape
+        self.reals = {}
+        self.top = []
+        self.early_views = []   # [6,4] views of [4,6] tensors, defined before the first control command
+
+    def fresh(self, prefix):
+        self.n += 1
+        return f"{prefix}{self.n}"
+
+    def pick(self, pool, shape=None):
+        c = [i for i, s in pool.items() if shape is None or s == shape]
+        return c[int(self.rng.integers(len(c)))] if c else None
+
+    def const(self, out, value, shape):
+        cid = self.fresh("c")
+        out.append(IR.CreateConstant(float(value), cid, list(shape)))
+        return cid
+
+    # ---- one straight-line command group appended to `out`
+    def compute(self, out, depth):
+        rng = self.rng
+        kind = int(rng.integers(10))
+        if kind == 0:      # real: a = 0.5 * (b + c)
+            a = self.pick(self.reals)
+            sh = self.reals[a]
+            b, c = self.pick(self.reals, sh), self.pick(self.reals, sh)
+            t = self.fresh("t")
+            out += [IR.ElwAdd(a=b, b=c, res=t), IR.ElwMultiply(a=t, b=self.const(out, 0.5, sh), res=a)]
+        elif kind == 1:    # real: a = sin(b) * c  (in place when a == b)
+            a = self.pick(self.reals)
+            sh = self.reals[a]
+            b, c = self.pick(self.reals, sh), self.pick(self.reals, sh)
+            t = self.fresh("t")
+            out += [IR.Sin(a=b, res=t), IR.ElwMultiply(a=t, b=c, res=a)]
+        elif kind == 2:    # real, in place: a += 0.25 * b ; a *= 0.5
+            a = self.pick(self.reals)
+            sh = self.reals[a]
+            b = self.pick(self.reals, sh)
+            t = self.fresh("t")
+            out += [IR.ElwMultiply(a=b, b=self.const(out, 0.25, sh), res=t), IR.ElwAddEq(s=a, o=t),
+                    IR.ElwMultiplyEq(s=a, o=self.const(out, 0.5, sh))]
+        elif kind == 3:    # real: row sums of a [4,6] spread back over another [4,6] through broadcast
+            a = self.pick(self.reals, [4, 6])
+            b = self.pick(self.reals, [4, 6])
+            s, v, w, t = self.fresh("t"), self.fresh("t"), self.fresh("t"), self.fresh("t")
+            out += [IR.Sum(a=b, res=s), IR.View(a=s, target_dim=[4, 1], res=v), IR.Broadcast(a=v, dim=1, r=6, res=w),
+                    IR.ElwMultiply(a=w, b=self.const(out, 1.0 / 8.0, [4, 6]), res=t), IR.ElwAdd(a=t, b=a, res=a),
+                    IR.ElwMultiplyEq(s=a, o=self.const(out, 0.5, [4, 6]))]
+        elif kind == 4:    # real: column sums via permute, written to a [6]
+            a = self.pick(self.reals, [6])
+            b = self.pick(self.reals, [4, 6])
+            p, s = self.fresh("t"), self.fresh("t")
+            out += [IR.Permute(a=b, p=[1, 0], res=p), IR.Sum(a=p, res=s),
+                    IR.ElwMultiply(a=s, b=self.const(out, 0.25, [6]), res=a)]
+        elif kind == 5:    # real: [4,6] x [6,4] -> [4,4] -> row sums -> [4]
+            a = self.pick(self.reals, [4])
+            x, y = self.pick(self.reals, [4, 6]), self.pick(self.reals, [6, 4])
+            d, s = self.fresh("t"), self.fresh("t")
+            out += [IR.DotProduct(a=x, b=y, res=d), IR.Sum(a=d, res=s),
+                    IR.ElwMultiply(a=s, b=self.const(out, 1.0 / 32.0, [4]), res=a)]
+        elif kind == 6:    # real: transposed copy between the two matrix shapes (out[i] = in[p[i]]), through a fresh
+            a = self.pick(self.reals, [6, 4])   # view or through one that was taken before any control flow
+            if self.early_views and rng.integers(2):
+                p = self.early_views[int(rng.integers(len(self.early_views)))]
+                out += [IR.ElwMultiply(a=p, b=self.const(out, 0.5, [6, 4]), res=a)]
+            else:
+                b = self.pick(self.reals, [4, 6])
+                p = self.fresh("t")
+                out += [IR.Permute(a=b, p=[1, 0], res=p), IR.Contigious(a=p, res=a)]
+        elif kind == 7:    # int: a = b + c or a = -b or a += small
+            a = self.pick(self.ints)
+            sh = self.ints[a]
+            r = int(rng.integers(3))
+            if r == 0:
+                out.append(IR.ElwAdd(a=self.pick(self.ints, sh), b=self.pick(self.ints, sh), res=a))
+            elif r == 1:
+                out.append(IR.ElwMultiply(a=self.pick(self.ints, sh), b=self.const(out, -1.0, sh), res=a))
+            else:
+                out.append(IR.ElwAddEq(s=a, o=self.const(out, float(rng.integers(-3, 4)), sh)))
+        elif kind == 8:    # int: scalar k[1] = sum of a [4] (through a [1,4] view)
+            a = self.pick(self.ints, [1])
+            b = self.pick(self.ints, [4])
+            v, s = self.fresh("t"), self.fresh("t")
+            out += [IR.View(a=b, target_dim=[1, 4], res=v), IR.Sum(a=v, res=s), IR.ElwAdd(a=s, b=a, res=a)]
+        else:              # int: a [4] += broadcast of a scalar
+            a = self.pick(self.ints, [4])
+            b = self.pick(self.ints, [1])
+            w = self.fresh("t")
+            out += [IR.Broadcast(a=b, dim=0, r=4, res=w), IR.ElwAddEq(s=a, o=w)]
+
+    def predicate(self, out):
+        """A [1] predicate (0/1) from an integer-valued scalar: k > c, k < c or k == c."""
+        k = self.pick(self.ints, [1])
+        t, p = self.fresh("t"), self.fresh("p")
+        out.append(IR.ElwAdd(a=k, b=self.const(out, -float(self.rng.integers(-4, 5)), [1]), res=t))
+        cmp = [IR.MoreZero, IR.LessZero, IR.EqualZero][int(self.rng.integers(3))]
+        out.append(cmp(a=t, res=p))
+        return p
+
+    def block(self, out, depth, n_cmds):
+        for _ in range(n_cmds):
+            r = int(self.rng.integers(10))
+            if depth < 2 and r == 0:
+                self.loop(out, depth, counted=True)
+            elif depth < 2 and r == 1:
+                self.loop(out, depth, counted=False)
+            elif depth < 3 and r == 2:
+                self.branch(out, depth)
+            else:
+                self.compute(out, depth)
+
+    def loop(self, out, depth, counted):
+        """Trip count 0..3.  Counted: the `x += 1; t = x + (-n); c = t < 0` shape of the front end's for-loop.
+        Otherwise the predicate is the product of that comparison and a data-dependent one."""
+        self.counters += 1
+        i, t, c = f"i{self.counters}", f"it{self.counters}", f"ic{self.counters}"
+        n = int(self.rng.integers(0, 4))
+        self.top.append(IR.CreateMat(np.zeros(1, np.float32), [1], i))
+        body = []
+        self.block(body, depth + 1, int(self.rng.integers(1, 4)))
+
+        def head(dst):
+            dst.append(IR.ElwAdd(a=i, b=self.const(dst, -float(n), [1]), res=t))
+            dst.append(IR.LessZero(a=t, res=c))
+        out.append(IR.ElwMultiplyEq(s=i, o=self.const(out, 0.0, [1])))   # the counter restarts each time the loop is met
+        head(out)
+        cond = c
+        body.append(IR.ElwAddEq(s=i, o=self.const(body, 1.0, [1])))
+        head(body)
+        if not counted:
+            cond = f"iw{self.counters}"
+            k = self.pick(self.ints, [1])
+            lim = float(self.rng.integers(0, 12))
+
+            def data_pred(dst):
+                tt, pp = self.fresh("t"), self.fresh("p")
+                dst.append(IR.ElwAdd(a=k, b=self.const(dst, -lim, [1]), res=tt))
+                dst.append(IR.LessZero(a=tt, res=pp))
+                dst.append(IR.ElwMultiply(a=c, b=pp, res=cond))
+            data_pred(out)
+            data_pred(body)
+        out.append(IR.While(conditional_var=cond, block=IR.IRProcedure(f"loop{self.counters}", body)))
+
+    def branch(self, out, depth):
+        arms = []
+        for _ in range(int(self.rng.integers(1, 3))):
+            p = self.predicate(out)
+            body = []
+            self.block(body, depth + 1, int(self.rng.integers(1, 3)))
+            arms.append((p, IR.IRProcedure(self.fresh("arm"), body)))
+        else_proc = None
+        if self.rng.integers(2):
+            body = []
+            self.block(body, depth + 1, int(self.rng.integers(1, 3)))
+            else_proc = IR.IRProcedure(self.fresh("else"), body)
+        out.append(IR.If(conditions=arms, else_proc=else_proc))
+
+
+def random_control_program(seed: int):
+    """Returns (procedure, keep list, names of the integer-valued ids)."""
+    g = _Gen(seed)
+    rng = g.rng
+    for sh in SHAPES:
+        for _ in range(2):
+            rid = g.fresh("f")
+            g.reals[rid] = sh
+            g.top.append(IR.CreateMat(rng.uniform(-1.0, 1.0, int(np.prod(sh))).astype(np.float32), list(sh), rid))
+    for sh in ([4], [4], [1], [1], [1]):
+        kid = g.fresh("k")
+        g.ints[kid] = sh
+        g.top.append(IR.CreateMat(rng.integers(-3, 4, int(np.prod(sh))).astype(np.float32), list(sh), kid))
+    # views taken before any control flow; blocks read them after their sources changed (views bind late)
+    for rid in [i for i, sh in g.reals.items() if sh == [4, 6]]:
+        v = g.fresh("v")
+        g.top.append(IR.Permute(a=rid, p=[1, 0], res=v))
+        g.early_views.append(v)
+    main = []
+    g.block(main, 0, int(rng.integers(6, 12)))
+    keep = sorted(list(g.reals) + list(g.ints) + [f"i{j + 1}" for j in range(g.counters)])
+    proc = IR.IRProcedure("main", g.top + main + [IR.EX()])
+    return proc, keep, sorted(g.ints)

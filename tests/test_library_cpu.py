@@ -179,3 +179,16 @@ def test_generated_sine_is_accurate_on_the_host(tmp_path, monkeypatch):
     out = np.empty_like(special)
     lib.apply(special.ctypes.data, out.ctypes.data, 3)
     assert np.isnan(out).all()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_control_flow_programs_lower(seed):
+    """Random nested loops / branches over redefined ids: the lowering must accept them (range checks of every
+    generated load run here too); the first few are also compiled for gfx950."""
+    from fuzz_control import random_control_program
+    proc, keep, _ = random_control_program(seed)
+    text = lower_describe(proc, set(keep))
+    assert "exit" in text
+    if seed < 3:
+        rc, msg = _compile_check(proc, set(keep))
+        assert rc == 0, msg

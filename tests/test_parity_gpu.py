@@ -355,3 +355,26 @@ def test_repeated_execute_rebinds_payloads(hip_device):
         v = rng.standard_normal(2 * width).astype(np.float32)
         out = _run_ir(hip_device, [IR.CreateMat(v, [2, width], "v"), IR.Sum(a="v", res="s")], ["s"])
         assert_close(out["s"].data, v.reshape(2, width).astype(np.float64).sum(1), RED_RTOL * math.sqrt(width), f"width {width}")
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_control_flow_matches_oracle(seed, hip_device):
+    """Random programs with nested counted loops, data-dependent loops and branches (tests/fuzz_control.py):
+    integer-valued tensors (which drive every predicate) bit-exact, the others within the element-wise / reduction
+    tolerance."""
+    print(f"[case] control fuzz seed {seed}", flush=True)
+    from fuzz_control import random_control_program
+    proc, keep, ints = random_control_program(seed)
+    ref_dev = OracleDevice()
+    ref_dev.execute(proc, set(keep))
+    ref = {k: ref_dev.get_tensor(k) for k in keep}
+    if max(float(np.max(np.abs(ref[k].data))) for k in ints) >= 2.0 ** 22:
+        pytest.skip("integer-valued tensors left the exactly representable range")
+    hip_device.execute(proc, set(keep))
+    for k in keep:
+        got = hip_device.get_tensor(k)
+        assert not got.is_none and got.dim == ref[k].dim, k
+        if k in ints or k.startswith("i"):
+            assert_exact(got.data, ref[k].data, k)
+        else:
+            assert_close(got.data, ref[k].data, 2e-5, k, scale=max(1.0, float(np.max(np.abs(ref[k].data)))))
