@@ -825,12 +825,13 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         }
         const int64_t CH = (RV + chunks - 1) / chunks;  // vector elements per chunk
         k.kind = side ? "reduce_row_store" : "reduce_row";
-        std::string sig = side ? "const int* __restrict__ guard, float* out" : "const int* __restrict__ guard, float* __restrict__ out";
+        // no __restrict__: the result (and a stored operand) may share a buffer with an input it replaces in place
+        std::string sig = "const int* __restrict__ guard, float* out";
         std::vector<Node*> order{const_cast<Node*>(n)};
         if (side)
             for (size_t i = 0; i < spec.side_outputs.size(); ++i) { sig += strf(", float* w%zu", i); order.push_back(spec.side_outputs[i]); }
         // a stored value may update one of the inputs in place, so nothing is restrict-qualified then
-        for (auto& gb : g.bufs) { sig += std::string(", const float* ") + (side ? "" : "__restrict__ ") + gb.param; order.push_back(gb.node); }
+        for (auto& gb : g.bufs) { sig += std::string(", const float* ") + gb.param; order.push_back(gb.node); }
         src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
         src += strf("    const unsigned lane = threadIdx.x %% %du;\n", T);
@@ -897,9 +898,9 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         // only a handful of rows to walk and all its loads are in flight together
         const int YG = (bx * chunks < 1024 && CH >= 64) ? 16 : 4;
         k.kind = "reduce_col";
-        std::string sig = "const int* __restrict__ guard, float* __restrict__ out";
+        std::string sig = "const int* __restrict__ guard, float* out";
         std::vector<Node*> order{const_cast<Node*>(n)};
-        for (auto& gb : g.bufs) { sig += ", const float* __restrict__ " + gb.param; order.push_back(gb.node); }
+        for (auto& gb : g.bufs) { sig += ", const float* " + gb.param; order.push_back(gb.node); }
         src += strf("extern \"C\" __global__ __launch_bounds__(%d) void %s(%s) {\n", 64 * YG, k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
         src += strf("    __shared__ float part[%d][64][%d];\n", YG, vec);

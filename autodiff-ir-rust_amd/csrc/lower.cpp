@@ -234,6 +234,11 @@ struct Lowerer {
     }
 
     void transfer_cmd(const Cmd& c, IdSet& live) {
+        auto ru = reuse.find(&c);
+        if (ru != reuse.end()) {
+            if (ru->second != c.res) { live.erase(c.res); add_use(live, ru->second); }
+            return;
+        }
         switch (c.tag) {
         case T_CREATE_MAT: case T_CREATE_CONSTANT: live.erase(c.res); break;
         case T_ELW_MULTIPLY: case T_ELW_ADD: case T_DOT_PRODUCT:
@@ -246,6 +251,132 @@ struct Lowerer {
         default:
             if (!is_control(c.tag)) { live.erase(c.res); add_use(live, c.a); }
         }
+    }
+
+    // -----------------------------------------------------------------------------------
+    // available reductions and products
+    //
+    // A forward analysis over the structured program: after `s = Sum(v)` (or a DotProduct) the fact "s holds
+    // Sum(<v written out down to the ids it views>)" stays true until s or one of those ids is redefined.  Facts are
+    // intersected where paths join and iterated to a fixed point around loops.  A later Sum / DotProduct whose
+    // operands spell the same expression does not run again: its result id is bound to s.  This is what removes the
+    // second pass over the data from a loop whose predicate and body both reduce the same tensor (the predicate's sum
+    // at the end of one iteration is the body's sum at the start of the next).
+    // -----------------------------------------------------------------------------------
+    struct AvEntry {
+        std::string text;             // views: expression over root ids; facts: id that holds the value
+        std::set<std::string> roots;  // ids the expression reads
+        bool operator==(const AvEntry& o) const { return text == o.text && roots == o.roots; }
+    };
+    struct AvState {
+        std::map<std::string, AvEntry> views;  // view id -> what it spells (expanded when the view is made, as aliases are)
+        std::map<std::string, AvEntry> facts;  // expression -> holder
+        bool operator==(const AvState& o) const { return views == o.views && facts == o.facts; }
+    };
+    std::map<const Cmd*, std::string> reuse;  // Sum / DotProduct commands whose value an id already holds
+    bool av_poison = false;
+
+    static AvEntry av_canon(const AvState& st, const std::string& id) {
+        auto it = st.views.find(id);
+        if (it != st.views.end()) return it->second;
+        return AvEntry{"#" + id, {id}};
+    }
+    static void av_define(AvState& st, const std::string& id) {
+        st.views.erase(id);
+        for (auto it = st.facts.begin(); it != st.facts.end();) {
+            if (it->second.text == id || it->second.roots.count(id)) it = st.facts.erase(it);
+            else ++it;
+        }
+    }
+    static AvState av_join(const AvState& a, const AvState& b) {
+        AvState o;
+        for (auto& kv : a.views) { auto it = b.views.find(kv.first); if (it != b.views.end() && it->second == kv.second) o.views.insert(kv); }
+        for (auto& kv : a.facts) { auto it = b.facts.find(kv.first); if (it != b.facts.end() && it->second == kv.second) o.facts.insert(kv); }
+        return o;
+    }
+    void av_cmd(AvState& st, const Cmd& c, bool record) {
+        switch (c.tag) {
+        case T_HEADING: case T_EX: return;
+        case T_CREATE_MAT: case T_CREATE_CONSTANT: av_define(st, c.res); return;
+        case T_VIEW: case T_INDEX: case T_PERMUTE: case T_BROADCAST: case T_CONCAT: {
+            AvEntry a = av_canon(st, c.a);
+            AvEntry e;
+            e.roots = a.roots;
+            e.text = std::string(tag_name(c.tag)) + shape_str(c.dims) + strf("[%lld,%lld](", (long long)c.i0, (long long)c.i1) + a.text;
+            if (c.tag == T_CONCAT) {
+                AvEntry b = av_canon(st, c.b);
+                e.text += "," + b.text;
+                e.roots.insert(b.roots.begin(), b.roots.end());
+            }
+            e.text += ")";
+            if (e.roots.count(c.res)) av_poison = true;  // a view of itself: nothing here reasons about that
+            av_define(st, c.res);
+            st.views[c.res] = e;
+            return;
+        }
+        case T_SUM: case T_DOT_PRODUCT: {
+            AvEntry a = av_canon(st, c.a);
+            std::string key = std::string(tag_name(c.tag)) + "(" + a.text;
+            std::set<std::string> roots = a.roots;
+            if (c.tag == T_DOT_PRODUCT) {
+                AvEntry b = av_canon(st, c.b);
+                key += "|" + b.text;
+                roots.insert(b.roots.begin(), b.roots.end());
+            }
+            key += ")";
+            auto hit = st.facts.find(key);
+            const bool have = hit != st.facts.end();
+            const std::string holder = have ? hit->second.text : std::string();
+            if (record && have) reuse[&c] = holder;
+            if (have && holder == c.res) return;  // the id already holds exactly this
+            av_define(st, c.res);
+            if (have) return;                     // the older holder stays the one later commands are pointed to
+            if (!roots.count(c.res)) st.facts[key] = AvEntry{c.res, roots};
+            return;
+        }
+        case T_WHILE: {
+            AvState head = st;
+            for (int it = 0; it < 64; ++it) {
+                AvState out = head;
+                av_block(out, *c.block, false);
+                AvState next = av_join(head, out);
+                if (next == head) break;
+                head = next;
+                if (it == 63) { head = AvState(); }
+            }
+            AvState out = head;
+            av_block(out, *c.block, record);
+            st = head;
+            return;
+        }
+        case T_IF: {
+            AvState in = st;
+            bool first = true;
+            AvState acc;
+            auto fold = [&](const AvState& o) { acc = first ? o : av_join(acc, o); first = false; };
+            for (auto& arm : c.conds) {
+                AvState a = in;
+                av_block(a, *arm.second, record);
+                fold(a);
+            }
+            if (c.else_block) {
+                AvState a = in;
+                av_block(a, *c.else_block, record);
+                fold(a);
+            } else {
+                fold(in);
+            }
+            st = acc;
+            return;
+        }
+        default:
+            // every other command defines c.res (the in-place forms have res == their first operand)
+            av_define(st, c.res);
+            return;
+        }
+    }
+    void av_block(AvState& st, const Proc& p, bool record) {
+        for (const Cmd& c : p.cmds) av_cmd(st, c, record);
     }
 
     // Returns the live-in set of the block; records the live-out set of every region.
@@ -450,6 +581,17 @@ struct Lowerer {
     }
 
     void build_cmd(const Cmd& c, bool once) {
+        auto ru = reuse.find(&c);
+        if (ru != reuse.end()) {
+            // the value is already held by another id (see "available reductions and products")
+            if (ru->second == c.res) return;
+            Binding& bf = lookup(ru->second);
+            ADHIP_CHECK(bf.kind == Binding::VAL || bf.kind == Binding::HOME, "internal: holder of a reused value is not a tensor");
+            const Shape sh = bf.shape;
+            Node* n = bf.kind == Binding::VAL ? bf.node : get_livein(ru->second);
+            bind_val(c.res, n, sh);
+            return;
+        }
         switch (c.tag) {
         case T_HEADING: return;
         case T_CREATE_MAT: {
@@ -598,6 +740,42 @@ struct Lowerer {
         rows = R;
         cols = V;
         return a.base;
+    }
+
+    // True when, below the reduction `sum` over a [V,R] space, every read of `old` (V values) is the broadcast
+    // (v, r) -> old[v] reached through element-for-element references only.
+    static bool reads_at_kept_coordinate_only(Node* sum, Node* old, int64_t V, int64_t R) {
+        if (numel(old->shape) != V) return false;
+        bool ok = true;
+        std::set<Node*> seen;
+        std::function<bool(Node*)> reaches = [&](Node* n) {
+            bool r = false;
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                if (s == old) r = true;
+                else if (!in_mem(s) && !r) r = reaches(s);
+            });
+            return r;
+        };
+        std::function<void(Node*)> walk = [&](Node* n) {
+            for_each_src(n, [&](Node* s, const Piece& p, const TRef& t) {
+                if (!ok) return;
+                if (s == old) {
+                    const bool row = t.single_full() && t.shape == Shape{V, R} && p.view.st.size() == 1 &&
+                                     p.view.st[0].shape == Shape{V, R} && p.view.st[0].stride == Shape{1, 0} &&
+                                     p.view.st[0].offset == 0;
+                    if (!row) ok = false;
+                    return;
+                }
+                if (in_mem(s)) return;
+                if (!(identity_piece(p, t) && numel(s->shape) == V * R)) {
+                    if (reaches(s)) ok = false;
+                    return;
+                }
+                if (seen.insert(s).second) walk(s);
+            });
+        };
+        walk(sum);
+        return ok;
     }
 
     // in-memory nodes a root reads (through folded nodes); value = every path is an identity view
@@ -1056,7 +1234,16 @@ struct Lowerer {
                             auto it = greads[g2].find(old);
                             if (it == greads[g2].end()) continue;
                             if (g2 > g) direct = false;
-                            if (g2 == g && !(it->second && is_member)) direct = false;
+                            if (g2 == g && !(it->second && is_member)) {
+                                // a reduction may still update its result in place when it reads the old result only
+                                // at the position it is about to write (s = Sum(f(x, s broadcast along the reduced
+                                // dim))): the block that owns an output element loads before it stores, and a
+                                // chunked reduction stores in its second pass
+                                const bool own_sum = groups[g].kind == Group::SUM && m == groups[g].members[0] && m->op == Op::SUM &&
+                                                     m->in[0].shape.size() == 2 &&
+                                                     reads_at_kept_coordinate_only(m, old, m->in[0].shape[0], m->in[0].shape[1]);
+                                if (!own_sum) direct = false;
+                            }
                         }
                     }
                     int hb = home(id, numel(m->shape));
@@ -1437,6 +1624,11 @@ struct Lowerer {
 
     std::unique_ptr<Plan> run() {
         collect_alias_srcs(prog);
+        if (opt.fuse) {
+            AvState st;
+            av_block(st, prog, true);
+            if (av_poison) reuse.clear();
+        }
         IdSet end_live;
         for (auto& d : deps) end_live.insert(d);
         const IdSet start_live = live_block(prog, end_live);
