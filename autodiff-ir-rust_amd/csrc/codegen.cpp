@@ -133,6 +133,7 @@ struct Gen {
     std::map<const Node*, int> buf_index;
     std::vector<GenBuffer> bufs;
     std::set<const Node*> members;  // computed in this kernel, never loaded
+    std::map<const Node*, std::string> preset;  // nodes whose value is a variable the kernel already holds
     std::vector<LoadRec> loads;
     std::vector<Aff> recorded;  // every index expression over base atoms, for dim merging
     int tmp = 0;
@@ -431,6 +432,10 @@ struct Gen {
     bool in_memory(const Node* n) const { return (op_is_leaf(n->op) || n->root) && !members.count(n); }
 
     Val gen_node(const Node* n, const Aff& l, const std::string& pred) {
+        {
+            auto ps = preset.find(n);
+            if (ps != preset.end()) return {ps->second, false};
+        }
         if (in_memory(n)) return load(n, l, pred);
         if (n->op == Op::FILL) return {flit(n->cval), false};
         ADHIP_CHECK(op_is_elw(n->op), "internal: node %d (%s) is neither in memory nor element-wise", n->id, op_name(n->op));
@@ -825,12 +830,39 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         }
         const int64_t CH = (RV + chunks - 1) / chunks;  // vector elements per chunk
         k.kind = side ? "reduce_row_store" : "reduce_row";
+        // Epilogue: element-wise consumers of the finished sums, evaluated at index x by the lane that stores the sum.
+        // Generated with the same buffer table; its statements are taken out of the loop body's lists, and nothing
+        // memoised inside the loop is visible to it.
+        std::vector<std::string> epi_code, epi_exprs;
+        const bool epi = !spec.epilogue_outputs.empty() && chunks == 1;
+        if (epi) {
+            auto memo = g.val_memo;
+            g.val_memo.clear();
+            const int vec_saved = g.vec, lane_saved = g.lane_atom;
+            g.vec = 1;
+            g.lane_atom = -1;
+            const size_t a0 = g.codeA.size(), b0 = g.codeB.size();
+            const double flops_saved = g.flops;
+            g.preset[n] = "sum_value";
+            for (Node* e : spec.epilogue_outputs) g.members.insert(e);
+            const Aff at_x = aff_atom(0, 1);  // atom 0 is x
+            for (Node* e : spec.epilogue_outputs) epi_exprs.push_back(g.gen_node(e, at_x, "").expr);
+            ADHIP_CHECK(g.codeB.size() == b0, "internal: reduction epilogue produced per-lane code");
+            epi_code.assign(g.codeA.begin() + (long)a0, g.codeA.end());
+            g.codeA.resize(a0);
+            g.flops = flops_saved;
+            g.vec = vec_saved;
+            g.lane_atom = lane_saved;
+            g.val_memo = memo;
+            k.epilogue_done = true;
+        }
         // no __restrict__: the result (and a stored operand) may share a buffer with an input it replaces in place
         std::string sig = "const int* __restrict__ guard, float* out";
         std::vector<Node*> order{const_cast<Node*>(n)};
         if (side)
             for (size_t i = 0; i < spec.side_outputs.size(); ++i) { sig += strf(", float* w%zu", i); order.push_back(spec.side_outputs[i]); }
-        // a stored value may update one of the inputs in place, so nothing is restrict-qualified then
+        if (epi)
+            for (size_t i = 0; i < spec.epilogue_outputs.size(); ++i) { sig += strf(", float* e%zu", i); order.push_back(spec.epilogue_outputs[i]); }
         for (auto& gb : g.bufs) { sig += std::string(", const float* ") + gb.param; order.push_back(gb.node); }
         src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
@@ -861,13 +893,22 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += "    }\n";
         if (vec == 4) src += "    float s = (acc[0] + acc[1]) + (acc[2] + acc[3]);\n";
         else src += "    float s = acc[0];\n";
+        std::string epilogue;
+        if (epi) {
+            epilogue = join(epi_code, "        ");
+            for (size_t i = 0; i < epi_exprs.size(); ++i) epilogue += strf("        e%zu[x] = %s;\n", i, epi_exprs[i].c_str());
+        }
         if (T == 64) {
             src += "    s = wave_sum(s);\n";
-            src += strf("    if (lane == 0 && row_ok) out[(%s)chunk * %lldu + x] = s;\n", g.idx_t(), (long long)V);
+            src += "    if (lane == 0 && row_ok) {\n        const float sum_value = s;\n";
+            src += strf("        out[(%s)chunk * %lldu + x] = sum_value;\n", g.idx_t(), (long long)V);
+            src += epilogue + "    }\n";
         } else {
             src += "    __shared__ float part[4];\n    s = wave_sum(s);\n";
             src += "    if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = s;\n    __syncthreads();\n";
-            src += strf("    if (threadIdx.x == 0 && row_ok) out[(%s)chunk * %lldu + x] = (part[0] + part[1]) + (part[2] + part[3]);\n", g.idx_t(), (long long)V);
+            src += "    if (threadIdx.x == 0 && row_ok) {\n        const float sum_value = (part[0] + part[1]) + (part[2] + part[3]);\n";
+            src += strf("        out[(%s)chunk * %lldu + x] = sum_value;\n", g.idx_t(), (long long)V);
+            src += epilogue + "    }\n";
         }
         src += "}\n";
         k.buffer_args = order;

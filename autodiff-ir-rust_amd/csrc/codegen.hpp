@@ -41,6 +41,10 @@ struct ReduceKernelSpec {
     // Element-wise values with V*R elements that this kernel also stores (row layout only): the
     // reduction's own operand chain is evaluated once, stored and summed in the same pass.
     std::vector<Node*> side_outputs;
+    // Element-wise values with V elements that follow the reduction (they read its result element for element):
+    // the lane that holds a finished sum also evaluates and stores them, so no further kernel is needed.  Done only
+    // in the row layout when one pass finishes the sum; `GeneratedKernel::epilogue_done` tells.
+    std::vector<Node*> epilogue_outputs;
 };
 
 struct GeneratedKernel {
@@ -56,6 +60,7 @@ struct GeneratedKernel {
     // (for element-wise kernels with column sums: the number of row tiles)
     int64_t chunks = 1;
     bool side_done = false;  // the reduction stored its side outputs
+    bool epilogue_done = false;  // the reduction evaluated and stored its epilogue outputs
 };
 
 // `in_memory(n)` tells whether node n's value can be loaded from a buffer in this kernel.

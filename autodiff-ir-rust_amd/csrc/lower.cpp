@@ -180,6 +180,8 @@ struct Group {
     int64_t cs_rows = 0, cs_cols = 0;
     // element-wise values a row reduction stores while it sums them
     std::vector<Node*> side;
+    // element-wise values of the result's size that the reduction evaluates and stores right after summing
+    std::vector<Node*> epi;
     bool dead = false;  // its only member was absorbed by another group
 };
 
@@ -1183,8 +1185,43 @@ struct Lowerer {
                 spec.node = G.members[0];
                 spec.name = name;
                 spec.side_outputs = G.side;
+                // the element-wise group scheduled right after this reduction, if all it needs from it is the result
+                // element for element, becomes the reduction's epilogue (the reference's Reduce + ELW fusion,
+                // src/kernel/fusion/reduce_elw.rs:12-143)
+                int ge = -1;
+                if (opt.fuse) {
+                    Node* S = G.members[0];
+                    size_t nx = g + 1;
+                    while (nx < groups.size() && groups[nx].dead) ++nx;
+                    if (nx < groups.size() && groups[nx].kind == Group::ELW && groups[nx].colsums.empty() &&
+                        groups[nx].n == numel(S->shape)) {
+                        bool uses = false, ok = true;
+                        for (Node* m : groups[nx].members) {
+                            auto it = reads[m].find(S);
+                            if (it == reads[m].end()) continue;
+                            uses = true;
+                            ok = ok && it->second;
+                        }
+                        if (uses && ok) { ge = (int)nx; spec.epilogue_outputs = groups[nx].members; }
+                    }
+                }
                 gks[g].k = gen_reduce_kernel(spec);
                 ADHIP_CHECK(G.side.empty() || gks[g].k.side_done, "internal: row reduction did not take over its operand's store");
+                if (ge >= 0 && gks[g].k.epilogue_done) {
+                    G.epi = groups[ge].members;
+                    groups[ge].dead = true;
+                    std::set<Node*> own(G.epi.begin(), G.epi.end());
+                    own.insert(G.members[0]);
+                    for (Node* m : G.epi) {
+                        group_of[m] = (int)g;
+                        for (auto& rd : reads[m]) {
+                            if (own.count(rd.first)) continue;
+                            auto it = greads[g].find(rd.first);
+                            if (it == greads[g].end()) greads[g][rd.first] = rd.second;
+                            else it->second = it->second && rd.second;
+                        }
+                    }
+                }
                 if (gks[g].k.chunks > 1) {
                     // second pass over the partial sums [chunks][V]
                     Node* n = G.members[0];
@@ -1217,6 +1254,7 @@ struct Lowerer {
             std::vector<Node*> produced = groups[g].members;
             for (auto& cs : groups[g].colsums) produced.push_back(cs.second);
             for (Node* sd : groups[g].side) produced.push_back(sd);
+            for (Node* ep : groups[g].epi) produced.push_back(ep);
             for (Node* m : produced) {
                 auto ho = home_of.find(m);
                 bool direct = false;
@@ -1226,7 +1264,8 @@ struct Lowerer {
                     auto li = livein.find(id);
                     if (li != livein.end()) {
                         Node* old = li->second;
-                        const bool is_side = std::find(groups[g].side.begin(), groups[g].side.end(), m) != groups[g].side.end();
+                        const bool is_side = std::find(groups[g].side.begin(), groups[g].side.end(), m) != groups[g].side.end() ||
+                                             std::find(groups[g].epi.begin(), groups[g].epi.end(), m) != groups[g].epi.end();
                         const bool is_member = is_side || (groups[g].kind == Group::ELW &&
                             std::find(groups[g].members.begin(), groups[g].members.end(), m) != groups[g].members.end());
                         for (size_t g2 = 0; g2 < groups.size(); ++g2) {

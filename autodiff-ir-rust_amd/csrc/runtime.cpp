@@ -515,7 +515,10 @@ void program_run(adhip_program* p) {
 void program_readback(adhip_program* p) {
     adhip_ctx* ctx = p->ctx;
     HIP_OK(hipSetDevice(ctx->device));
-    ctx->results.clear();
+    // host buffers of the previous read-back are reused where an id comes back again: fresh pages of a large
+    // result cost more than the copy itself
+    std::map<std::string, HostResult> previous;
+    previous.swap(ctx->results);
     struct Staged { HostResult* r; size_t off, nb; };
     std::vector<Staged> staged;
     size_t used = 0;
@@ -527,6 +530,8 @@ void program_readback(adhip_program* p) {
     };
     for (auto& kv : p->plan->results) {
         HostResult& r = ctx->results[kv.first];
+        auto prev = previous.find(kv.first);
+        if (prev != previous.end()) r.data = std::move(prev->second.data);
         for (auto d : kv.second.shape) r.dims.push_back((uint64_t)d);
         const int64_t ne = numel(kv.second.shape);
         r.data.resize((size_t)ne);
@@ -606,7 +611,13 @@ const char* adhip_last_error(adhip_ctx* ctx) { return ctx ? ctx->last_error.c_st
 int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, const char* const* dep_ids, size_t n_dep_ids) {
     if (!ctx) return 2;
     return guarded(ctx, [&] {
-        ctx->results.clear();
+        // results of an earlier call stay in place until the read-back replaces them (it reuses their host
+        // buffers); a call that fails leaves none visible
+        struct ClearOnFailure {
+            adhip_ctx* c;
+            bool ok = false;
+            ~ClearOnFailure() { if (!ok) c->results.clear(); }
+        } results_guard{ctx};
         const char* cenv = getenv("ADHIP_EXEC_CACHE");
         const bool caching = !(cenv && *cenv == '0');
         adhip_program* p = nullptr;
@@ -688,6 +699,7 @@ int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, co
             throw;
         }
         if (!keep) program_free(p);
+        results_guard.ok = true;
     });
 }
 
