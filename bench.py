@@ -22,7 +22,7 @@ for p in (ROOT, os.path.join(ROOT, "autodiff-ir-rust_amd")):
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # HBM bytes per launch of the fused forward+backward kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
 # plain copy kernel (profiles/fused_elw_8192x8192.hbm_traffic_pmc.txt).  Valid for the 8192x8192 workload only.
-FUSED_ELW_TRAFFIC_BYTES = 805784371 + 1082130944
+FUSED_ELW_TRAFFIC_BYTES = 805459399 + 1082131484
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 
 

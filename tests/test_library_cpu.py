@@ -192,3 +192,37 @@ def test_random_control_flow_programs_lower(seed):
     if seed < 3:
         rc, msg = _compile_check(proc, set(keep))
         assert rc == 0, msg
+
+
+def _loop_body(text):
+    """Launch lines inside the first while-block of a plan description."""
+    lines = text.splitlines()
+    start = next(i for i, l in enumerate(lines) if l.startswith("while "))
+    end = next(i for i in range(start, len(lines)) if lines[i] == "}")
+    return [l.strip() for l in lines[start + 1:end] if l.strip().startswith("launch")]
+
+
+def test_loop_reuses_the_sum_its_predicate_computed():
+    """`while not (r.sum(1) < 1).all(): r -= 0.01 * r.sum(1)[:, None]`: the row sums that the predicate needs at the
+    end of one iteration are the ones the body needs at the start of the next, so an iteration has one pass over r
+    (update + store + row sums, updating the sums in place) and one small kernel (the all() count with the predicate
+    arithmetic as its epilogue)."""
+    dev = Capture()
+    wl = W.manip_loop(dev)   # full size: the plan depends on the shapes
+    proc, deps = wl.finish()
+    body = _loop_body(lower_describe(proc, deps))
+    assert len(body) == 2, body
+    assert "[reduce_row_store]" in body[0] and "[reduce_row]" in body[1], body
+    assert not any("commit_" in l for l in body)
+
+
+def test_reduction_epilogue_is_fused():
+    """s = Sum(x) followed by element-wise work on s (y = 2*s + b; b += s) is one kernel."""
+    import numpy as np
+    x = IR.CreateMat(np.zeros(300 * 64, np.float32), [300, 64], "x")
+    b = IR.CreateMat(np.zeros(300, np.float32), [300], "b")
+    cmds = [x, b, IR.Sum(a="x", res="s"), IR.CreateConstant(2.0, "two", [300]), IR.ElwMultiply(a="s", b="two", res="t"),
+            IR.ElwAdd(a="t", b="b", res="y"), IR.ElwAddEq(s="b", o="s"), IR.EX()]
+    text = lower_describe(IR.IRProcedure("main", cmds), {"y", "b", "s"})
+    launches = [l for l in text.splitlines() if l.startswith("launch")]
+    assert len(launches) == 1 and "[reduce_row]" in launches[0], text

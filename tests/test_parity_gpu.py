@@ -378,3 +378,26 @@ def test_random_control_flow_matches_oracle(seed, hip_device):
             assert_exact(got.data, ref[k].data, k)
         else:
             assert_close(got.data, ref[k].data, 2e-5, k, scale=max(1.0, float(np.max(np.abs(ref[k].data)))))
+
+
+@pytest.mark.parametrize("V,R", [(300, 64), (1, 5000), (7, 3), (2048, 1024), (5, 40000), (70000, 8)])
+def test_reduction_epilogue_values(V, R, hip_device):
+    """Row sums followed by element-wise consumers of the sums (one of them an in-place update of its own operand):
+    wave-per-row, block-per-row and chunked shapes, so both the fused epilogue and the unfused fallback are covered."""
+    print(f"[case] reduction epilogue V={V} R={R}", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(V * 131 + R)
+    x = rng.standard_normal(V * R).astype(np.float32)
+    b = rng.standard_normal(V).astype(np.float32)
+    cmds = [IR.CreateMat(x, [V, R], "x"), IR.CreateMat(b, [V], "b"), IR.Sum(a="x", res="s"),
+            IR.CreateConstant(2.0, "two", [V]), IR.ElwMultiply(a="s", b="two", res="t"), IR.ElwAdd(a="t", b="b", res="y"),
+            IR.Sin(a="y", res="z"), IR.ElwAddEq(s="b", o="s")]
+    got = _run_ir(hip_device, cmds, ["s", "y", "z", "b"])
+    s = x.reshape(V, R).astype(np.float64).sum(1)
+    tol = RED_RTOL * math.sqrt(R)
+    scale = float(np.abs(x.reshape(V, R)).sum(1).max())
+    assert_close(got["s"].data, s, tol, "s", scale=scale)
+    assert_close(got["y"].data, 2 * s + b, tol, "y", scale=2 * scale)
+    assert_close(got["b"].data, b + s, tol, "b", scale=scale)
+    # z against the device's own y: the sine of a float32 argument
+    assert_close(got["z"].data, np.sin(got["y"].data.astype(np.float64)), ELW_RTOL, "z", scale=1.0)
