@@ -114,3 +114,38 @@ def test_manip_loop_runs_to_the_iteration_limit(hip_device):
     assert out["i"].data[0] == 50.0
     got = out["r"].numpy()
     assert not np.isfinite(got).all()
+
+
+def test_tensor_beyond_32_bit_indices(hip_device):
+    """A tensor of 2^31 + 4096 elements (8.6 GB): element-wise, gather, row-reduction and column-reduction kernels
+    must switch to 64-bit index arithmetic.  y[i, j] = i + j/4096 is built from two broadcasts, materialised, and
+    checked through its last row (bit-exact), its row sums and its column sums (closed forms)."""
+    print("[case] 2^31 + 4096 elements", flush=True)
+    from adhip import ir as IR
+    R, C = (1 << 19) + 1, 4096
+    v = (np.arange(C, dtype=np.float32) / np.float32(C)).astype(np.float32)
+    r = np.arange(R, dtype=np.float32)
+    cmds = [
+        IR.CreateMat(v, [C], "v"), IR.View(a="v", target_dim=[1, C], res="v1"), IR.Broadcast(a="v1", dim=0, r=R, res="vb"),
+        IR.CreateMat(r, [R], "r"), IR.View(a="r", target_dim=[R, 1], res="r1"), IR.Broadcast(a="r1", dim=1, r=C, res="rb"),
+        IR.ElwAdd(a="vb", b="rb", res="y0"), IR.Contigious(a="y0", res="y"),
+        IR.Index(a="y", index=R - 1, dim=0, res="last_v"), IR.Contigious(a="last_v", res="last"),
+        IR.Sum(a="y", res="rows"),
+        IR.Permute(a="y", p=[1, 0], res="yt"), IR.Sum(a="yt", res="cols"),
+        IR.EX(),
+    ]
+    hip_device.execute(IR.IRProcedure("main", cmds), {"last", "rows", "cols"})
+    last = hip_device.get_tensor("last")
+    rows = hip_device.get_tensor("rows")
+    cols = hip_device.get_tensor("cols")
+    assert last.dim == [C] and rows.dim == [R] and cols.dim == [C]
+    assert_exact(last.data, v + np.float32(R - 1), "last row")
+    # row i: sum_j fl(i + j/4096); the addends are exact multiples of 2^-12 below 2^19 + 1, rounded to 24 bits
+    idx = np.array([0, 1, 1000, 65536, 300000, R - 2, R - 1])
+    exp_rows = np.array([(v + np.float32(i)).astype(np.float64).sum() for i in idx])
+    assert_close(rows.data[idx], exp_rows, RED_RTOL * math.sqrt(C), "row sums")
+    exp_all_rows = r.astype(np.float64) * C + float(v.astype(np.float64).sum())
+    assert_close(rows.data, exp_all_rows, 1e-4, "all row sums (fl(i + j/4096) rounds at 2^-5 for large i)")
+    jdx = np.array([0, 1, 2047, 4095])
+    exp_cols = np.array([(r + v[j]).astype(np.float64).sum() for j in jdx])
+    assert_close(cols.data[jdx], exp_cols, RED_RTOL * math.sqrt(R), "column sums")
