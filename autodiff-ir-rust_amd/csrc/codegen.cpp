@@ -732,6 +732,39 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
     return k;
 }
 
+DotEpilogueCode gen_dot_epilogue(const Node* dot, const std::vector<Node*>& outputs) {
+    ADHIP_CHECK(dot->op == Op::DOT && dot->shape.size() == 2, "internal: malformed product for an epilogue");
+    const int64_t M = dot->shape[0], N = dot->shape[1];
+    Gen g;
+    g.vec = 1;
+    std::vector<Node*> all(outputs.begin(), outputs.end());
+    g.wide = needs_wide(all) || M * N >= (int64_t(1) << 31) - 1024;
+    const int ar = g.add_atom("er", M, false), ac = g.add_atom("ec", N, false);
+    const Aff lin = aff_add(aff_atom(ar, N), aff_atom(ac, 1));
+    g.preset[dot] = "sum_value";
+    for (Node* o : outputs) {
+        ADHIP_CHECK(numel(o->shape) == M * N && op_is_elw(o->op), "internal: product epilogue output of the wrong kind");
+        g.members.insert(o);
+    }
+    std::vector<std::string> exprs;
+    for (Node* o : outputs) exprs.push_back(g.gen_node(o, lin, "").expr);
+    ADHIP_CHECK(g.codeB.empty(), "internal: product epilogue produced per-lane code");
+    DotEpilogueCode e;
+    e.code = strf("const %s er = (%s)row, ec = (%s)col;\n", g.idx_t(), g.idx_t(), g.idx_t());
+    e.code += join(g.codeA, "");
+    for (size_t i = 0; i < outputs.size(); ++i) {
+        e.code += strf("e%zu[er * %lld%s + ec] = %s;\n", i, (long long)N, g.wide ? "ull" : "u", exprs[i].c_str());
+        e.params += strf(", float* e%zu", i);
+        e.buffer_args.push_back(outputs[i]);
+    }
+    for (auto& gb : g.bufs) {
+        e.params += ", const float* " + gb.param;
+        e.buffer_args.push_back(gb.node);
+    }
+    e.flops = g.flops;
+    return e;
+}
+
 // ---------------------------------------------------------------------------------------
 // reductions
 // ---------------------------------------------------------------------------------------

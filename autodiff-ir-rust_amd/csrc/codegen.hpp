@@ -80,6 +80,16 @@ struct Affine2D {
 };
 bool tref_affine2d(const TRef& t, Affine2D& out);
 
+// Element-wise values with M*N elements that follow a matrix product `dot` ([M,N]) and read it element for element:
+// statements for the product kernel's store loop (they use `row`, `col`, `sum_value`), the extra parameters, and the
+// buffers behind them in parameter order (outputs first).
+struct DotEpilogueCode {
+    std::string params, code;
+    std::vector<Node*> buffer_args;
+    double flops = 0;  // per output element
+};
+DotEpilogueCode gen_dot_epilogue(const Node* dot, const std::vector<Node*>& outputs);
+
 const char* kernel_prelude();
 
 }  // namespace adhip

@@ -12,8 +12,24 @@
 
 namespace adhip {
 
-std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry) {
+std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry, const GemmEpilogue* epilogue) {
     std::string s;
+    if (epilogue) s += epilogue->prelude;
+    s += strf("#define STORE_C %d\n#define EPI_PARAMS %s\n", (!epilogue || epilogue->store_c) ? 1 : 0,
+              epilogue ? epilogue->params.c_str() : "");
+    {
+        // the epilogue statements become one macro (line continuations), expanded where an element is finished
+        std::string body = epilogue ? epilogue->code : std::string();
+        std::string m = "#define EPILOGUE";
+        size_t pos = 0;
+        while (pos < body.size()) {
+            size_t nl = body.find('\n', pos);
+            if (nl == std::string::npos) nl = body.size();
+            m += " \\\n    " + body.substr(pos, nl - pos);
+            pos = nl + 1;
+        }
+        s += m + "\n";
+    }
     s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n", cfg.a_kcontig ? 1 : 0, cfg.b_kcontig ? 1 : 0,
               cfg.edge ? 1 : 0);
     s += strf("#define KERNEL_NAME %s\n#define BM %d\n", entry.c_str(), cfg.bm);
@@ -34,7 +50,7 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     const int* __restrict__ guard, float* __restrict__ C, const float* __restrict__ A, const float* __restrict__ B,
     long long M, long long N, long long K, long long a_off, long long a_sm, long long a_sk, long long b_off,
-    long long b_sk, long long b_sn) {
+    long long b_sk, long long b_sn EPI_PARAMS) {
     if (guard && *guard == 0) return;
     __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDB];
@@ -224,7 +240,13 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
 #if EDGE
                     if (row < M && col < N)
 #endif
-                        C[row * N + col] = acc[i][j][4 * g + r];
+                    {
+                        const float sum_value = acc[i][j][4 * g + r];
+#if STORE_C
+                        C[row * N + col] = sum_value;
+#endif
+                        EPILOGUE
+                    }
                 }
 }
 )";

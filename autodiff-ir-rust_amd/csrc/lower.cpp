@@ -199,6 +199,7 @@ struct Lowerer {
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
     int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1;
+    int dot_epilogue_counter = 0;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
 
     // per region
@@ -1139,7 +1140,13 @@ struct Lowerer {
         // ---- 6. generate code per group (no buffers needed yet)
         std::map<Node*, std::string> home_of_early;
         for (auto& w : wanted) home_of_early[w.second] = w.first;
-        struct GK { GeneratedKernel k; std::vector<GeneratedKernel> extra; std::vector<Node*> extra_nodes; };
+        struct GK {
+            GeneratedKernel k;
+            std::vector<GeneratedKernel> extra;
+            std::vector<Node*> extra_nodes;
+            DotEpilogueCode dot_epi;   // DOT groups with an epilogue
+            bool dot_store = true;     // ... and whether the product itself is still written
+        };
         std::vector<GK> gks(groups.size());
         // reads per group, with "identity only" flags, for hazard analysis
         std::vector<std::map<Node*, bool>> greads(groups.size());
@@ -1180,6 +1187,57 @@ struct Lowerer {
                     gks[g].extra_nodes.push_back(fin);
                 }
                 gks[g].k = gen_elw_kernel(spec, members);
+            } else if (G.kind == Group::DOT) {
+                // the element-wise group scheduled right after a matrix-core product, if all it needs from the
+                // product is the result element for element, runs on the accumulators before they are stored (the
+                // reference's DotProd + ELW fusion, src/kernel/fusion/dp_elw.rs:13-149); the product itself is
+                // written only if something else still reads it
+                Node* D = G.members[0];
+                size_t nx = g + 1;
+                while (nx < groups.size() && groups[nx].dead) ++nx;
+                if (opt.fuse && dot_uses_mfma(D) && nx < groups.size() && groups[nx].kind == Group::ELW &&
+                    groups[nx].colsums.empty() && groups[nx].n == numel(D->shape)) {
+                    bool uses = false, ok = true;
+                    for (Node* m : groups[nx].members) {
+                        auto it = reads[m].find(D);
+                        if (it == reads[m].end()) continue;
+                        uses = true;
+                        ok = ok && it->second;
+                    }
+                    if (uses && ok) {
+                        gks[g].dot_epi = gen_dot_epilogue(D, groups[nx].members);
+                        G.epi = groups[nx].members;
+                        groups[nx].dead = true;
+                        std::set<Node*> own(G.epi.begin(), G.epi.end());
+                        own.insert(D);
+                        for (Node* m : G.epi) {
+                            group_of[m] = (int)g;
+                            for (auto& rd : reads[m]) {
+                                if (own.count(rd.first)) continue;
+                                auto it = greads[g].find(rd.first);
+                                if (it == greads[g].end()) greads[g][rd.first] = rd.second;
+                                else it->second = it->second && rd.second;
+                            }
+                        }
+                        // is the product itself still needed in memory?
+                        bool needed = home_of_early.count(D) != 0;
+                        for (size_t g2 = 0; g2 < groups.size() && !needed; ++g2) {
+                            if (groups[g2].dead || g2 == g) continue;
+                            std::vector<Node*> rs = groups[g2].members;
+                            for (Node* sd : groups[g2].side) rs.push_back(sd);
+                            for (Node* ep : groups[g2].epi) rs.push_back(ep);
+                            for (Node* m : rs)
+                                if (reads[m].count(D)) needed = true;
+                            for (auto& cs : groups[g2].colsums) {
+                                std::map<Node*, bool> er;
+                                if (in_mem(cs.first)) er[cs.first] = true;
+                                else collect_reads(cs.first, er);
+                                if (er.count(D)) needed = true;
+                            }
+                        }
+                        gks[g].dot_store = needed;
+                    }
+                }
             } else if (G.kind == Group::SUM) {
                 ReduceKernelSpec spec;
                 spec.node = G.members[0];
@@ -1255,6 +1313,7 @@ struct Lowerer {
             for (auto& cs : groups[g].colsums) produced.push_back(cs.second);
             for (Node* sd : groups[g].side) produced.push_back(sd);
             for (Node* ep : groups[g].epi) produced.push_back(ep);
+            if (groups[g].kind == Group::DOT && !gks[g].dot_store) produced.erase(produced.begin());  // lives in registers only
             for (Node* m : produced) {
                 auto ho = home_of.find(m);
                 bool direct = false;
@@ -1331,7 +1390,8 @@ struct Lowerer {
             Group& G = groups[g];
             if (G.dead) continue;
             if (G.kind == Group::DOT) {
-                emit_dot(G.members[0], out);
+                if (!G.epi.empty()) emit_dot(G.members[0], out, &gks[g].dot_epi, gks[g].dot_store);
+                else emit_dot(G.members[0], out);
                 continue;
             }
             if (G.kind == Group::TRANSPOSE) {
@@ -1443,13 +1503,23 @@ struct Lowerer {
         push_launch(out, l, "transpose");
     }
 
-    void emit_dot(Node* n, std::vector<Step>& out) {
+    // whether a product goes to the matrix-core kernel (else the one-thread-per-output kernel)
+    static bool dot_uses_mfma(const Node* n) {
+        Affine2D a, b;
+        if (!tref_affine2d(n->in[0], a) || !tref_affine2d(n->in[1], b)) return false;
+        const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
+        const bool a_unit = a.s1 == 1 || a.s0 == 1, b_unit = b.s0 == 1 || b.s1 == 1;
+        return M * N * K >= 64 * 64 * 64 && a_unit && b_unit;
+    }
+
+    void emit_dot(Node* n, std::vector<Step>& out, const DotEpilogueCode* epi = nullptr, bool store_c = true) {
         Affine2D a, b;
         ADHIP_CHECK(tref_affine2d(n->in[0], a) && tref_affine2d(n->in[1], b), "internal: matmul operand is not a strided view");
         const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
         auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: matmul operand without buffer"); q.buf = x->buffer; return q; };
         auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
         const bool a_unit = a.s1 == 1 || a.s0 == 1, b_unit = b.s0 == 1 || b.s1 == 1;
+        ADHIP_CHECK(!epi || dot_uses_mfma(n), "internal: product epilogue on the small-product kernel");
         if (M * N * K >= 64 * 64 * 64 && a_unit && b_unit) {
             // matrix-core kernel; operands keep their strides (x^T, W^T are never copied)
             GemmConfig cfg;
@@ -1461,13 +1531,34 @@ struct Lowerer {
             cfg.bm = (!cfg.edge && M % 256 == 0 && (M / 256) * (N / 128) >= 512) ? 256 : 128;
             std::string entry = strf("adhip_gemm_%c%c_%d%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm, cfg.edge ? "_edge" : "");
             Launch l;
-            l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
+            if (epi) {
+                // the element-wise group that followed the product runs on the accumulators; every distinct
+                // epilogue is its own kernel
+                entry += strf("_e%d", dot_epilogue_counter++);
+                GemmEpilogue ge;
+                ge.prelude = kernel_prelude();
+                ge.params = epi->params;
+                ge.code = epi->code;
+                ge.store_c = store_c;
+                l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry, &ge), "dot_mfma");
+            } else {
+                l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
+            }
             l.block[0] = (unsigned)(cfg.bm * 2);
             l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + 127) / 128));
-            l.args = {B(n), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
+            // a product that is not stored has no buffer; the kernel never touches C then
+            Node* c_arg = store_c ? n : (epi ? epi->buffer_args[0] : n);
+            l.args = {B(c_arg), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
             l.label = strf("dot_%s_%lldx%lldx%lld", n->name.c_str(), (long long)M, (long long)N, (long long)K);
-            l.bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
+            l.bytes = 4.0 * ((double)M * K + (double)K * N + (store_c ? (double)M * N : 0.0));
             l.flops = 2.0 * (double)M * (double)N * (double)K;
+            if (epi) {
+                for (Node* x : epi->buffer_args) {
+                    l.args.push_back(B(x));
+                    l.bytes += 4.0 * (double)std::min<int64_t>(numel(x->shape), M * N);
+                }
+                l.flops += epi->flops * (double)M * (double)N;
+            }
             push_launch(out, l, "dot_mfma");
             return;
         }

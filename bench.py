@@ -74,6 +74,28 @@ def cpu_baseline_fused_elw(rows, cols):
             f"{dt:.2f} s wall", "seconds": dt}
 
 
+def measure_mlp(dev, iters):
+    """BASELINE.json configs[3]: `iters` training steps inside one resident program run."""
+    from adhip import workloads as W
+    wl4 = W.mlp_train(dev, 4096, (4096, 4096, 4096, 1024), iters, seed=0)
+    p4 = compile_resident(dev, wl4)
+    p4.run()      # warm-up: compiles nothing new, touches every buffer once
+    p4.upload()   # a run consumes the loop counter; restore the initial state (not timed)
+    t0 = time.perf_counter()
+    p4.run()
+    dt4 = time.perf_counter() - t0
+    k4 = profile_once(p4)
+    for k in k4:
+        k["launches_per_run"] = k.pop("launches")
+    dot_ms = sum(k["avg_ms"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
+    dot_fl = sum(k["flops"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
+    p4.close()
+    return {"steps_per_s": iters / dt4, "ms_per_train_step": dt4 * 1e3 / iters,
+            "matmul_TFLOPs": dot_fl / (dot_ms * 1e-3) / 1e12 if dot_ms else None,
+            "matmul_frac_of_fp32_mfma_peak": dot_fl / (dot_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS if dot_ms else None,
+            "flops_per_train_step": wl4.flops / iters}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -111,13 +133,7 @@ def main():
                           "kernels": profile(pc, 3)}))
         return
     if args.workload == "mlp":
-        wl4 = W.mlp_train(dev, 4096, (4096, 4096, 4096, 1024), args.mlp_iters, seed=0)
-        p4 = compile_resident(dev, wl4)
-        t0 = time.perf_counter()
-        p4.run()
-        dt4 = time.perf_counter() - t0
-        print(json.dumps({"metric": "fp32 MLP train steps/s", "value": args.mlp_iters / dt4, "unit": "steps/s",
-                          "ms_per_train_step": dt4 * 1e3 / args.mlp_iters}))
+        print(json.dumps(dict(measure_mlp(dev, args.mlp_iters), metric="fp32 MLP train steps/s")))
         return
     wl = W.fused_elw(dev, rows, cols, seed=0)
     prog = compile_resident(dev, wl)
@@ -172,23 +188,7 @@ def main():
         extra["manip_loop"] = {"ms_total": ms5, "kernels": profile_once(p5)}
         p5.close()
         # config 4: dense MLP training
-        wl4 = W.mlp_train(dev, 4096, (4096, 4096, 4096, 1024), args.mlp_iters, seed=0)
-        p4 = compile_resident(dev, wl4)
-        p4.run()      # warm-up: compiles nothing new, touches every buffer once
-        p4.upload()   # a run consumes the loop counter; restore the initial state (not timed)
-        t0 = time.perf_counter()
-        p4.run()
-        dt4 = time.perf_counter() - t0
-        k4 = profile_once(p4)
-        for k in k4:
-            k["launches_per_run"] = k.pop("launches")
-        dot_ms = sum(k["avg_ms"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
-        dot_fl = sum(k["flops"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
-        extra["mlp_train"] = {"steps_per_s": args.mlp_iters / dt4, "ms_per_train_step": dt4 * 1e3 / args.mlp_iters,
-                              "matmul_TFLOPs": dot_fl / (dot_ms * 1e-3) / 1e12 if dot_ms else None,
-                              "matmul_frac_of_fp32_mfma_peak": dot_fl / (dot_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS if dot_ms else None,
-                              "flops_per_train_step": wl4.flops / args.mlp_iters}
-        p4.close()
+        extra["mlp_train"] = measure_mlp(dev, args.mlp_iters)
 
     cpu = None
     if not args.skip_cpu:

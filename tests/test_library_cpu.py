@@ -226,3 +226,17 @@ def test_reduction_epilogue_is_fused():
     text = lower_describe(IR.IRProcedure("main", cmds), {"y", "b", "s"})
     launches = [l for l in text.splitlines() if l.startswith("launch")]
     assert len(launches) == 1 and "[reduce_row]" in launches[0], text
+
+
+def test_matmul_epilogue_is_fused_and_compiles():
+    """Linear + sigmoid on the matrix-core kernel: the bias/sigmoid group that follows the product runs on the
+    accumulators (no separate element-wise launch between the first two products), and the kernel with the generated
+    epilogue compiles for gfx950."""
+    dev = Capture()
+    wl = W.mlp_train(dev, 256, (256, 256, 256, 128), 2)
+    proc, deps = wl.finish()
+    body = _loop_body(lower_describe(proc, deps))
+    assert "[dot_mfma]" in body[0] and "[dot_mfma]" in body[1], body[:3]
+    assert len(body[0].split("args:")[1].split()) > 12, body[0]   # epilogue buffers follow the twelve product arguments
+    rc, msg = _compile_check(proc, deps)
+    assert rc == 0, msg
