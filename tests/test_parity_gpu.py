@@ -401,3 +401,38 @@ def test_reduction_epilogue_values(V, R, hip_device):
     assert_close(got["b"].data, b + s, tol, "b", scale=scale)
     # z against the device's own y: the sine of a float32 argument
     assert_close(got["z"].data, np.sin(got["y"].data.astype(np.float64)), ELW_RTOL, "z", scale=1.0)
+
+
+@pytest.mark.parametrize("keep_p", [True, False])
+@pytest.mark.parametrize("m,k,n", [(256, 192, 128), (130, 70, 257), (512, 64, 384), (20, 10, 12)])
+def test_product_epilogue_values(m, k, n, keep_p, hip_device):
+    """W += c * (A x B) with only W kept: on the matrix-core kernel the update runs on the accumulators and the product
+    is never written (aligned and edge variants); the small case takes the unfused path.  A second consumer (y =
+    sin(P) + bias) in the same program keeps a stored product next to its epilogue."""
+    print(f"[case] product epilogue {m}x{k}x{n}", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(m * 7 + n)
+    a = rng.standard_normal(m * k).astype(np.float32)
+    b = rng.standard_normal(k * n).astype(np.float32)
+    w = rng.standard_normal(m * n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    cmds = [IR.CreateMat(a, [m, k], "a"), IR.CreateMat(b, [k, n], "b"), IR.CreateMat(w, [m, n], "w"),
+            IR.CreateMat(bias, [n], "bias"),
+            IR.DotProduct(a="a", b="b", res="d"), IR.CreateConstant(-0.01, "c", [m, n]), IR.ElwMultiply(a="d", b="c", res="t"),
+            IR.ElwAddEq(s="w", o="t"),
+            IR.DotProduct(a="a", b="b", res="p"), IR.View(a="bias", target_dim=[1, n], res="b1"),
+            IR.Broadcast(a="b1", dim=0, r=m, res="bb"), IR.Sin(a="p", res="sp"), IR.ElwAdd(a="sp", b="bb", res="y")]
+    got = _run_ir(hip_device, cmds, ["w", "y", "p"] if keep_p else ["w", "y"])
+    d = a.reshape(m, k).astype(np.float64) @ b.reshape(k, n).astype(np.float64)
+    tol = RED_RTOL * math.sqrt(k)
+    scale = float((np.abs(a.reshape(m, k)).astype(np.float64) @ np.abs(b.reshape(k, n)).astype(np.float64)).max())
+    assert_close(got["w"].data, (w.reshape(m, n) - 0.01 * d).reshape(-1), tol, "w", scale=scale)
+    if keep_p:
+        assert_close(got["p"].data, d.reshape(-1), tol, "p", scale=scale)
+        # y against the device's own p: the sine of a float32 argument plus one addition
+        exp_y = np.sin(got["p"].data.astype(np.float64)).reshape(m, n) + bias
+        assert_close(got["y"].data, exp_y.reshape(-1), 2e-6, "y", scale=1.0 + float(np.abs(bias).max()))
+    else:
+        # the product never reaches memory; sin amplifies its rounding error by at most 1
+        exp_y = np.sin(d) + bias
+        assert_close(got["y"].data, exp_y.reshape(-1), tol, "y", scale=scale)
