@@ -7,6 +7,7 @@
 // CreateMat payloads are uploaded once, not on every execution of their Alloc (kernels/alloc.rs:5-12);
 // counted loops cost one host synchronisation in total, not one per iteration (device.rs:133).
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hiprtc.h>
 
 #include <sys/stat.h>
@@ -352,18 +353,26 @@ void launch(adhip_program* p, const Launch& l) {
         }
         ptrs.push_back(&vals[i]);
     }
-    hipEvent_t e0 = nullptr, e1 = nullptr;
     if (p->profiling) {
-        e0 = get_event(p);
-        e1 = get_event(p);
-        HIP_OK(hipEventRecord(e0, ctx->stream));
-    }
-    HIP_OK(hipModuleLaunchKernel(p->fn[l.kernel], l.grid[0], l.grid[1], l.grid[2], l.block[0], l.block[1], l.block[2],
-                                 l.lds_bytes, ctx->stream, ptrs.data(), nullptr));
-    if (p->profiling) {
-        HIP_OK(hipEventRecord(e1, ctx->stream));
+        // the launch carries its own start and stop events, which take the kernel's begin and end on the device
+        // (events recorded around the launch would include the dispatch gap before it)
+        hipEvent_t e0 = get_event(p), e1 = get_event(p);
+        const uint64_t gx = (uint64_t)l.grid[0] * l.block[0], gy = (uint64_t)l.grid[1] * l.block[1],
+                       gz = (uint64_t)l.grid[2] * l.block[2];
+        if (gx <= 0xffffffffull && gy <= 0xffffffffull && gz <= 0xffffffffull) {
+            HIP_OK(hipExtModuleLaunchKernel(p->fn[l.kernel], (uint32_t)gx, (uint32_t)gy, (uint32_t)gz, l.block[0], l.block[1],
+                                            l.block[2], l.lds_bytes, ctx->stream, ptrs.data(), nullptr, e0, e1, 0));
+        } else {
+            HIP_OK(hipEventRecord(e0, ctx->stream));
+            HIP_OK(hipModuleLaunchKernel(p->fn[l.kernel], l.grid[0], l.grid[1], l.grid[2], l.block[0], l.block[1], l.block[2],
+                                         l.lds_bytes, ctx->stream, ptrs.data(), nullptr));
+            HIP_OK(hipEventRecord(e1, ctx->stream));
+        }
         p->pending.push_back({l.stat, {e0, e1}});
         if (p->pending.size() > 4096) drain_events(p);
+    } else {
+        HIP_OK(hipModuleLaunchKernel(p->fn[l.kernel], l.grid[0], l.grid[1], l.grid[2], l.block[0], l.block[1], l.block[2],
+                                     l.lds_bytes, ctx->stream, ptrs.data(), nullptr));
     }
     p->plan->stats[l.stat].launches++;
 }
