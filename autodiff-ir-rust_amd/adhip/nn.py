@@ -127,3 +127,105 @@ class SGD:
     def zero_grad(self):
         for p in self.n:
             p.reset_grad()
+
+
+# ---- attention / transformer encoder (reference src/nn/transformer.rs) ------------------------------
+# Everything works on 2-D tensors [sequence, features]: DotProduct is 2-D in the IR.  `softmax` is the
+# reference's composition (core.Tensor.softmax: exp(x) / exp(x).sum(dim), the sum broadcast back by the usual
+# trailing-dim rule, no maximum subtracted).
+
+def Attention(Q: Tensor, K: Tensor, V: Tensor, d_model: int) -> Tensor:
+    """dot(softmax(dot(Q, K^T) / sqrt(d_model), -1), V)  (transformer.rs:10-18)."""
+    import math
+    return dot((dot(Q, K.t()) / math.sqrt(float(d_model))).softmax(-1), V)
+
+
+def AttentionMasked(Q: Tensor, K: Tensor, V: Tensor, d_model: int, mask: Tensor) -> Tensor:
+    """As Attention with the scaled scores multiplied by `mask` before the softmax (transformer.rs:21-30)."""
+    import math
+    return dot((dot(Q, K.t()) / math.sqrt(float(d_model)) * mask).softmax(-1), V)
+
+
+class MultiHeadAttention(Module):
+    """Per head its own Linear(d_model, d_model / heads, no bias) for query, key and value; heads concatenated on
+    the last dim, then Linear(d_model, d_model, no bias) (transformer.rs:34-99)."""
+
+    def __init__(self, d_model: int, num_heads: int, mask: Optional[Tensor] = None):
+        assert d_model % num_heads == 0, "d_model must be divisible by num heads"
+        d_v = d_model // num_heads
+        self.wq = [Linear(d_model, d_v, False) for _ in range(num_heads)]
+        self.wk = [Linear(d_model, d_v, False) for _ in range(num_heads)]
+        self.wv = [Linear(d_model, d_v, False) for _ in range(num_heads)]
+        self.wo = Linear(d_model, d_model, False)
+        self.num_heads = num_heads
+        self.d_model = d_model
+        self.mask = mask
+
+    def params(self):
+        out: List[Tensor] = []
+        for group in (self.wq, self.wk, self.wv):
+            for lin in group:
+                out.extend(lin.params())
+        out.extend(self.wo.params())
+        return out
+
+    def f(self, query: Tensor, key: Optional[Tensor] = None, value: Optional[Tensor] = None) -> Tensor:
+        key = query if key is None else key
+        value = query if value is None else value
+        heads = []
+        for i in range(self.num_heads):
+            q, k, v = self.wq[i].f(query), self.wk[i].f(key), self.wv[i].f(value)
+            if self.mask is not None:
+                heads.append(AttentionMasked(q, k, v, self.d_model, self.mask))
+            else:
+                heads.append(Attention(q, k, v, self.d_model))
+        from .core import concat
+        return self.wo.f(concat(heads, -1))
+
+
+def MaskedMultiHeadAttention(d_model: int, num_heads: int, mask: Tensor) -> MultiHeadAttention:
+    return MultiHeadAttention(d_model, num_heads, mask)
+
+
+class AttentionFeedforward(Module):
+    """Linear(d_model, inner, bias) then Linear(inner, d_model, bias), nothing in between (transformer.rs:130-155)."""
+
+    def __init__(self, d_model: int, inner_dim: int):
+        self.w_expand = Linear(d_model, inner_dim, True)
+        self.w_contract = Linear(inner_dim, d_model, True)
+
+    def params(self):
+        return self.w_expand.params() + self.w_contract.params()
+
+    def f(self, x):
+        return self.w_contract.f(self.w_expand.f(x))
+
+
+class TransformerEncoderLayer(Module):
+    """y = LayerNorm(x + MHA(x, x, x)); LayerNorm(y + FF(y))  (transformer.rs:158-192)."""
+
+    def __init__(self, d_model: int, num_heads: int, ff_dim: int):
+        self.attention = MultiHeadAttention(d_model, num_heads)
+        self.layer_norm_att = LayerNorm(d_model)
+        self.layer_norm_ffwd = LayerNorm(d_model)
+        self.ffwd = AttentionFeedforward(d_model, ff_dim)
+
+    def params(self):
+        return self.attention.params() + self.ffwd.params() + self.layer_norm_att.params() + self.layer_norm_ffwd.params()
+
+    def f(self, x):
+        y = self.layer_norm_att.f(x + self.attention.f(x, x, x))
+        return self.layer_norm_ffwd.f(y + self.ffwd.f(y))
+
+
+class TransformerEncoder(Module):
+    def __init__(self, num_layers: int, d_model: int, num_heads: int, ff_dim: int):
+        self.layers = Sequential()
+        for _ in range(num_layers):
+            self.layers.insert(TransformerEncoderLayer(d_model, num_heads, ff_dim))
+
+    def params(self):
+        return self.layers.params()
+
+    def f(self, x):
+        return self.layers.f(x)

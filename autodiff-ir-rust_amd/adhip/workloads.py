@@ -232,3 +232,67 @@ def manip_loop(dev, nb: int = 64, n1: int = 512, n2: int = 1024, n3: int = 256, 
     outs = {"gathered": g0.val(), "r": r.val(), "i": i.val()}
     return Workload("manip_loop", outs, {"p": pn, "q": qn, "w": wn},
                     algorithmic_bytes=4.0 * 2 * rows * width)
+
+
+# ---- a transformer encoder layer (the caller-side modules of reference src/nn/transformer.rs) ----------
+
+def encoder_layer(dev, seq: int = 64, d_model: int = 32, heads: int = 4, ff_dim: int = 64, seed: int = 0,
+                  backward: bool = True) -> Workload:
+    """x [seq, d_model]; y = TransformerEncoderLayer(d_model, heads, ff_dim)(x); L = (y * r).sum(0).sum(0) with a fixed
+    random r; backward to x and every parameter.  Weights are N(0, 1/fan_in) and passed in explicitly (the
+    reference's `randn` is unseeded), so a restatement in another framework can use the same values."""
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    inputs: Dict[str, np.ndarray] = {}
+
+    def mat(name, fan_in, fan_out):
+        w = (rng.standard_normal((fan_in, fan_out)) / np.sqrt(fan_in)).astype(np.float32)
+        inputs[name] = w
+        return autodiff.tensor(w, [fan_in, fan_out])
+
+    def vec(name, n):
+        b = (0.1 * rng.standard_normal(n)).astype(np.float32)
+        inputs[name] = b
+        return autodiff.tensor(b, [n])
+
+    layer = nn.TransformerEncoderLayer(d_model, heads, ff_dim)
+    d_v = d_model // heads
+    named = {}
+    for h in range(heads):
+        for kind, group in (("wq", layer.attention.wq), ("wk", layer.attention.wk), ("wv", layer.attention.wv)):
+            group[h].w = mat(f"{kind}{h}", d_model, d_v)
+            named[f"{kind}{h}"] = group[h].w
+    layer.attention.wo.w = mat("wo", d_model, d_model)
+    named["wo"] = layer.attention.wo.w
+    layer.ffwd.w_expand.w = mat("w1", d_model, ff_dim)
+    layer.ffwd.w_expand.b = vec("b1", ff_dim)
+    layer.ffwd.w_contract.w = mat("w2", ff_dim, d_model)
+    layer.ffwd.w_contract.b = vec("b2", d_model)
+    named.update({"w1": layer.ffwd.w_expand.w, "b1": layer.ffwd.w_expand.b, "w2": layer.ffwd.w_contract.w,
+                  "b2": layer.ffwd.w_contract.b, "ln1_scale": layer.layer_norm_att.scale,
+                  "ln2_scale": layer.layer_norm_ffwd.scale})
+    xn = rng.standard_normal((seq, d_model)).astype(np.float32)
+    rn = rng.standard_normal((seq, d_model)).astype(np.float32)
+    inputs["x"], inputs["r"] = xn, rn
+    x = autodiff.tensor(xn, [seq, d_model])
+    r = autodiff.tensor(rn, [seq, d_model])
+    y = layer.f(x)
+    L = (y * r).sum(0).sum(0)
+    L.forward()
+    y.val().keep()
+    L.val().keep()
+    outs = {"y": y.val(), "L": L.val()}
+    if backward:
+        L.backward()
+        outs["dx"] = x.grad()
+        for name, p in named.items():
+            outs["d" + name] = p.grad()
+        for v in outs.values():
+            v.keep()
+    # matmul flops: forward 2*M*N*K per product, backward twice that
+    fl = 0.0
+    fl += heads * 3 * 2.0 * seq * d_model * d_v            # q, k, v projections
+    fl += heads * 2 * 2.0 * seq * seq * d_v                # scores and weighted values
+    fl += 2.0 * seq * d_model * d_model                     # output projection
+    fl += 2 * 2.0 * seq * d_model * ff_dim                  # feed-forward
+    return Workload("encoder_layer", outs, inputs, flops=fl * (3.0 if backward else 1.0))

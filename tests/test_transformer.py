@@ -1,0 +1,72 @@
+"""The attention / transformer-encoder modules of the caller side (reference src/nn/transformer.rs) end to end:
+forward and every gradient of one encoder layer against a float64 restatement in torch, on the oracle (CPU) and on
+the device (GPU), and the device against the oracle."""
+import math
+
+import numpy as np
+import pytest
+
+from adhip import autodiff
+from adhip import workloads as W
+from adhip.core import dot
+from oracle.interp import OracleDevice
+from parity import RED_RTOL, assert_close
+from transformer_ref import encoder_layer_reference
+
+
+def _against_reference(out, inputs, heads, rtol):
+    ref = encoder_layer_reference(inputs, heads)
+    assert set(out) == set(ref)
+    for k, v in out.items():
+        assert not v.is_none, k
+        assert list(v.dim) == list(ref[k].shape), k
+        assert_close(v.data, ref[k].reshape(-1), rtol, k)
+
+
+@pytest.mark.parametrize("seq,d_model,heads,ff", [(8, 16, 4, 32), (12, 8, 1, 8), (24, 32, 2, 48)])
+def test_encoder_layer_oracle_matches_float64_autograd(seq, d_model, heads, ff):
+    wl = W.encoder_layer(OracleDevice(), seq, d_model, heads, ff, seed=seq)
+    _against_reference(wl.run(), wl.inputs, heads, 2e-5)
+
+
+def test_leaf_gradients_do_not_alias():
+    """v = x + w feeds two consumers: the gradient value handed to x and to w is one and the same IR id, so adding
+    the second contribution in place (as the reference does) would change both leaves' gradients twice."""
+    autodiff.set_device(OracleDevice())
+    rng = np.random.default_rng(3)
+    xn, wn = rng.standard_normal((6, 8)).astype(np.float32), rng.standard_normal((6, 8)).astype(np.float32)
+    x, w = autodiff.tensor(xn, [6, 8]), autodiff.tensor(wn, [6, 8])
+    v = x + w
+    L = (v * v).sum(0).sum(0)
+    L.forward()
+    L.backward()
+    gx, gw = x.grad(), w.grad()
+    gx.keep()
+    gw.keep()
+    autodiff.execute()
+    expect = 2.0 * (xn.astype(np.float64) + wn)
+    assert_close(gx.get().data, expect.reshape(-1), 1e-6, "dx")
+    assert_close(gw.get().data, expect.reshape(-1), 1e-6, "dw")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seq,d_model,heads,ff", [(8, 16, 4, 32), (64, 32, 4, 64), (200, 96, 3, 160)])
+def test_encoder_layer_device_matches_oracle_and_reference(seq, d_model, heads, ff, hip_device):
+    print(f"[case] encoder layer {seq}x{d_model} heads {heads} ff {ff}", flush=True)
+    got = W.encoder_layer(hip_device, seq, d_model, heads, ff, seed=seq).run()
+    wl = W.encoder_layer(OracleDevice(), seq, d_model, heads, ff, seed=seq)
+    ref = wl.run()
+    tol = 4 * RED_RTOL * math.sqrt(max(seq, d_model, ff))
+    for k, rv in ref.items():
+        assert got[k].dim == rv.dim, k
+        assert_close(got[k].data, rv.data, tol, k)
+    _against_reference(got, wl.inputs, heads, 1e-4)
+
+
+@pytest.mark.gpu
+def test_encoder_layer_matrix_core_sizes(hip_device):
+    """Sizes at which every product goes to the MFMA kernel (aligned and edge variants, epilogues included), checked
+    against float64 autograd only (the oracle's one-thread-per-output matmul is too slow here)."""
+    print("[case] encoder layer 512x256", flush=True)
+    wl = W.encoder_layer(hip_device, 512, 256, 4, 1024, seed=5)
+    _against_reference(wl.run(), wl.inputs, 4, 2e-4)
