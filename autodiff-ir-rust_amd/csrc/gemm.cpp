@@ -3,9 +3,10 @@
 // The reference multiplies with one work-item per output element, a sequential k loop and two
 // global loads per multiply-add (reference src/devices/opencl/kernels/dotprod.rs:23-53); transposed
 // operands are folded into its index expressions.  Here both operands are described by strides
-// (so x^T and W^T of the backward pass need no copy), staged through LDS in 128x128x16 or 256x128x16
-// tiles with register prefetch of the next tile, and each of the four (eight) wavefronts of a block
-// owns a 64x64 sub-tile = 2x2 MFMA blocks of 32x32.
+// (so x^T and W^T of the backward pass need no copy), staged through LDS in 256x128x16, 128x128x16 or
+// 64x64x16 tiles with register prefetch of the next tile.  A wavefront owns a 64x64 sub-tile (2x2 MFMA
+// blocks of 32x32) in the two large tiles and one 32x32 block in the small one, which exists so that
+// products with a small output still put a few hundred blocks on the chip.
 #include "gemm.hpp"
 
 #include "common.hpp"
@@ -30,16 +31,20 @@ std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry, 
         }
         s += m + "\n";
     }
-    s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n", cfg.a_kcontig ? 1 : 0, cfg.b_kcontig ? 1 : 0,
-              cfg.edge ? 1 : 0);
-    s += strf("#define KERNEL_NAME %s\n#define BM %d\n", entry.c_str(), cfg.bm);
+    s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n#define SPLITK %d\n", cfg.a_kcontig ? 1 : 0,
+              cfg.b_kcontig ? 1 : 0, cfg.edge ? 1 : 0, cfg.split_k ? 1 : 0);
+    // tile geometry: BM x BN block tile, TM x TN MFMA blocks per wave, WGN waves along n
+    const int tm = cfg.bm == 64 ? 1 : 2, bn = cfg.bm == 64 ? 64 : 128;
+    const int waves = (cfg.bm / (32 * tm)) * (bn / (32 * tm));
+    s += strf("#define KERNEL_NAME %s\n#define BM %d\n#define BN %d\n#define TM %d\n#define TN %d\n#define NT %d\n", entry.c_str(),
+              cfg.bm, bn, tm, tm, waves * 64);
     s += R"(
-#define BN 128
 #define BK 16
 #define LDA (BM + 4)
 #define LDB (BN + 4)
-#define NT (BM * 2)            /* threads: one wave per 64x64 sub-tile */
-#define B_LOADS (512 / NT)     /* float4 loads of the B tile per thread */
+#define WGN (BN / (32 * TN))            /* waves along n */
+#define A_LOADS (BM * BK / 4 / NT)      /* float4 loads of the A tile per thread */
+#define B_LOADS (BN * BK / 4 / NT)      /* float4 loads of the B tile per thread */
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
@@ -47,17 +52,31 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 // A_KCONTIG: a_sk == 1 (else a_sm == 1).  B_KCONTIG: b_sk == 1 (else b_sn == 1).
 // EDGE: M, N or K is not a multiple of the tile, or an operand is not 16-byte aligned; every
 // access is then bounds-checked and scalar.
+// SPLITK: the block at blockIdx.y multiplies only k in [y*k_chunk, (y+1)*k_chunk) and writes slice y of a
+// [gridDim.y][M][N] buffer; the caller adds the slices in a fixed order.  For products whose output alone gives
+// too few blocks to hide the latency of the operand loads.
 extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     const int* __restrict__ guard, float* __restrict__ C, const float* __restrict__ A, const float* __restrict__ B,
     long long M, long long N, long long K, long long a_off, long long a_sm, long long a_sk, long long b_off,
-    long long b_sk, long long b_sn EPI_PARAMS) {
+    long long b_sk, long long b_sn
+#if SPLITK
+    , long long k_chunk
+#endif
+    EPI_PARAMS) {
     if (guard && *guard == 0) return;
+#if SPLITK
+    const long long k_lo = (long long)blockIdx.y * k_chunk;
+    const long long k_hi = min(K, k_lo + k_chunk);
+    C += (long long)blockIdx.y * M * N;
+#else
+    const long long k_lo = 0, k_hi = K;
+#endif
     __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDB];
 
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u, wave = tid >> 6;
-    const unsigned wm = wave >> 1, wn = wave & 1u;
+    const unsigned wm = wave / WGN, wn = wave % WGN;
     const unsigned li = lane & 31u, lh = lane >> 5;
 
     // Block -> tile.  Consecutive block ids go to different XCDs (8 of them, each with its own L2), so
@@ -79,19 +98,19 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     A += a_off;
     B += b_off;
 
-    float16_t acc[2][2];
+    float16_t acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    float4_t ra0[2], rb0[B_LOADS];
+    float4_t ra0[A_LOADS], rb0[B_LOADS];
 
     auto load_a = [&](long long k0, float4_t* ra) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < A_LOADS; ++i) {
 #if A_KCONTIG
             const unsigned kq = tid & 3u, mr = (tid >> 2) + (NT / 4) * i;
             const long long m = bm + mr, k = k0 + 4 * kq;
@@ -100,18 +119,18 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
             if (m < M) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    if (k + j < K) v[j] = A[m * a_sm + (k + j) * a_sk];
+                    if (k + j < k_hi) v[j] = A[m * a_sm + (k + j) * a_sk];
             }
             ra[i] = v;
 #else
             ra[i] = *(const float4_t*)(A + m * a_sm + k);
 #endif
 #else
-            const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + 8u * i;
+            const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + (NT / (BM / 4)) * i;
             const long long m = bm + 4 * mq, k = k0 + kr;
 #if EDGE
             float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (k < K) {
+            if (k < k_hi) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     if (m + j < M) v[j] = A[(m + j) * a_sm + k * a_sk];
@@ -134,18 +153,18 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
             if (n < N) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    if (k + j < K) v[j] = B[(k + j) * b_sk + n * b_sn];
+                    if (k + j < k_hi) v[j] = B[(k + j) * b_sk + n * b_sn];
             }
             rb[i] = v;
 #else
             rb[i] = *(const float4_t*)(B + n * b_sn + k);
 #endif
 #else
-            const unsigned nq = tid & 31u, kr = (tid >> 5) + (NT / 32) * i;
+            const unsigned nq = tid % (BN / 4), kr = tid / (BN / 4) + (NT / (BN / 4)) * i;
             const long long n = bn + 4 * nq, k = k0 + kr;
 #if EDGE
             float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (k < K) {
+            if (k < k_hi) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     if (n + j < N) v[j] = B[k * b_sk + (n + j) * b_sn];
@@ -159,13 +178,13 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     };
     auto store_tiles = [&](int buf, const float4_t* ra, const float4_t* rb) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < A_LOADS; ++i) {
 #if A_KCONTIG
             const unsigned kq = tid & 3u, mr = (tid >> 2) + (NT / 4) * i;
 #pragma unroll
             for (int j = 0; j < 4; ++j) As[buf][4 * kq + j][mr] = ra[i][j];
 #else
-            const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + 8u * i;
+            const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + (NT / (BM / 4)) * i;
             *(float4_t*)&As[buf][kr][4 * mq] = ra[i];
 #endif
         }
@@ -176,7 +195,7 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
 #pragma unroll
             for (int j = 0; j < 4; ++j) Bs[buf][4 * kq + j][nr] = rb[i][j];
 #else
-            const unsigned nq = tid & 31u, kr = (tid >> 5) + (NT / 32) * i;
+            const unsigned nq = tid % (BN / 4), kr = tid / (BN / 4) + (NT / (BN / 4)) * i;
             *(float4_t*)&Bs[buf][kr][4 * nq] = rb[i];
 #endif
         }
@@ -186,57 +205,58 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     // four MFMAs of step ks are issued, and half way through the tile that was prefetched into registers (sa, sb)
     // is parked in the other LDS buffer, which nobody reads during this iteration.
     auto compute = [&](int cur, bool park, const float4_t* sa, const float4_t* sb) {
-        float fa0[2], fa1[2], fb0[2], fb1[2];
-        fa0[0] = As[cur][lh][wm * 64 + li];
-        fa1[0] = As[cur][lh][wm * 64 + 32 + li];
-        fb0[0] = Bs[cur][lh][wn * 64 + li];
-        fb1[0] = Bs[cur][lh][wn * 64 + 32 + li];
+        float fa[TM][2], fb[TN][2];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i][0] = As[cur][lh][wm * (32 * TM) + 32 * i + li];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j][0] = Bs[cur][lh][wn * (32 * TN) + 32 * j + li];
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ++ks) {
             const int c = ks & 1, nx = c ^ 1;
             if (ks + 1 < BK / 2) {
-                fa0[nx] = As[cur][2 * (ks + 1) + lh][wm * 64 + li];
-                fa1[nx] = As[cur][2 * (ks + 1) + lh][wm * 64 + 32 + li];
-                fb0[nx] = Bs[cur][2 * (ks + 1) + lh][wn * 64 + li];
-                fb1[nx] = Bs[cur][2 * (ks + 1) + lh][wn * 64 + 32 + li];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i][nx] = As[cur][2 * (ks + 1) + lh][wm * (32 * TM) + 32 * i + li];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fb[j][nx] = Bs[cur][2 * (ks + 1) + lh][wn * (32 * TN) + 32 * j + li];
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads ahead of the MFMAs that hide their latency
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0[c], fb0[c], acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0[c], fb1[c], acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1[c], fb0[c], acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1[c], fb1[c], acc[1][1], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][c], fb[j][c], acc[i][j], 0, 0, 0);
             if (ks == BK / 4 - 1 && park) store_tiles(cur ^ 1, sa, sb);
         }
     };
 
     // The next tile's global loads are issued before the current tile is multiplied (one tile ahead).
-    const long long KT = (K + BK - 1) / BK;
-    load_a(0, ra0);
-    load_b(0, rb0);
+    const long long KT = (k_hi - k_lo + BK - 1) / BK;
+    load_a(k_lo, ra0);
+    load_b(k_lo, rb0);
     store_tiles(0, ra0, rb0);
     __syncthreads();
 
     for (long long kt = 0; kt < KT; ++kt) {
         const bool more = kt + 1 < KT;
         if (more) {
-            load_a((kt + 1) * BK, ra0);
-            load_b((kt + 1) * BK, rb0);
+            load_a(k_lo + (kt + 1) * BK, ra0);
+            load_b(k_lo + (kt + 1) * BK, rb0);
         }
         compute((int)(kt & 1), more, ra0, rb0);
         __syncthreads();
     }
 
-    // acc[i][j][4g + r] holds C[row = 32i + 8g + 4*lh + r][col = 32j + li] of the wave's 64x64 tile
+    // acc[i][j][4g + r] holds C[row = 32i + 8g + 4*lh + r][col = 32j + li] of the wave's sub-tile
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int g = 0; g < 4; ++g)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const long long row = bm + wm * 64 + 32 * i + 8 * g + 4 * lh + r;
-                    const long long col = bn + wn * 64 + 32 * j + li;
+                    const long long row = bm + wm * (32 * TM) + 32 * i + 8 * g + 4 * lh + r;
+                    const long long col = bn + wn * (32 * TN) + 32 * j + li;
 #if EDGE
                     if (row < M && col < N)
 #endif

@@ -135,6 +135,31 @@ extern "C" __global__ __launch_bounds__(1024) void adhip_colsum_finalize(
     }
 }
 
+// out[i] = slices[0][i] + slices[1][i] + ... in that order, i < n; four elements per thread when n allows.
+// Adds the partial products of a matrix product whose k range was cut into `count` pieces.
+extern "C" __global__ __launch_bounds__(256) void adhip_sum_slices(const int* __restrict__ guard, float* __restrict__ out,
+                                                                   const float* __restrict__ slices, long long count,
+                                                                   long long n) {
+    if (guard && *guard == 0) return;
+    const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    if ((n & 3) == 0) {
+        float4 acc = *(const float4*)(slices + i);
+#pragma unroll 4
+        for (long long s = 1; s < count; ++s) {
+            const float4 v = *(const float4*)(slices + s * n + i);
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+        *(float4*)(out + i) = acc;
+    } else {
+        for (long long j = i; j < n && j < i + 4; ++j) {
+            float acc = slices[j];
+            for (long long s = 1; s < count; ++s) acc += slices[s * n + j];
+            out[j] = acc;
+        }
+    }
+}
+
 // One thread per output element, k ascending, one accumulator: the reference's dot kernel
 // (src/devices/opencl/kernels/dotprod.rs:23-53).  Used for small products.
 extern "C" __global__ __launch_bounds__(256) void adhip_dot_naive(const int* __restrict__ guard, float* __restrict__ c,
@@ -198,7 +223,7 @@ struct Lowerer {
     std::vector<std::unique_ptr<Node>> arena;
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
-    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1;
+    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sum_slices = -1;
     int dot_epilogue_counter = 0;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
 
@@ -1195,7 +1220,13 @@ struct Lowerer {
                 Node* D = G.members[0];
                 size_t nx = g + 1;
                 while (nx < groups.size() && groups[nx].dead) ++nx;
-                if (opt.fuse && dot_uses_mfma(D) && nx < groups.size() && groups[nx].kind == Group::ELW &&
+                DotLaunchPlan dpl;
+                if (dot_uses_mfma(D)) dpl = plan_dot(D);
+                if (dpl.splits > 1) {
+                    Node* partial = new_node(Op::COPY, Shape{dpl.splits, numel(D->shape)}, {}, D->name + ".slices", 0.f, false);
+                    partial->root = true;
+                    gks[g].extra_nodes.push_back(partial);
+                } else if (opt.fuse && dot_uses_mfma(D) && nx < groups.size() && groups[nx].kind == Group::ELW &&
                     groups[nx].colsums.empty() && groups[nx].n == numel(D->shape)) {
                     bool uses = false, ok = true;
                     for (Node* m : groups[nx].members) {
@@ -1391,7 +1422,7 @@ struct Lowerer {
             if (G.dead) continue;
             if (G.kind == Group::DOT) {
                 if (!G.epi.empty()) emit_dot(G.members[0], out, &gks[g].dot_epi, gks[g].dot_store);
-                else emit_dot(G.members[0], out);
+                else emit_dot(G.members[0], out, nullptr, true, gks[g].extra_nodes.empty() ? nullptr : gks[g].extra_nodes[0]);
                 continue;
             }
             if (G.kind == Group::TRANSPOSE) {
@@ -1512,7 +1543,51 @@ struct Lowerer {
         return M * N * K >= 64 * 64 * 64 && a_unit && b_unit;
     }
 
-    void emit_dot(Node* n, std::vector<Step>& out, const DotEpilogueCode* epi = nullptr, bool store_c = true) {
+    // How a matrix-core product is launched: tile, bounds checking, and how many ranges of k it is split into.
+    struct DotLaunchPlan {
+        GemmConfig cfg;
+        int bn_tile = 128;
+        int64_t splits = 1, k_chunk = 0;
+    };
+    static DotLaunchPlan plan_dot(const Node* n) {
+        Affine2D a, b;
+        tref_affine2d(n->in[0], a);
+        tref_affine2d(n->in[1], b);
+        const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
+        DotLaunchPlan pl;
+        GemmConfig& cfg = pl.cfg;
+        cfg.a_kcontig = a.s1 == 1;
+        cfg.b_kcontig = b.s0 == 1;
+        const int64_t a_ld = cfg.a_kcontig ? a.s0 : a.s1, b_ld = cfg.b_kcontig ? b.s1 : b.s0;
+        const bool unaligned = (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
+        // the largest block tile that still puts enough blocks on the chip's 256 CUs: 256x128 (8 waves) with at
+        // least two blocks per CU, 128x128 with at least one -- counting the ranges k can be cut into (each at
+        // least 256 deep; the slices are added afterwards) -- else 64x64, cut the same way.  A block that has a CU
+        // to itself cannot hide the latency of its operand loads, hence the target of about 512 blocks.
+        const int64_t blocks128 = ((M + 127) / 128) * ((N + 127) / 128);
+        const int64_t max_splits = std::min<int64_t>(K / 256, 32);
+        auto splits_for = [&](int64_t blocks) {
+            if (blocks >= 256 || max_splits < 2) return (int64_t)1;
+            return std::max<int64_t>(std::min<int64_t>((512 + blocks - 1) / blocks, max_splits), 1);
+        };
+        if (!unaligned && M % 256 == 0 && N % 128 == 0 && (M / 256) * (N / 128) >= 512) cfg.bm = 256;
+        else if (blocks128 * splits_for(blocks128) >= 256) cfg.bm = 128;
+        else cfg.bm = 64;
+        pl.bn_tile = cfg.bm == 64 ? 64 : 128;
+        cfg.edge = unaligned || (M % cfg.bm) || (N % pl.bn_tile);
+        const int64_t blocks = ((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile);
+        const int64_t want = cfg.bm == 256 ? 1 : splits_for(blocks);
+        if (want > 1) {
+            pl.k_chunk = (((K + want - 1) / want) + 15) / 16 * 16;
+            pl.splits = (K + pl.k_chunk - 1) / pl.k_chunk;
+            cfg.split_k = pl.splits > 1;
+            if (!cfg.split_k) pl.splits = 1;
+        }
+        return pl;
+    }
+
+    void emit_dot(Node* n, std::vector<Step>& out, const DotEpilogueCode* epi = nullptr, bool store_c = true,
+                  Node* partial = nullptr) {
         Affine2D a, b;
         ADHIP_CHECK(tref_affine2d(n->in[0], a) && tref_affine2d(n->in[1], b), "internal: matmul operand is not a strided view");
         const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
@@ -1522,14 +1597,12 @@ struct Lowerer {
         ADHIP_CHECK(!epi || dot_uses_mfma(n), "internal: product epilogue on the small-product kernel");
         if (M * N * K >= 64 * 64 * 64 && a_unit && b_unit) {
             // matrix-core kernel; operands keep their strides (x^T, W^T are never copied)
-            GemmConfig cfg;
-            cfg.a_kcontig = a.s1 == 1;
-            cfg.b_kcontig = b.s0 == 1;
-            const int64_t a_ld = cfg.a_kcontig ? a.s0 : a.s1, b_ld = cfg.b_kcontig ? b.s1 : b.s0;
-            cfg.edge = (M % 128) || (N % 128) || (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
-            // 256-row tiles (8 waves) when that still leaves two blocks per CU; else 128-row tiles
-            cfg.bm = (!cfg.edge && M % 256 == 0 && (M / 256) * (N / 128) >= 512) ? 256 : 128;
-            std::string entry = strf("adhip_gemm_%c%c_%d%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm, cfg.edge ? "_edge" : "");
+            DotLaunchPlan pl = plan_dot(n);
+            GemmConfig cfg = pl.cfg;
+            const int bn_tile = pl.bn_tile;
+            ADHIP_CHECK(!cfg.split_k || (partial && !epi), "internal: split product without its slice buffer");
+            std::string entry = strf("adhip_gemm_%c%c_%d%s%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
+                                     cfg.edge ? "_edge" : "", cfg.split_k ? "_splitk" : "");
             Launch l;
             if (epi) {
                 // the element-wise group that followed the product runs on the accumulators; every distinct
@@ -1544,11 +1617,15 @@ struct Lowerer {
             } else {
                 l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
             }
-            l.block[0] = (unsigned)(cfg.bm * 2);
-            l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + 127) / 128));
+            l.block[0] = cfg.bm == 64 ? 256u : (unsigned)(cfg.bm * 2);
+            l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + bn_tile - 1) / bn_tile));
             // a product that is not stored has no buffer; the kernel never touches C then
-            Node* c_arg = store_c ? n : (epi ? epi->buffer_args[0] : n);
+            Node* c_arg = cfg.split_k ? partial : (store_c ? n : (epi ? epi->buffer_args[0] : n));
             l.args = {B(c_arg), B(a.base), B(b.base), I(M), I(N), I(K), I(a.offset), I(a.s0), I(a.s1), I(b.offset), I(b.s0), I(b.s1)};
+            if (cfg.split_k) {
+                l.args.push_back(I(pl.k_chunk));
+                l.grid[1] = (unsigned)pl.splits;
+            }
             l.label = strf("dot_%s_%lldx%lldx%lld", n->name.c_str(), (long long)M, (long long)N, (long long)K);
             l.bytes = 4.0 * ((double)M * K + (double)K * N + (store_c ? (double)M * N : 0.0));
             l.flops = 2.0 * (double)M * (double)N * (double)K;
@@ -1560,6 +1637,19 @@ struct Lowerer {
                 l.flops += epi->flops * (double)M * (double)N;
             }
             push_launch(out, l, "dot_mfma");
+            if (cfg.split_k) {
+                // add the slices in a fixed order
+                if (fixed_sum_slices < 0) fixed_sum_slices = add_kernel("adhip_sum_slices", fixed_kernels_source(), "sum_slices");
+                Launch lf;
+                lf.kernel = fixed_sum_slices;
+                lf.block[0] = 256;
+                lf.grid[0] = (unsigned)((M * N + 1023) / 1024);
+                lf.args = {B(n), B(partial), I(pl.splits), I(M * N)};
+                lf.label = l.label + "_sum";
+                lf.bytes = 4.0 * (double)M * (double)N * (double)(pl.splits + 1);
+                lf.flops = (double)M * (double)N * (double)pl.splits;
+                push_launch(out, lf, "sum_slices");
+            }
             return;
         }
         if (fixed_dot < 0) fixed_dot = add_kernel("adhip_dot_naive", fixed_kernels_source(), "dot_naive");

@@ -189,6 +189,17 @@ def main():
         p5.close()
         # config 4: dense MLP training
         extra["mlp_train"] = measure_mlp(dev, args.mlp_iters)
+        # beyond BASELINE.json's configs: one transformer encoder layer (the caller side's attention modules),
+        # forward + backward, [2048, 1024] activations, 8 heads, feed-forward width 4096
+        wl6 = W.encoder_layer(dev, 2048, 1024, 8, 4096, seed=0)
+        p6 = compile_resident(dev, wl6)
+        ms6 = timed_runs(p6, 5, 2)
+        k6 = profile(p6, 2)
+        dot6 = sum(k["avg_ms"] * k["launches_per_run"] for k in k6 if k["kernel"].startswith("dot"))
+        extra["encoder_layer"] = {"ms_per_step": ms6, "matmul_flops_per_step": wl6.flops,
+                                  "matmul_TFLOPs_whole_step": wl6.flops / (ms6 * 1e-3) / 1e12,
+                                  "matmul_kernels_ms": dot6, "launches_per_step": sum(k["launches_per_run"] for k in k6)}
+        p6.close()
 
     cpu = None
     if not args.skip_cpu:

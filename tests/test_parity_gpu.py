@@ -282,7 +282,15 @@ def test_shape_errors_are_reported(hip_device):
 
 @pytest.mark.parametrize("m,k,n", [(2048, 256, 4096), (1024, 64, 8192)])
 def test_dot_large_tile_variant(m, k, n, hip_device):
-    """Shapes that select the 256-row block tile (8 waves) of the MFMA kernel, all three operand layouts."""
+    """Shapes that select the 128x128 block tile of the MFMA kernel (the small shapes above take the 64x64 tile, the
+    full-size MLP test the 256x128 one), all three operand layouts."""
+    test_dot_forward_backward(m, k, n, hip_device)
+
+
+@pytest.mark.parametrize("m,k,n", [(128, 4096, 128), (256, 1024, 64), (100, 2000, 70), (64, 520, 192)])
+def test_dot_split_k(m, k, n, hip_device):
+    """Small outputs with a long inner dimension: k is cut into ranges computed by different blocks and the slices are
+    added afterwards (aligned and bounds-checked variants, a last range shorter than the others)."""
     test_dot_forward_backward(m, k, n, hip_device)
 
 
