@@ -240,3 +240,24 @@ def test_matmul_epilogue_is_fused_and_compiles():
     assert len(body[0].split("args:")[1].split()) > 12, body[0]   # epilogue buffers follow the twelve product arguments
     rc, msg = _compile_check(proc, deps)
     assert rc == 0, msg
+
+
+def test_no_gpu_means_an_error_not_a_fallback():
+    """Without a GPU the device cannot be created and says so; there is no CPU path to fall back to.  (Skipped where a
+    GPU is present.)"""
+    lib = load_library()
+    lib.adhip_create.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
+    lib.adhip_create.restype = ctypes.c_int
+    lib.adhip_last_error.argtypes = [ctypes.c_void_p]
+    lib.adhip_last_error.restype = ctypes.c_char_p
+    ctx = ctypes.c_void_p()
+    rc = lib.adhip_create(0, ctypes.byref(ctx))
+    if rc == 0:
+        lib.adhip_destroy.argtypes = [ctypes.c_void_p]
+        lib.adhip_destroy(ctx)
+        pytest.skip("a GPU is present")
+    assert not ctx.value
+    assert lib.adhip_last_error(None), "a failed adhip_create must leave a message"
+    from adhip import HipDevice
+    with pytest.raises(RuntimeError):
+        HipDevice(0)
