@@ -70,3 +70,47 @@ def test_encoder_layer_matrix_core_sizes(hip_device):
     print("[case] encoder layer 512x256", flush=True)
     wl = W.encoder_layer(hip_device, 512, 256, 4, 1024, seed=5)
     _against_reference(wl.run(), wl.inputs, 4, 2e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["layernorm", "rms", "softmax"])
+@pytest.mark.parametrize("rows,cols", [(2048, 768), (333, 1000)])
+def test_norm_modules_at_scale_match_float64_autograd(kind, rows, cols, hip_device):
+    """LayerNorm, RMS and the reference's softmax composition over a few thousand rows, forward and backward, against
+    float64 autograd (their small known-answer tests are in the reference's norm.rs)."""
+    print(f"[case] {kind} {rows}x{cols}", flush=True)
+    import torch
+    from adhip import nn
+    rng = np.random.default_rng(rows + cols)
+    xn = rng.standard_normal((rows, cols)).astype(np.float32)
+    rn = rng.standard_normal((rows, cols)).astype(np.float32)
+    if kind == "softmax":
+        rows = cols = min(rows, cols)          # the composition divides [R,C] by a [R] vector: square inputs only
+        xn, rn = xn[:rows, :cols].copy(), rn[:rows, :cols].copy()
+        xn *= 0.25
+    autodiff.set_device(hip_device)
+    x = autodiff.tensor(xn, [rows, cols])
+    mod = {"layernorm": lambda: nn.LayerNorm(cols), "rms": lambda: nn.RMS(cols), "softmax": lambda: nn.Softmax(-1)}[kind]()
+    y = mod.f(x)
+    L = (y * autodiff.tensor(rn, [rows, cols])).sum(0).sum(0)
+    L.forward()
+    L.backward()
+    y.val().keep()
+    x.grad().keep()
+    autodiff.execute()
+    got_y, got_dx = y.val().get(), x.grad().get()
+
+    xt = torch.tensor(xn, dtype=torch.float64, requires_grad=True)
+    if kind == "layernorm":
+        mean = xt.mean(-1, keepdim=True)
+        var = ((xt - mean) ** 2).sum(-1) / cols
+        yt = (xt - mean) / torch.sqrt(var + 1e-9).unsqueeze(-1)
+    elif kind == "rms":
+        yt = xt / torch.sqrt((xt ** 2).mean(-1, keepdim=True) + 1e-9)
+    else:
+        e = torch.exp(xt)
+        yt = e / e.sum(-1)
+    (yt * torch.tensor(rn, dtype=torch.float64)).sum().backward()
+    tol = RED_RTOL * math.sqrt(cols)
+    assert_close(got_y.data, yt.detach().numpy().reshape(-1), tol, "y")
+    assert_close(got_dx.data, xt.grad.numpy().reshape(-1), 4 * tol, "dx")
