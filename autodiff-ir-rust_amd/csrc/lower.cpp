@@ -1175,6 +1175,49 @@ struct Lowerer {
         std::vector<GK> gks(groups.size());
         // reads per group, with "identity only" flags, for hazard analysis
         std::vector<std::map<Node*, bool>> greads(groups.size());
+        // The element-wise group that can run as the epilogue of group g, whose result P has n_elems elements: the
+        // first later group that reads P, provided it is element-wise over n_elems, reads P element for element only,
+        // and may be moved up to g's position: everything else it reads exists before g runs, and no group in between
+        // reads the old contents of a buffer it overwrites in place.  -1 if there is none.
+        auto reads_node = [&](const Group& H, Node* what) {
+            std::vector<Node*> rs = H.members;
+            for (Node* sd : H.side) rs.push_back(sd);
+            for (Node* ep : H.epi) rs.push_back(ep);
+            for (Node* m : rs)
+                if (reads[m].count(what)) return true;
+            for (auto& cs : H.colsums) {
+                std::map<Node*, bool> er;
+                if (in_mem(cs.first)) er[cs.first] = true;
+                else collect_reads(cs.first, er);
+                if (er.count(what)) return true;
+            }
+            return false;
+        };
+        auto find_epilogue = [&](size_t g, Node* P, int64_t n_elems) -> int {
+            for (size_t ge = g + 1; ge < groups.size(); ++ge) {
+                Group& E = groups[ge];
+                if (E.dead) continue;
+                if (!reads_node(E, P)) continue;
+                if (E.kind != Group::ELW || !E.colsums.empty() || E.n != n_elems) return -1;
+                for (Node* m : E.members) {
+                    auto it = reads[m].find(P);
+                    if (it != reads[m].end() && !it->second) return -1;
+                    for (auto& rd : reads[m]) {
+                        if (rd.first == P) continue;
+                        auto gi = group_of.find(rd.first);
+                        if (gi != group_of.end() && gi->second >= (int)g && gi->second != (int)ge) return -1;
+                    }
+                    auto ho = home_of_early.find(m);
+                    if (ho == home_of_early.end()) continue;
+                    auto li = livein.find(ho->second);
+                    if (li == livein.end()) continue;
+                    for (size_t h = g + 1; h < ge; ++h)
+                        if (!groups[h].dead && reads_node(groups[h], li->second)) return -1;
+                }
+                return (int)ge;
+            }
+            return -1;
+        };
         for (size_t g = 0; g < groups.size(); ++g) {
             Group& G = groups[g];
             if (G.dead) continue;
@@ -1218,24 +1261,15 @@ struct Lowerer {
                 // reference's DotProd + ELW fusion, src/kernel/fusion/dp_elw.rs:13-149); the product itself is
                 // written only if something else still reads it
                 Node* D = G.members[0];
-                size_t nx = g + 1;
-                while (nx < groups.size() && groups[nx].dead) ++nx;
                 DotLaunchPlan dpl;
                 if (dot_uses_mfma(D)) dpl = plan_dot(D);
+                const int nx = (dpl.splits > 1 || !opt.fuse || !dot_uses_mfma(D)) ? -1 : find_epilogue(g, D, numel(D->shape));
                 if (dpl.splits > 1) {
                     Node* partial = new_node(Op::COPY, Shape{dpl.splits, numel(D->shape)}, {}, D->name + ".slices", 0.f, false);
                     partial->root = true;
                     gks[g].extra_nodes.push_back(partial);
-                } else if (opt.fuse && dot_uses_mfma(D) && nx < groups.size() && groups[nx].kind == Group::ELW &&
-                    groups[nx].colsums.empty() && groups[nx].n == numel(D->shape)) {
-                    bool uses = false, ok = true;
-                    for (Node* m : groups[nx].members) {
-                        auto it = reads[m].find(D);
-                        if (it == reads[m].end()) continue;
-                        uses = true;
-                        ok = ok && it->second;
-                    }
-                    if (uses && ok) {
+                } else if (nx >= 0) {
+                    {
                         gks[g].dot_epi = gen_dot_epilogue(D, groups[nx].members);
                         G.epi = groups[nx].members;
                         groups[nx].dead = true;
@@ -1277,23 +1311,8 @@ struct Lowerer {
                 // the element-wise group scheduled right after this reduction, if all it needs from it is the result
                 // element for element, becomes the reduction's epilogue (the reference's Reduce + ELW fusion,
                 // src/kernel/fusion/reduce_elw.rs:12-143)
-                int ge = -1;
-                if (opt.fuse) {
-                    Node* S = G.members[0];
-                    size_t nx = g + 1;
-                    while (nx < groups.size() && groups[nx].dead) ++nx;
-                    if (nx < groups.size() && groups[nx].kind == Group::ELW && groups[nx].colsums.empty() &&
-                        groups[nx].n == numel(S->shape)) {
-                        bool uses = false, ok = true;
-                        for (Node* m : groups[nx].members) {
-                            auto it = reads[m].find(S);
-                            if (it == reads[m].end()) continue;
-                            uses = true;
-                            ok = ok && it->second;
-                        }
-                        if (uses && ok) { ge = (int)nx; spec.epilogue_outputs = groups[nx].members; }
-                    }
-                }
+                const int ge = opt.fuse ? find_epilogue(g, G.members[0], numel(G.members[0]->shape)) : -1;
+                if (ge >= 0) spec.epilogue_outputs = groups[ge].members;
                 gks[g].k = gen_reduce_kernel(spec);
                 ADHIP_CHECK(G.side.empty() || gks[g].k.side_done, "internal: row reduction did not take over its operand's store");
                 if (ge >= 0 && gks[g].k.epilogue_done) {
