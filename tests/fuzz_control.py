@@ -205,3 +205,71 @@ def random_control_program(seed: int):
     keep = sorted(list(g.reals) + list(g.ints) + [f"i{j + 1}" for j in range(g.counters)])
     proc = IR.IRProcedure("main", g.top + main + [IR.EX()])
     return proc, keep, sorted(g.ints)
+
+
+def random_epilogue_program(seed: int):
+    """Straight-line programs around 64x64 matrix products (large enough for the matrix-core kernel) and row sums,
+    with element-wise consumers placed at random distances after their producer and in-place updates of the same
+    tensors in between: the cases in which a consumer may or may not be moved up into its producer's kernel.
+    Returns (procedure, keep list)."""
+    rng = np.random.default_rng(seed)
+    n = 64
+    cmds, mats, vecs = [], [], []
+    for i in range(4):
+        cmds.append(IR.CreateMat((rng.standard_normal(n * n) / 8).astype(np.float32), [n, n], f"m{i}"))
+        mats.append(f"m{i}")
+    for i in range(2):
+        cmds.append(IR.CreateMat(rng.standard_normal(n).astype(np.float32), [n], f"v{i}"))
+        vecs.append(f"v{i}")
+    cnt = [0]
+
+    def fresh(p):
+        cnt[0] += 1
+        return f"{p}{cnt[0]}"
+
+    def const(v, shape):
+        c = fresh("c")
+        cmds.append(IR.CreateConstant(float(v), c, list(shape)))
+        return c
+
+    pending = []   # (kind, producer id) whose consumer has not been emitted yet
+    for _ in range(int(rng.integers(8, 14))):
+        r = int(rng.integers(9))
+        pick = lambda pool: pool[int(rng.integers(len(pool)))]  # noqa: E731
+        if r == 0:      # product
+            d = fresh("d")
+            a, b = pick(mats), pick(mats)
+            if rng.integers(2):
+                t = fresh("t")
+                cmds.append(IR.Permute(a=b, p=[1, 0], res=t))
+                b = t
+            cmds.append(IR.DotProduct(a=a, b=b, res=d))
+            pending.append(("mat", d))
+        elif r == 1:    # row sums
+            s = fresh("s")
+            cmds.append(IR.Sum(a=pick(mats), res=s))
+            pending.append(("vec", s))
+        elif r in (2, 7, 8) and pending:   # consumer of an earlier producer: in-place update of a tensor or a new value
+            kind, p = pending.pop(int(rng.integers(len(pending))))
+            pool, shape = (mats, [n, n]) if kind == "mat" else (vecs, [n])
+            t = fresh("t")
+            cmds.append(IR.ElwMultiply(a=p, b=const(-0.125, shape), res=t))
+            if rng.integers(2):
+                cmds.append(IR.ElwAddEq(s=pick(pool), o=t))
+            else:
+                y = fresh("y")
+                cmds += [IR.ElwAdd(a=t, b=pick(pool), res=y), IR.Sin(a=y, res=pick(pool))]
+        elif r == 3:    # in-place scaling of a matrix (a write between producers and consumers)
+            cmds.append(IR.ElwMultiplyEq(s=pick(mats), o=const(0.5, [n, n])))
+        elif r == 4:    # matrix = matrix + matrix^T
+            t = fresh("t")
+            cmds += [IR.Permute(a=pick(mats), p=[1, 0], res=t), IR.ElwAdd(a=pick(mats), b=t, res=pick(mats))]
+        elif r == 5:    # vector broadcast over a matrix, in place
+            t, w = fresh("t"), fresh("t")
+            cmds += [IR.View(a=pick(vecs), target_dim=[1, n], res=t), IR.Broadcast(a=t, dim=0, r=n, res=w),
+                     IR.ElwAddEq(s=pick(mats), o=w)]
+        else:           # vector update
+            cmds.append(IR.ElwAddEq(s=pick(vecs), o=pick(vecs)))
+            cmds.append(IR.ElwMultiplyEq(s=vecs[0], o=const(0.5, [n])))
+    keep = mats + vecs + [p for _, p in pending]
+    return IR.IRProcedure("main", cmds + [IR.EX()]), keep

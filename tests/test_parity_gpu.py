@@ -444,3 +444,20 @@ def test_product_epilogue_values(m, k, n, keep_p, hip_device):
         # the product never reaches memory; sin amplifies its rounding error by at most 1
         exp_y = np.sin(d) + bias
         assert_close(got["y"].data, exp_y.reshape(-1), tol, "y", scale=scale)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_epilogue_placement_matches_oracle(seed, hip_device):
+    """Matrix-core products and row sums whose element-wise consumers sit at random distances behind them, with
+    in-place updates in between (tests/fuzz_control.py::random_epilogue_program): whatever is or is not fused into
+    the producer's kernel, the values must be the oracle's."""
+    print(f"[case] epilogue fuzz seed {seed}", flush=True)
+    from fuzz_control import random_epilogue_program
+    proc, keep = random_epilogue_program(seed)
+    ref_dev = OracleDevice()
+    ref_dev.execute(proc, set(keep))
+    hip_device.execute(proc, set(keep))
+    for k in keep:
+        got, ref = hip_device.get_tensor(k), ref_dev.get_tensor(k)
+        assert not got.is_none and got.dim == ref.dim, k
+        assert_close(got.data, ref.data, RED_RTOL * 8, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
