@@ -69,9 +69,24 @@ def cpu_baseline_fused_elw(rows, cols):
     t0 = time.perf_counter()
     wl.run()
     dt = time.perf_counter() - t0
-    return {"value": wl.algorithmic_bytes / dt / 1e9, "unit": "GB/s", "cores": int(c_kernels().ref_num_threads()),
-            "kind": "port", "sample": f"fused_elw forward+backward on {rows}x{cols} f32 ({rows}/8192 of the rows), "
-            f"{dt:.2f} s wall", "seconds": dt}
+    out = {"value": wl.algorithmic_bytes / dt / 1e9, "unit": "GB/s", "cores": int(c_kernels().ref_num_threads()),
+           "kind": "port", "sample": f"fused_elw forward+backward on {rows}x{cols} f32 ({rows}/8192 of the rows), "
+           f"{dt:.2f} s wall", "seconds": dt}
+    # the other two rooflines, on bounded samples: configs[2] whole, and one 2048^3 product of configs[3]'s kind
+    import numpy as np
+    from oracle.interp import ref_dot
+    wl3 = W.reductions(OracleDevice(), 16384, 4096, seed=0)
+    t0 = time.perf_counter()
+    wl3.run()
+    dt3 = time.perf_counter() - t0
+    a = np.ones((2048, 2048), dtype=np.float32)
+    t0 = time.perf_counter()
+    ref_dot(a, a)
+    dtd = time.perf_counter() - t0
+    out["other"] = {"reductions_GBps": wl3.algorithmic_bytes / dt3 / 1e9, "reductions_seconds": dt3,
+                    "matmul_GFLOPs": 2.0 * 2048 ** 3 / dtd / 1e9, "matmul_sample": "one 2048x2048x2048 f32 product, "
+                    "one output element per work-item, sequential k", "matmul_seconds": dtd}
+    return out
 
 
 def measure_mlp(dev, iters):
