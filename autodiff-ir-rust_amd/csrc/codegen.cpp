@@ -614,10 +614,9 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     std::vector<Node*> order;
     // no __restrict__ and no unrolling of the row loop: both make the compiler keep two rows of operands live, and
     // the lower occupancy costs more than the earlier loads gain
-    const char* rq = "";
-    for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* %so%zu", rq, i); order.push_back(spec.outputs[i]); }
-    for (size_t i = 0; i < spec.colsums.size(); ++i) { sig += strf(", float* %sq%zu", rq, i); order.push_back(spec.colsums[i].partial); }
-    for (auto& gb : g.bufs) { sig += strf(", const float* %s%s", rq, gb.param.c_str()); order.push_back(gb.node); }
+    for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* o%zu", i); order.push_back(spec.outputs[i]); }
+    for (size_t i = 0; i < spec.colsums.size(); ++i) { sig += strf(", float* q%zu", i); order.push_back(spec.colsums[i].partial); }
+    for (auto& gb : g.bufs) { sig += strf(", const float* %s", gb.param.c_str()); order.push_back(gb.node); }
     const char* it = g.idx_t();
     const char* sfx = wide ? "ull" : "u";
     std::string src = kernel_prelude();

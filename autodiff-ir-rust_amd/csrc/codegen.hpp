@@ -63,12 +63,9 @@ struct GeneratedKernel {
     bool epilogue_done = false;  // the reduction evaluated and stored its epilogue outputs
 };
 
-// `in_memory(n)` tells whether node n's value can be loaded from a buffer in this kernel.
-using InMemoryFn = bool (*)(const Node*, const void*);
-
 GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members);
 // Reduce over the last dim of a [V,R] operand.  If the result needs `chunks > 1`, the kernel writes
-// partial sums laid out [chunks][V]; the caller reduces those with gen_partial_sum_kernel.
+// partial sums laid out [chunks][V]; the caller reduces those with a second (column) reduction over the partials.
 GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks = 0);
 // Number of row tiles an element-wise kernel with column sums over [rows, cols] will use.
 int64_t elw_colsum_tiles(int64_t rows, int64_t cols);
