@@ -28,7 +28,7 @@ const char* adhip_version(void);
  * Replaces OpenCL::new(CLDeviceType) -- reference src/devices/opencl/device.rs:41-58. */
 int adhip_create(int device_ordinal, adhip_ctx** out);
 
-/* Release the context, its compiled kernels and its result buffers. */
+/* Release the context, its compiled kernels, the programs it kept and its result buffers. */
 void adhip_destroy(adhip_ctx* ctx);
 
 /* Message of the last failure on this context (empty string if none).  ctx may be NULL for failures of
@@ -39,7 +39,10 @@ const char* adhip_last_error(adhip_ctx* ctx);
  * `program` is the serialised nested IR procedure (wire format: autodiff-ir-rust_amd/adhip/ir.py and
  * csrc/ir.cpp), ending in EX; `dep_ids` is the keep list (reference src/core/dependency.rs).  Starts from
  * fresh device state, uploads every CreateMat payload (host pointers inside `program` are borrowed until
- * the call returns), runs until the first EX and copies every kept id back to host memory owned by ctx. */
+ * the call returns), runs until the first EX and copies every kept id back to host memory owned by ctx.
+ * The context keeps the plans and device buffers of the last few distinct programs (same command stream and
+ * keep list; payload contents may differ), so executing a program again costs upload + run + read-back only;
+ * ADHIP_EXEC_CACHE=0 in the environment turns that off. */
 int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, const char* const* dep_ids,
                   size_t n_dep_ids);
 
