@@ -261,3 +261,20 @@ def test_no_gpu_means_an_error_not_a_fallback():
     from adhip import HipDevice
     with pytest.raises(RuntimeError):
         HipDevice(0)
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/adhip.h is what a cgo / Rust-bindgen / ctypes user reads: it must compile as C99 on its own, and a C
+    program that only declares and links the entry points must link against the library."""
+    import subprocess
+    hdr = os.path.join(ROOT, "include", "adhip.h")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", hdr], check=True)
+    src = tmp_path / "link.c"
+    src.write_text('#include "adhip.h"\n#include <stdio.h>\nint main(void) { printf("%s\\n", adhip_version()); '
+                   'uint64_t a[2] = {2, 3}, b[2] = {3, 4}, o[2]; return adhip_dot_prod_shape(a, 2, b, 2, o) || o[0] != 2 || o[1] != 4; }\n')
+    exe = tmp_path / "link"
+    libdir = os.path.dirname(library_path())
+    subprocess.run(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe), "-L", libdir,
+                    "-ladhip", "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert out.startswith("adhip")
