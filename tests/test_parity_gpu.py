@@ -461,3 +461,37 @@ def test_random_epilogue_placement_matches_oracle(seed, hip_device):
         got, ref = hip_device.get_tensor(k), ref_dev.get_tensor(k)
         assert not got.is_none and got.dim == ref.dim, k
         assert_close(got.data, ref.data, RED_RTOL * 8, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
+
+
+def test_graph_replay_matches_direct_launches(hip_device, monkeypatch):
+    """A resident program whose launches are replayed as a hipGraph from the third run on: every replay, with uploads
+    and read-backs (eager work and synchronisations) between them, must give exactly what direct launches give, also
+    for a counted loop whose body is replayed once per iteration."""
+    print("[case] graph replay", flush=True)
+    from adhip import HipDevice
+
+    def runs(dev, builder, n):
+        wl = builder(dev)
+        proc, deps = wl.finish()
+        prog = dev.compile(proc, deps)
+        out = []
+        for _ in range(n):
+            prog.upload()
+            prog.run()
+            prog.readback()
+            out.append({k: np.array(dev.get_tensor(v.id).data, copy=True) for k, v in wl.outputs.items()})
+        assert "launch" in prog.describe()
+        prog.close()
+        return out
+
+    builders = [lambda d: W.readme_mlp(d, seed=3), lambda d: W.mlp_train(d, 32, (16, 24, 16, 8), 3)]
+    for builder in builders:
+        with_graphs = runs(hip_device, builder, 6)
+        monkeypatch.setenv("ADHIP_GRAPHS", "0")
+        direct = runs(HipDevice(0), builder, 2)
+        monkeypatch.delenv("ADHIP_GRAPHS")
+        for i, got in enumerate(with_graphs):
+            for k, v in got.items():
+                assert_exact(v, direct[0][k], f"run {i} {k}")
+        for k, v in direct[1].items():
+            assert_exact(v, direct[0][k], f"direct rerun {k}")
