@@ -48,10 +48,39 @@ struct Module {
     }
 };
 
+// A kept tensor on the host.  Small ones live in a vector and arrive through the staging area; large ones live in
+// pinned memory of their own, which the copy engine writes directly (about five times the rate of a copy into
+// pageable memory) and which is kept for the next read-back of the same id.
 struct HostResult {
     std::vector<float> data;
+    float* pinned = nullptr;
+    size_t pinned_elems = 0;
     std::vector<uint64_t> dims;
+    const float* ptr() const { return pinned ? pinned : data.data(); }
+    HostResult() = default;
+    HostResult(const HostResult&) = delete;
+    HostResult& operator=(const HostResult&) = delete;
+    HostResult(HostResult&& o) noexcept { *this = std::move(o); }
+    HostResult& operator=(HostResult&& o) noexcept {
+        if (this != &o) {
+            release();
+            data = std::move(o.data);
+            dims = std::move(o.dims);
+            pinned = o.pinned;
+            pinned_elems = o.pinned_elems;
+            o.pinned = nullptr;
+            o.pinned_elems = 0;
+        }
+        return *this;
+    }
+    void release() {
+        if (pinned) (void)hipHostFree(pinned);
+        pinned = nullptr;
+        pinned_elems = 0;
+    }
+    ~HostResult() { release(); }
 };
+constexpr size_t kPinnedResultBytes = size_t(1) << 20;  // results at least this large get pinned memory
 
 }  // namespace
 
@@ -540,12 +569,24 @@ void program_readback(adhip_program* p) {
     for (auto& kv : p->plan->results) {
         HostResult& r = ctx->results[kv.first];
         auto prev = previous.find(kv.first);
-        if (prev != previous.end()) r.data = std::move(prev->second.data);
+        if (prev != previous.end()) r = std::move(prev->second);
+        r.dims.clear();
         for (auto d : kv.second.shape) r.dims.push_back((uint64_t)d);
         const int64_t ne = numel(kv.second.shape);
-        r.data.resize((size_t)ne);
+        const size_t nb = (size_t)std::max<int64_t>(ne, 0) * sizeof(float);
+        if (nb >= kPinnedResultBytes) {
+            if (r.pinned_elems < (size_t)ne) {
+                r.release();
+                HIP_OK(hipHostMalloc((void**)&r.pinned, nb, hipHostMallocDefault));
+                r.pinned_elems = (size_t)ne;
+            }
+            r.data.clear();
+            HIP_OK(hipMemcpyAsync(r.pinned, p->buf_ptr[kv.second.buf], nb, hipMemcpyDeviceToHost, ctx->stream));
+            continue;
+        }
+        r.release();
+        r.data.resize((size_t)std::max<int64_t>(ne, 0));
         if (ne <= 0) continue;
-        const size_t nb = (size_t)ne * sizeof(float);
         if (nb <= kStageMaxItem) {
             if (used + nb > kStageBytes) drain();
             HIP_OK(hipMemcpyAsync(ctx->stage + used, p->buf_ptr[kv.second.buf], nb, hipMemcpyDeviceToHost, ctx->stream));
@@ -716,7 +757,7 @@ int adhip_get_tensor(adhip_ctx* ctx, const char* id, const float** data, const u
     if (!ctx || !id || !data || !dims || !ndim) return 2;
     auto it = ctx->results.find(id);
     if (it == ctx->results.end()) return 1;
-    *data = it->second.data.data();
+    *data = it->second.ptr();
     *dims = it->second.dims.data();
     *ndim = it->second.dims.size();
     return 0;
