@@ -222,6 +222,14 @@ std::shared_ptr<Module> compile_module(adhip_ctx* ctx, const std::string& source
     std::vector<char> code = compile_code_object(source, ctx->arch);
     auto m = std::make_shared<Module>();
     HIP_OK(hipModuleLoadData(&m->mod, code.data()));
+    // a long-lived context that keeps seeing new programs does not keep every module it ever loaded: beyond a
+    // bound, the ones no live program refers to are unloaded (their code objects stay in the on-disk cache)
+    if (ctx->modules.size() >= 1024) {
+        for (auto it2 = ctx->modules.begin(); it2 != ctx->modules.end();) {
+            if (it2->second.use_count() == 1) it2 = ctx->modules.erase(it2);
+            else ++it2;
+        }
+    }
     ctx->modules[source] = m;
     return m;
 }
