@@ -10,9 +10,11 @@
 #include <hip/hip_ext.h>
 #include <hip/hiprtc.h>
 
+#include <dirent.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <cerrno>
 #include <cmath>
 #include <cstring>
@@ -165,23 +167,62 @@ std::string cache_path(const std::string& source, const std::string& arch_name) 
 
 std::vector<char> compile_code_object_uncached(const std::string& source, const std::string& arch_name);
 
+// Once per process, when the cache directory holds more than `limit` entries, the older half (by modification
+// time) is removed: a cache nobody ever empties would otherwise grow with every program the machine has seen.
+void prune_cache_dir(const std::string& file_in_dir, size_t limit = 8192) {
+    static bool done = false;
+    if (done) return;
+    done = true;
+    const size_t slash = file_in_dir.rfind('/');
+    if (slash == std::string::npos) return;
+    const std::string dir = file_in_dir.substr(0, slash);
+    DIR* d = opendir(dir.c_str());
+    if (!d) return;
+    std::vector<std::pair<time_t, std::string>> entries;
+    while (dirent* e = readdir(d)) {
+        const std::string name = e->d_name;
+        if (name.size() < 7 || name.compare(name.size() - 6, 6, ".hsaco") != 0) continue;
+        struct stat st;
+        const std::string path = dir + "/" + name;
+        if (stat(path.c_str(), &st) == 0) entries.push_back({st.st_mtime, path});
+    }
+    closedir(d);
+    if (entries.size() <= limit) return;
+    std::sort(entries.begin(), entries.end());
+    for (size_t i = 0; i < entries.size() / 2; ++i) remove(entries[i].second.c_str());
+}
+
+// Cache file: "ADHC1\n", the source length, the source text, then the code object.  The source is stored so that a
+// hit is only taken when the text matches: the file name is a 64-bit hash, and a collision must not load the wrong
+// kernel.
 std::vector<char> compile_code_object(const std::string& source, const std::string& arch_name) {
     const std::string path = cache_path(source, arch_name);
+    static const char kMagic[6] = {'A', 'D', 'H', 'C', '1', '\n'};
     if (!path.empty()) {
         if (FILE* f = fopen(path.c_str(), "rb")) {
-            std::vector<char> code;
+            std::vector<char> blob;
             char buf[65536];
             size_t n;
-            while ((n = fread(buf, 1, sizeof buf, f)) > 0) code.insert(code.end(), buf, buf + n);
+            while ((n = fread(buf, 1, sizeof buf, f)) > 0) blob.insert(blob.end(), buf, buf + n);
             fclose(f);
-            if (code.size() > 64) return code;
+            const size_t head = sizeof kMagic + sizeof(uint64_t);
+            if (blob.size() > head && memcmp(blob.data(), kMagic, sizeof kMagic) == 0) {
+                uint64_t sl = 0;
+                memcpy(&sl, blob.data() + sizeof kMagic, sizeof sl);
+                if (sl == source.size() && blob.size() > head + sl + 64 && memcmp(blob.data() + head, source.data(), sl) == 0)
+                    return std::vector<char>(blob.begin() + (long)(head + sl), blob.end());
+            }
         }
     }
     std::vector<char> code = compile_code_object_uncached(source, arch_name);
     if (!path.empty()) {
+        prune_cache_dir(path);
         std::string tmp = path + strf(".tmp%d", (int)getpid());
         if (FILE* f = fopen(tmp.c_str(), "wb")) {
-            const bool ok = fwrite(code.data(), 1, code.size(), f) == code.size();
+            const uint64_t sl = source.size();
+            bool ok = fwrite(kMagic, 1, sizeof kMagic, f) == sizeof kMagic && fwrite(&sl, 1, sizeof sl, f) == sizeof sl &&
+                      fwrite(source.data(), 1, source.size(), f) == source.size() &&
+                      fwrite(code.data(), 1, code.size(), f) == code.size();
             fclose(f);
             if (ok) rename(tmp.c_str(), path.c_str());
             else remove(tmp.c_str());

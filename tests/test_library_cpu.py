@@ -278,3 +278,25 @@ def test_header_is_plain_c(tmp_path):
                     "-ladhip", "-Wl,-rpath," + libdir], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
     assert out.startswith("adhip")
+
+
+def test_code_object_cache_checks_the_source(tmp_path, monkeypatch):
+    """A cache entry holds the source it was compiled from; a file whose stored source differs (a hash collision, a
+    damaged file) is ignored and rewritten, never loaded."""
+    import numpy as np
+    monkeypatch.setenv("ADHIP_CACHE_DIR", str(tmp_path))
+    proc = IR.IRProcedure("main", [IR.CreateMat(np.zeros(8, np.float32), [2, 4], "a"), IR.Sin(a="a", res="s"), IR.EX()])
+    rc, msg = _compile_check(proc, {"s"})
+    assert rc == 0, msg
+    files = [f for f in os.listdir(tmp_path) if f.endswith(".hsaco")]
+    assert len(files) == 1
+    path = os.path.join(tmp_path, files[0])
+    blob = open(path, "rb").read()
+    assert blob.startswith(b"ADHC1\n") and b"adhip_sinf" in blob
+    good_size = len(blob)
+    # damage the stored source (same length): the entry must be treated as a miss and replaced by a good one
+    damaged = blob.replace(b"adhip_sinf", b"adhip_sinX", 1)
+    open(path, "wb").write(damaged)
+    rc, msg = _compile_check(proc, {"s"})
+    assert rc == 0, msg
+    assert open(path, "rb").read() == blob and len(blob) == good_size
