@@ -15,6 +15,8 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <thread>
+#include <atomic>
 #include <cerrno>
 #include <cmath>
 #include <cstring>
@@ -170,9 +172,8 @@ std::vector<char> compile_code_object_uncached(const std::string& source, const 
 // Once per process, when the cache directory holds more than `limit` entries, the older half (by modification
 // time) is removed: a cache nobody ever empties would otherwise grow with every program the machine has seen.
 void prune_cache_dir(const std::string& file_in_dir, size_t limit = 8192) {
-    static bool done = false;
-    if (done) return;
-    done = true;
+    static std::atomic<bool> done{false};
+    if (done.exchange(true)) return;
     const size_t slash = file_in_dir.rfind('/');
     if (slash == std::string::npos) return;
     const std::string dir = file_in_dir.substr(0, slash);
@@ -257,10 +258,46 @@ std::vector<char> compile_code_object_uncached(const std::string& source, const 
     return code;
 }
 
-std::shared_ptr<Module> compile_module(adhip_ctx* ctx, const std::string& source) {
+// Code objects of several sources at once: hipRTC takes a few hundred milliseconds per kernel and a program can
+// have dozens of them, so the ones that are not cached are compiled on several host threads
+// (ADHIP_COMPILE_THREADS, default 8; 1 compiles one after the other).
+std::map<std::string, std::vector<char>> compile_code_objects(const std::vector<std::string>& sources, const std::string& arch) {
+    std::map<std::string, std::vector<char>> out;
+    std::vector<const std::string*> todo;
+    for (const std::string& src : sources)
+        if (out.emplace(src, std::vector<char>()).second) todo.push_back(&out.find(src)->first);
+    int threads = 8;
+    if (const char* e = getenv("ADHIP_COMPILE_THREADS")) threads = std::max(1, atoi(e));
+    threads = (int)std::min<size_t>((size_t)threads, todo.size());
+    if (threads <= 1) {
+        for (const std::string* src : todo) out[*src] = compile_code_object(*src, arch);
+        return out;
+    }
+    std::atomic<size_t> next{0};
+    std::vector<std::string> errors((size_t)threads);
+    std::vector<std::thread> pool;
+    for (int t = 0; t < threads; ++t)
+        pool.emplace_back([&, t] {
+            try {
+                for (size_t i = next.fetch_add(1); i < todo.size(); i = next.fetch_add(1)) {
+                    std::vector<char> code = compile_code_object(*todo[i], arch);
+                    out.find(*todo[i])->second = std::move(code);   // distinct keys: no two threads touch one entry
+                }
+            } catch (const std::exception& e) {
+                errors[(size_t)t] = e.what();
+                next.store(todo.size());
+            }
+        });
+    for (auto& th : pool) th.join();
+    for (auto& e : errors)
+        if (!e.empty()) throw Error(e);
+    return out;
+}
+
+std::shared_ptr<Module> compile_module(adhip_ctx* ctx, const std::string& source, const std::vector<char>* code_in = nullptr) {
     auto it = ctx->modules.find(source);
     if (it != ctx->modules.end()) return it->second;
-    std::vector<char> code = compile_code_object(source, ctx->arch);
+    std::vector<char> code = code_in ? *code_in : compile_code_object(source, ctx->arch);
     auto m = std::make_shared<Module>();
     HIP_OK(hipModuleLoadData(&m->mod, code.data()));
     // a long-lived context that keeps seeing new programs does not keep every module it ever loaded: beyond a
@@ -313,9 +350,14 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
     p->plan = lower_program(*p->ir, dep_vector(dep_ids, n));
     Plan& plan = *p->plan;
     try {
-        // kernels
+        // kernels: what the context has not loaded yet is compiled (or fetched from the disk cache) in parallel
+        std::vector<std::string> missing;
+        for (const KernelDef& k : plan.kernels)
+            if (!ctx->modules.count(k.source)) missing.push_back(k.source);
+        std::map<std::string, std::vector<char>> fresh = compile_code_objects(missing, ctx->arch);
         for (const KernelDef& k : plan.kernels) {
-            auto m = compile_module(ctx, k.source);
+            auto f = fresh.find(k.source);
+            auto m = compile_module(ctx, k.source, f != fresh.end() ? &f->second : nullptr);
             p->mods.push_back(m);
             p->fn.push_back(get_function(*m, k.entry));
         }
@@ -903,8 +945,11 @@ int adhip_compile_check(const uint8_t* program, size_t program_len, const char* 
         auto plan = lower_program(*ir, dep_vector(dep_ids, n_dep_ids));
         size_t bytes = 0;
         const char* dump_dir = getenv("ADHIP_DUMP_CODE_DIR");
+        std::vector<std::string> sources;
+        for (auto& k : plan->kernels) sources.push_back(k.source);
+        std::map<std::string, std::vector<char>> objects = compile_code_objects(sources, arch && *arch ? arch : "gfx950");
         for (auto& k : plan->kernels) {
-            std::vector<char> code = compile_code_object(k.source, arch && *arch ? arch : "gfx950");
+            const std::vector<char>& code = objects[k.source];
             bytes += code.size();
             if (dump_dir && *dump_dir) {
                 std::string base = std::string(dump_dir) + "/" + k.entry;
