@@ -316,12 +316,17 @@ def test_single_ops_per_element(hip_device):
         IR.EqualZero(a="z", res="eq"), IR.MoreZero(a="z", res="gt"), IR.LessZero(a="z", res="lt"),
         IR.Exp2(a="a", res="exp2"), IR.Log2(a="p", res="log2"), IR.Sin(a="a", res="sin"),
     ]
-    keep = ["add", "mul", "ia", "im", "rcp", "sqrt", "eq", "gt", "lt", "exp2", "log2", "sin"]
+    # arguments far outside the fast range of the kernels' sine (it hands over to the library routine beyond 2^15),
+    # with the hand-over point itself and a few values next to multiples of pi
+    big = rng.uniform(-3.0e6, 3.0e6, n).astype(np.float32)
+    big[:8] = [32768.0, -32768.0, np.nextafter(np.float32(32768), np.float32(1e9)), 32767.998, 3.1415927, 6.2831855, 31415.926, 314159.27]
+    cmds += [IR.CreateMat(big, [64, 1024], "big"), IR.Sin(a="big", res="sin_big")]
+    keep = ["add", "mul", "ia", "im", "rcp", "sqrt", "eq", "gt", "lt", "exp2", "log2", "sin", "sin_big"]
     got = _run_ir(hip_device, cmds, keep)
     ref = _run_ir(OracleDevice(), cmds, keep)
     for k in ["add", "mul", "ia", "im", "rcp", "sqrt", "eq", "gt", "lt"]:
         assert_exact(got[k].data, ref[k].data, k)
-    for k in ["exp2", "log2", "sin"]:
+    for k in ["exp2", "log2", "sin", "sin_big"]:
         g = got[k].data.astype(np.float64)
         r = ref[k].data.astype(np.float64)
         rel = np.abs(g - r) / np.maximum(np.abs(r), 1e-30)
