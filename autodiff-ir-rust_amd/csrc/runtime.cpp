@@ -784,13 +784,13 @@ int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, co
                 for (size_t a = 0; ok && a < ptrs.size(); ++a)
                     for (size_t b = a + 1; ok && b < ptrs.size(); ++b)
                         if (q->payloads[a] == q->payloads[b] && ptrs[a] != ptrs[b]) ok = false;
-                auto entry = ctx->exec_cache[i];
+                auto entry = std::move(ctx->exec_cache[i]);
                 ctx->exec_cache.erase(ctx->exec_cache.begin() + (long)i);
                 if (ok) {
                     for (size_t bi = 0; bi < q->plan->buffers.size(); ++bi)
                         if (q->payload_of[bi] >= 0) q->plan->buffers[bi].host = ptrs[(size_t)q->payload_of[bi]];
                     q->payloads = ptrs;
-                    ctx->exec_cache.insert(ctx->exec_cache.begin(), entry);
+                    ctx->exec_cache.insert(ctx->exec_cache.begin(), std::move(entry));
                     p = q;
                 } else {
                     program_free(q);
