@@ -632,11 +632,12 @@ void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
     }
 }
 
-void program_run(adhip_program* p) {
+void program_run(adhip_program* p, bool wait = true) {
     adhip_ctx* ctx = p->ctx;
     HIP_OK(hipSetDevice(ctx->device));
     p->exited = false;
     exec_steps(p, p->plan->steps);
+    if (!wait) return;
     HIP_OK(hipStreamSynchronize(ctx->stream));
     if (p->profiling) drain_events(p);
 }
@@ -876,6 +877,20 @@ int adhip_program_upload(adhip_program* p) {
 int adhip_program_run(adhip_program* p) {
     if (!p) return 2;
     return guarded(p->ctx, [&] { program_run(p); });
+}
+
+int adhip_program_enqueue(adhip_program* p) {
+    if (!p) return 2;
+    return guarded(p->ctx, [&] { program_run(p, false); });
+}
+
+int adhip_program_sync(adhip_program* p) {
+    if (!p) return 2;
+    return guarded(p->ctx, [&] {
+        HIP_OK(hipSetDevice(p->ctx->device));
+        HIP_OK(hipStreamSynchronize(p->ctx->stream));
+        if (p->profiling) drain_events(p);
+    });
 }
 
 int adhip_program_readback(adhip_program* p) {

@@ -27,11 +27,14 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 
 
 def timed_runs(prog, steps, warmup):
+    """`steps` runs queued back to back on the device's stream, bracketed by a wait on both sides."""
     for _ in range(warmup):
         prog.run()
+    prog.sync()
     t0 = time.perf_counter()
     for _ in range(steps):
-        prog.run()
+        prog.enqueue()
+    prog.sync()
     t1 = time.perf_counter()
     return (t1 - t0) * 1e3 / steps
 

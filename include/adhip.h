@@ -66,6 +66,11 @@ int adhip_program_create(adhip_ctx* ctx, const uint8_t* program, size_t program_
 int adhip_program_upload(adhip_program* p);
 /* Run from the current device state to the first EX; returns after the stream has drained. */
 int adhip_program_run(adhip_program* p);
+/* The same without the final wait: the kernels are queued on the context's stream and the call returns (a loop or
+ * branch that the host has to decide still waits for its predicate).  Several runs can be queued back to back;
+ * adhip_program_sync waits for all of them and must be called before upload, read-back or destroy. */
+int adhip_program_enqueue(adhip_program* p);
+int adhip_program_sync(adhip_program* p);
 /* Copy kept ids to host memory owned by the context (then served by adhip_get_tensor). */
 int adhip_program_readback(adhip_program* p);
 void adhip_program_destroy(adhip_program* p);

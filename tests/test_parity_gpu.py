@@ -500,3 +500,26 @@ def test_graph_replay_matches_direct_launches(hip_device, monkeypatch):
                 assert_exact(v, direct[0][k], f"run {i} {k}")
         for k, v in direct[1].items():
             assert_exact(v, direct[0][k], f"direct rerun {k}")
+
+
+def test_enqueue_and_sync(hip_device):
+    """Runs queued back to back without waiting in between behave like the same number of waited-for runs: an in-place
+    update (x += 1 followed by a row sum) accumulates once per queued run."""
+    print("[case] enqueue / sync", flush=True)
+    from adhip import ir as IR
+    x0 = np.arange(12, dtype=np.float32)
+    cmds = [IR.CreateMat(x0, [3, 4], "x"), IR.CreateConstant(1.0, "one", [3, 4]), IR.ElwAddEq(s="x", o="one"),
+            IR.Sum(a="x", res="s"), IR.EX()]
+    prog = hip_device.compile(IR.IRProcedure("main", cmds), {"x", "s"})
+    prog.upload()
+    prog.run()
+    prog.readback()
+    assert_exact(hip_device.get_tensor("x").data, x0 + 1, "one waited-for run")
+    for _ in range(4):
+        prog.enqueue()
+    prog.sync()
+    prog.readback()
+    # the top-level CreateMat is an upload, not a kernel: it is not repeated by a run
+    assert_exact(hip_device.get_tensor("x").data, x0 + 5, "four queued runs after one waited-for run")
+    assert_exact(hip_device.get_tensor("s").data, (x0 + 5).reshape(3, 4).sum(1), "row sums of the last run")
+    prog.close()
