@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the device path on one MI355X.
 
-A step is one pass of the hot path (`adhip_program_run`: every kernel of the lowered program, to
-EX) over one batch of synthetic input that is already resident in HBM.  The headline workload is
+A step is one pass of the hot path (every kernel of the lowered program, to EX) over one batch of
+synthetic input that is already resident in HBM; the timed steps are queued back to back on the
+device's stream (`adhip_program_enqueue`) between two waits (`adhip_program_sync`).  The headline workload is
 BASELINE.json configs[1]: fused element-wise + broadcast, forward and backward, 8192x8192 f32.
 The other configs are measured too (shorter) and reported under "extra".
 
