@@ -34,10 +34,11 @@ std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry, 
     s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n#define SPLITK %d\n", cfg.a_kcontig ? 1 : 0,
               cfg.b_kcontig ? 1 : 0, cfg.edge ? 1 : 0, cfg.split_k ? 1 : 0);
     // tile geometry: BM x BN block tile, TM x TN MFMA blocks per wave, WGN waves along n
-    const int tm = cfg.bm == 64 ? 1 : 2, bn = cfg.bm == 64 ? 64 : 128;
-    const int waves = (cfg.bm / (32 * tm)) * (bn / (32 * tm));
+    const int bn = cfg.bn ? cfg.bn : (cfg.bm == 64 ? 64 : 128);
+    const int tm = cfg.bm == 64 ? 1 : 2, tn = (bn == 64) ? 1 : 2;
+    const int waves = (cfg.bm / (32 * tm)) * (bn / (32 * tn));
     s += strf("#define KERNEL_NAME %s\n#define BM %d\n#define BN %d\n#define TM %d\n#define TN %d\n#define NT %d\n", entry.c_str(),
-              cfg.bm, bn, tm, tm, waves * 64);
+              cfg.bm, bn, tm, tn, waves * 64);
     s += R"(
 #define BK 16
 #define LDA (BM + 4)

@@ -1593,6 +1593,8 @@ struct Lowerer {
         else if (blocks128 * splits_for(blocks128) >= 256) cfg.bm = 128;
         else cfg.bm = 64;
         pl.bn_tile = cfg.bm == 64 ? 64 : 128;
+        // one 128x128 block per CU is too few to hide its own latencies: halve the tile's width for two per CU
+        if (cfg.bm == 128 && blocks128 < 512 && splits_for(blocks128) == 1) { pl.bn_tile = 64; cfg.bn = 64; }
         cfg.edge = unaligned || (M % cfg.bm) || (N % pl.bn_tile);
         const int64_t blocks = ((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile);
         const int64_t want = cfg.bm == 256 ? 1 : splits_for(blocks);
@@ -1620,8 +1622,8 @@ struct Lowerer {
             GemmConfig cfg = pl.cfg;
             const int bn_tile = pl.bn_tile;
             ADHIP_CHECK(!cfg.split_k || (partial && !epi), "internal: split product without its slice buffer");
-            std::string entry = strf("adhip_gemm_%c%c_%d%s%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
-                                     cfg.edge ? "_edge" : "", cfg.split_k ? "_splitk" : "");
+            std::string entry = strf("adhip_gemm_%c%c_%d%s%s%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
+                                     cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? "_edge" : "", cfg.split_k ? "_splitk" : "");
             Launch l;
             if (epi) {
                 // the element-wise group that followed the product runs on the accumulators; every distinct

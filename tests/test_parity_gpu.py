@@ -280,10 +280,10 @@ def test_shape_errors_are_reported(hip_device):
             hip_device.execute(proc, {"a"})
 
 
-@pytest.mark.parametrize("m,k,n", [(2048, 256, 4096), (1024, 64, 8192)])
+@pytest.mark.parametrize("m,k,n", [(2048, 256, 4096), (1024, 64, 8192), (2048, 64, 2048), (2000, 48, 2100)])
 def test_dot_large_tile_variant(m, k, n, hip_device):
-    """Shapes that select the 128x128 block tile of the MFMA kernel (the small shapes above take the 64x64 tile, the
-    full-size MLP test the 256x128 one), all three operand layouts."""
+    """Shapes that select the 128x128 and 128x64 block tiles of the MFMA kernel (the small shapes above take the 64x64
+    tile, the full-size MLP test the 256x128 one), all three operand layouts, aligned and bounds-checked."""
     test_dot_forward_backward(m, k, n, hip_device)
 
 
