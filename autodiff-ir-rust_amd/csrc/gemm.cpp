@@ -31,8 +31,17 @@ std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry, 
         }
         s += m + "\n";
     }
-    s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n#define SPLITK %d\n", cfg.a_kcontig ? 1 : 0,
-              cfg.b_kcontig ? 1 : 0, cfg.edge ? 1 : 0, cfg.split_k ? 1 : 0);
+    s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n#define SPLITK %d\n#define GROUPED %d\n", cfg.a_kcontig ? 1 : 0,
+              cfg.b_kcontig ? 1 : 0, cfg.edge ? 1 : 0, cfg.split_k ? 1 : 0, cfg.grouped ? 1 : 0);
+    if (cfg.grouped) {
+        // one parameter triple per problem slot, and the (wave-uniform) choice among them by blockIdx.y
+        std::string params, pick = "switch (blockIdx.y) {";
+        for (int i = 0; i < kGemmGroupSlots; ++i) {
+            params += strf("float* c%d, const float* a%d, const float* b%d, ", i, i, i);
+            pick += strf(" case %d: C = c%d; A = a%d; B = b%d; break;", i, i, i, i);
+        }
+        s += "#define GROUP_PARAMS " + params + "\n#define GROUP_PICK " + pick + " default: return; }\n";
+    }
     // tile geometry: BM x BN block tile, TM x TN MFMA blocks per wave, WGN waves along n
     const int bn = cfg.bn ? cfg.bn : (cfg.bm == 64 ? 64 : 128);
     const int tm = cfg.bm == 64 ? 1 : 2, tn = (bn == 64) ? 1 : 2;
@@ -56,7 +65,21 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 // SPLITK: the block at blockIdx.y multiplies only k in [y*k_chunk, (y+1)*k_chunk) and writes slice y of a
 // [gridDim.y][M][N] buffer; the caller adds the slices in a fixed order.  For products whose output alone gives
 // too few blocks to hide the latency of the operand loads.
+// GROUPED: several independent products of one shape and one set of strides in a single launch; the block row
+// blockIdx.y works on problem y, whose three base pointers (operand offsets already applied) are parameters
+// c<y>, a<y>, b<y>.  For the same kind of product when there are many of them (the per-head projections of
+// multi-head attention), instead of cutting k.
 extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
+#if GROUPED
+    const int* __restrict__ guard, GROUP_PARAMS long long M, long long N, long long K, long long a_sm, long long a_sk,
+    long long b_sk, long long b_sn) {
+    if (guard && *guard == 0) return;
+    float* __restrict__ C;
+    const float* __restrict__ A;
+    const float* __restrict__ B;
+    GROUP_PICK
+    const long long a_off = 0, b_off = 0;
+#else
     const int* __restrict__ guard, float* __restrict__ C, const float* __restrict__ A, const float* __restrict__ B,
     long long M, long long N, long long K, long long a_off, long long a_sm, long long a_sk, long long b_off,
     long long b_sk, long long b_sn
@@ -65,6 +88,7 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
 #endif
     EPI_PARAMS) {
     if (guard && *guard == 0) return;
+#endif
 #if SPLITK
     const long long k_lo = (long long)blockIdx.y * k_chunk;
     const long long k_hi = min(K, k_lo + k_chunk);

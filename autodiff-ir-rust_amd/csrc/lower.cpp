@@ -1,6 +1,7 @@
 #include "lower.hpp"
 
 #include <algorithm>
+#include <array>
 #include <cctype>
 #include <cmath>
 #include <cstring>
@@ -1162,23 +1163,8 @@ struct Lowerer {
                 group_of[E] = (int)gs;
             }
         }
-        // ---- 6. generate code per group (no buffers needed yet)
         std::map<Node*, std::string> home_of_early;
         for (auto& w : wanted) home_of_early[w.second] = w.first;
-        struct GK {
-            GeneratedKernel k;
-            std::vector<GeneratedKernel> extra;
-            std::vector<Node*> extra_nodes;
-            DotEpilogueCode dot_epi;   // DOT groups with an epilogue
-            bool dot_store = true;     // ... and whether the product itself is still written
-        };
-        std::vector<GK> gks(groups.size());
-        // reads per group, with "identity only" flags, for hazard analysis
-        std::vector<std::map<Node*, bool>> greads(groups.size());
-        // The element-wise group that can run as the epilogue of group g, whose result P has n_elems elements: the
-        // first later group that reads P, provided it is element-wise over n_elems, reads P element for element only,
-        // and may be moved up to g's position: everything else it reads exists before g runs, and no group in between
-        // reads the old contents of a buffer it overwrites in place.  -1 if there is none.
         auto reads_node = [&](const Group& H, Node* what) {
             std::vector<Node*> rs = H.members;
             for (Node* sd : H.side) rs.push_back(sd);
@@ -1193,6 +1179,29 @@ struct Lowerer {
             }
             return false;
         };
+        // ---- 5d. matrix-core products of one shape that each fill only part of the chip and do not depend on one
+        // another (the per-head projections, scores and weighted values of multi-head attention, and their
+        // gradients) become one grouped launch.  Products are independent when they sit at the same depth, counted
+        // in products along the longest chain of dependencies; ordering the kernels by that depth, products last
+        // within a depth, puts everything such a set reads before all of it and everything that reads it after.
+        // Dependencies are the values a kernel reads plus, for a kernel that overwrites an id's buffer, the earlier
+        // kernels that still read the id's old contents.  Regions without such a set keep program order.
+        if (opt.fuse && opt.group_dots) group_products(groups, group_of, reads, home_of_early, reads_node);
+        // ---- 6. generate code per group (no buffers needed yet)
+        struct GK {
+            GeneratedKernel k;
+            std::vector<GeneratedKernel> extra;
+            std::vector<Node*> extra_nodes;
+            DotEpilogueCode dot_epi;   // DOT groups with an epilogue
+            bool dot_store = true;     // ... and whether the product itself is still written
+        };
+        std::vector<GK> gks(groups.size());
+        // reads per group, with "identity only" flags, for hazard analysis
+        std::vector<std::map<Node*, bool>> greads(groups.size());
+        // The element-wise group that can run as the epilogue of group g, whose result P has n_elems elements: the
+        // first later group that reads P, provided it is element-wise over n_elems, reads P element for element only,
+        // and may be moved up to g's position: everything else it reads exists before g runs, and no group in between
+        // reads the old contents of a buffer it overwrites in place.  -1 if there is none.
         auto find_epilogue = [&](size_t g, Node* P, int64_t n_elems) -> int {
             for (size_t ge = g + 1; ge < groups.size(); ++ge) {
                 Group& E = groups[ge];
@@ -1262,8 +1271,19 @@ struct Lowerer {
                 // written only if something else still reads it
                 Node* D = G.members[0];
                 DotLaunchPlan dpl;
-                if (dot_uses_mfma(D)) dpl = plan_dot(D);
-                const int nx = (dpl.splits > 1 || !opt.fuse || !dot_uses_mfma(D)) ? -1 : find_epilogue(g, D, numel(D->shape));
+                const bool grouped = G.members.size() > 1;  // one launch for all of them: whole k, no epilogue
+                if (dot_uses_mfma(D) && !grouped) dpl = plan_dot(D);
+                int nx = (grouped || dpl.splits > 1 || !opt.fuse || !dot_uses_mfma(D)) ? -1 : find_epilogue(g, D, numel(D->shape));
+                if (nx >= 0) {
+                    // an epilogue streams its other operands in the accumulator layout (32 floats of a row per half
+                    // wave); with many of them (a sum over all heads' gradients) a separate element-wise pass, with
+                    // 128-bit accesses, is faster than the product kernel held up by them
+                    std::set<Node*> big;
+                    for (Node* m : groups[nx].members)
+                        for (auto& rd : reads[m])
+                            if (rd.first != D && numel(rd.first->shape) * 2 >= numel(D->shape)) big.insert(rd.first);
+                    if (big.size() > 8) nx = -1;
+                }
                 if (dpl.splits > 1) {
                     Node* partial = new_node(Op::COPY, Shape{dpl.splits, numel(D->shape)}, {}, D->name + ".slices", 0.f, false);
                     partial->root = true;
@@ -1440,7 +1460,8 @@ struct Lowerer {
             Group& G = groups[g];
             if (G.dead) continue;
             if (G.kind == Group::DOT) {
-                if (!G.epi.empty()) emit_dot(G.members[0], out, &gks[g].dot_epi, gks[g].dot_store);
+                if (G.members.size() > 1) emit_dot_group(G.members, out);
+                else if (!G.epi.empty()) emit_dot(G.members[0], out, &gks[g].dot_epi, gks[g].dot_store);
                 else emit_dot(G.members[0], out, nullptr, true, gks[g].extra_nodes.empty() ? nullptr : gks[g].extra_nodes[0]);
                 continue;
             }
@@ -1551,6 +1572,166 @@ struct Lowerer {
         l.label = "transpose_" + n->name;
         l.bytes = 8.0 * (double)numel(st.shape);
         push_launch(out, l, "transpose");
+    }
+
+    // What must agree for products to share a grouped launch: sizes, strides and whether operands are 16-byte
+    // aligned.  False for products that fill the chip on their own or do not go to the matrix cores.
+    static bool dot_group_key(const Node* n, std::array<int64_t, 8>& key) {
+        if (!dot_uses_mfma(n)) return false;
+        Affine2D a, b;
+        tref_affine2d(n->in[0], a);
+        tref_affine2d(n->in[1], b);
+        const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
+        if (((M + 127) / 128) * ((N + 127) / 128) >= 256) return false;
+        const int64_t a_ld = a.s1 == 1 ? a.s0 : a.s1, b_ld = b.s0 == 1 ? b.s1 : b.s0;
+        const bool unaligned = (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
+        key = {M, N, K, a.s0, a.s1, b.s0, b.s1, unaligned ? 1 : 0};
+        return true;
+    }
+
+    template <class ReadsNode>
+    void group_products(std::vector<Group>& groups, std::map<Node*, int>& group_of, std::map<Node*, std::map<Node*, bool>>& reads,
+                        const std::map<Node*, std::string>& home_of_early, ReadsNode&& reads_node) {
+        const int G = (int)groups.size();
+        std::vector<std::array<int64_t, 8>> key(G);
+        std::vector<char> cand(G, 0);
+        int ncand = 0;
+        for (int g = 0; g < G; ++g)
+            if (!groups[g].dead && groups[g].kind == Group::DOT && dot_group_key(groups[g].members[0], key[g])) { cand[g] = 1; ++ncand; }
+        if (ncand < 2) return;
+        // depth of every kernel
+        std::vector<int> level(G, 0);
+        for (int g = 0; g < G; ++g) {
+            Group& H = groups[g];
+            if (H.dead) continue;
+            std::set<int> preds;
+            bool ok = true;
+            auto add_reads = [&](const std::map<Node*, bool>& rd) {
+                for (auto& kv : rd) {
+                    if (op_is_leaf(kv.first->op)) continue;
+                    auto it = group_of.find(kv.first);
+                    if (it == group_of.end() || it->second == g) continue;
+                    if (it->second > g) ok = false;
+                    preds.insert(it->second);
+                }
+            };
+            std::vector<Node*> produced = H.members;
+            for (Node* sd : H.side) produced.push_back(sd);
+            for (Node* m : produced) add_reads(reads[m]);
+            for (auto& cs : H.colsums) {
+                std::map<Node*, bool> er;
+                if (in_mem(cs.first)) er[cs.first] = true;
+                else collect_reads(cs.first, er);
+                add_reads(er);
+                produced.push_back(cs.second);
+            }
+            if (!ok) return;  // not in dependency order as it stands: leave the region alone
+            for (Node* m : produced) {
+                auto ho = home_of_early.find(m);
+                if (ho == home_of_early.end()) continue;
+                auto li = livein.find(ho->second);
+                if (li == livein.end()) continue;
+                for (int r = 0; r < g; ++r)
+                    if (!groups[r].dead && reads_node(groups[r], li->second)) preds.insert(r);
+            }
+            for (int p : preds) level[g] = std::max(level[g], level[p] + (groups[p].kind == Group::DOT ? 1 : 0));
+        }
+        // sets of at least two
+        std::map<std::pair<int, std::array<int64_t, 8>>, std::vector<int>> sets;
+        for (int g = 0; g < G; ++g)
+            if (cand[g]) sets[{level[g], key[g]}].push_back(g);
+        bool any = false;
+        for (auto& kv : sets) any = any || kv.second.size() >= 2;
+        if (!any) return;
+        // new order
+        std::vector<int> order;
+        for (int g = 0; g < G; ++g)
+            if (!groups[g].dead) order.push_back(g);
+        std::stable_sort(order.begin(), order.end(), [&](int x, int y) {
+            if (level[x] != level[y]) return level[x] < level[y];
+            return (groups[x].kind == Group::DOT) < (groups[y].kind == Group::DOT);
+        });
+        std::vector<int> new_index(G, -1);
+        std::vector<Group> sorted;
+        for (int g : order) {
+            new_index[g] = (int)sorted.size();
+            sorted.push_back(groups[g]);
+        }
+        for (auto& kv : group_of) {
+            ADHIP_CHECK(kv.second >= 0 && kv.second < G && new_index[kv.second] >= 0, "internal: value produced by a dropped kernel");
+            kv.second = new_index[kv.second];
+        }
+        groups.swap(sorted);
+        // merge each set into its first member, at most kGemmGroupSlots products per launch, evenly
+        for (auto& kv : sets) {
+            const std::vector<int>& set = kv.second;
+            if (set.size() < 2) continue;
+            const size_t launches = (set.size() + kGemmGroupSlots - 1) / kGemmGroupSlots;
+            const size_t per = (set.size() + launches - 1) / launches;
+            for (size_t i0 = 0; i0 < set.size(); i0 += per) {
+                const size_t i1 = std::min(set.size(), i0 + per);
+                if (i1 - i0 < 2) continue;
+                const int head = new_index[set[i0]];
+                for (size_t i = i0 + 1; i < i1; ++i) {
+                    Group& T = groups[new_index[set[i]]];
+                    groups[head].members.push_back(T.members[0]);
+                    group_of[T.members[0]] = head;
+                    T.dead = true;
+                }
+            }
+        }
+    }
+
+    // One launch for several products of the same shape (see group_products): problem y is block row y.
+    void emit_dot_group(const std::vector<Node*>& dots, std::vector<Step>& out) {
+        const int cnt = (int)dots.size();
+        ADHIP_CHECK(cnt >= 2 && cnt <= kGemmGroupSlots, "internal: grouped product launch of %d products", cnt);
+        std::array<int64_t, 8> key0{};
+        ADHIP_CHECK(dot_group_key(dots[0], key0), "internal: grouped launch of a product that does not qualify");
+        const int64_t M = key0[0], N = key0[1], K = key0[2];
+        GemmConfig cfg;
+        cfg.a_kcontig = key0[4] == 1;
+        cfg.b_kcontig = key0[5] == 1;
+        cfg.grouped = true;
+        // tile by the number of blocks the whole launch has, as for a single product
+        const int64_t blocks128 = ((M + 127) / 128) * ((N + 127) / 128) * cnt;
+        cfg.bm = blocks128 >= 256 ? 128 : 64;
+        int bn_tile = cfg.bm == 64 ? 64 : 128;
+        if (cfg.bm == 128 && blocks128 < 512) { bn_tile = 64; cfg.bn = 64; }
+        cfg.edge = key0[7] || (M % cfg.bm) || (N % bn_tile);
+        std::string entry = strf("adhip_gemm_%c%c_%d%s%s_grouped", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
+                                 cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? "_edge" : "");
+        Launch l;
+        l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
+        l.block[0] = cfg.bm == 64 ? 256u : (unsigned)(cfg.bm * 2);
+        l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + bn_tile - 1) / bn_tile));
+        l.grid[1] = (unsigned)cnt;
+        auto B = [&](Node* x, int64_t off) {
+            Arg q;
+            q.kind = Arg::BUF;
+            ADHIP_CHECK(x->buffer >= 0, "internal: matmul operand without buffer");
+            q.buf = x->buffer;
+            q.off = off;
+            return q;
+        };
+        auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
+        for (int i = 0; i < kGemmGroupSlots; ++i) {
+            Node* n = dots[std::min(i, cnt - 1)];  // unused slots repeat the last problem; no block reads them
+            std::array<int64_t, 8> key{};
+            ADHIP_CHECK(dot_group_key(n, key) && key == key0, "internal: grouped products differ in shape or strides");
+            Affine2D a, b;
+            tref_affine2d(n->in[0], a);
+            tref_affine2d(n->in[1], b);
+            l.args.push_back(B(n, 0));
+            l.args.push_back(B(a.base, a.offset));
+            l.args.push_back(B(b.base, b.offset));
+        }
+        for (int q = 0; q < 3; ++q) l.args.push_back(I(key0[q]));
+        for (int q = 3; q < 7; ++q) l.args.push_back(I(key0[q]));
+        l.label = strf("dots_%s_%dx_%lldx%lldx%lld", dots[0]->name.c_str(), cnt, (long long)M, (long long)N, (long long)K);
+        l.bytes = 4.0 * cnt * ((double)M * K + (double)K * N + (double)M * N);
+        l.flops = 2.0 * cnt * (double)M * (double)N * (double)K;
+        push_launch(out, l, "dot_mfma");
     }
 
     // whether a product goes to the matrix-core kernel (else the one-thread-per-output kernel)
@@ -1906,7 +2087,7 @@ void describe_steps(const std::vector<Step>& steps, const Plan& p, int indent, s
             o += pad + strf("launch %s [%s] grid=(%u,%u,%u) block=%u bytes=%.0f flops=%.0f args:", l.label.c_str(),
                             p.kernels[l.kernel].kind.c_str(), l.grid[0], l.grid[1], l.grid[2], l.block[0], l.bytes, l.flops);
             for (const Arg& a : l.args) {
-                if (a.kind == Arg::BUF) o += " " + p.buffers[a.buf].name + "#" + std::to_string(a.buf);
+                if (a.kind == Arg::BUF) o += " " + p.buffers[a.buf].name + "#" + std::to_string(a.buf) + (a.off ? strf("+%lld", (long long)a.off) : std::string());
                 else if (a.kind == Arg::F32) o += strf(" %g", a.fv);
                 else o += strf(" %lld", (long long)a.iv);
             }
@@ -1952,7 +2133,9 @@ std::string Plan::describe() const {
     return o;
 }
 
-std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids, const LowerOptions& opt) {
+std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids, const LowerOptions& opt_in) {
+    LowerOptions opt = opt_in;
+    if (const char* e = getenv("ADHIP_GROUP_DOTS")) opt.group_dots = opt.group_dots && atoi(e) != 0;
     Lowerer l(prog, dep_ids, opt);
     return l.run();
 }

@@ -14,6 +14,7 @@ namespace adhip {
 
 struct LowerOptions {
     bool fuse = true;  // false: one kernel per compute command (diagnostic mode)
+    bool group_dots = true;  // same-shape independent matrix products that under-fill the chip share a launch
 };
 
 std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids,

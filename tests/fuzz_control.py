@@ -273,3 +273,70 @@ def random_epilogue_program(seed: int):
             cmds.append(IR.ElwMultiplyEq(s=vecs[0], o=const(0.5, [n])))
     keep = mats + vecs + [p for _, p in pending]
     return IR.IRProcedure("main", cmds + [IR.EX()]), keep
+
+
+def random_grouped_products_program(seed: int):
+    """Many independent matrix products of one shape, the way multi-head attention issues them: per-head weights
+    that are slices of one packed tensor (so the operands differ only by an offset), element-wise work between two
+    levels of products, transposed operands, sums over the heads, and a rotation `w[h] = x . w[h+1]` in which every
+    product overwrites a matrix that another product of the same level still reads.  Sizes are large enough for the
+    matrix-core kernel, with aligned and unaligned variants.  Returns (procedure, keep list)."""
+    rng = np.random.default_rng(1000 + seed)
+    heads = int(rng.integers(2, 21))
+    M, N, K = [(64, 64, 64), (128, 64, 96), (72, 80, 66), (96, 32, 160), (64, 128, 64)][seed % 5]
+    cmds, keep = [], []
+
+    def mat(name, shape, scale=1.0):
+        cmds.append(IR.CreateMat((rng.standard_normal(int(np.prod(shape))) * scale).astype(np.float32), list(shape), name))
+        return name
+
+    x = mat("x", [M, K])
+    packing = int(rng.integers(3))
+    w = []
+    if packing == 0:      # [heads, K, N]: dense slices at an offset
+        mat("wp", [heads, K, N], K ** -0.5)
+        for h in range(heads):
+            cmds.append(IR.Index(a="wp", index=h, dim=0, res=f"w{h}"))
+            w.append(f"w{h}")
+    elif packing == 1:    # [K, heads, N]: strided slices at an offset
+        mat("wp", [K, heads, N], K ** -0.5)
+        for h in range(heads):
+            cmds.append(IR.Index(a="wp", index=h, dim=1, res=f"w{h}"))
+            w.append(f"w{h}")
+    else:                 # separate matrices
+        for h in range(heads):
+            w.append(mat(f"w{h}", [K, N], K ** -0.5))
+    # level 1: s[h] = x . w[h]
+    s = []
+    for h in range(heads):
+        cmds.append(IR.DotProduct(a=x, b=w[h], res=f"s{h}"))
+        s.append(f"s{h}")
+        if rng.integers(3) == 0:
+            keep.append(f"s{h}")
+    second = int(rng.integers(3))
+    if second == 0:
+        # level 2 behind element-wise work: g[h] = sin(s[h])^T . x, then the sum over the heads
+        for h in range(heads):
+            cmds += [IR.Sin(a=s[h], res=f"u{h}"), IR.Permute(a=f"u{h}", p=[1, 0], res=f"ut{h}"),
+                     IR.DotProduct(a=f"ut{h}", b=x, res=f"g{h}")]
+        cmds.append(IR.CreateConstant(0.0, "acc", [N, K]))
+        for h in range(heads):
+            cmds.append(IR.ElwAddEq(s="acc", o=f"g{h}"))
+        keep += ["acc", f"g{heads - 1}"]
+    elif second == 1:
+        # level 2 on transposed weights: dx = sum over h of s[h] . w[h]^T
+        cmds.append(IR.CreateConstant(0.0, "dx", [M, K]))
+        for h in range(heads):
+            cmds += [IR.Permute(a=w[h], p=[1, 0], res=f"wt{h}"), IR.DotProduct(a=s[h], b=f"wt{h}", res=f"d{h}"),
+                     IR.ElwAddEq(s="dx", o=f"d{h}")]
+        keep += ["dx", "d0"]
+    else:
+        keep.append(s[0])
+    if M == N == K:
+        # rotation over square matrices: every product reads the old contents of the matrix the next one overwrites
+        r = [mat(f"r{h}", [K, K], K ** -0.5) for h in range(heads)]
+        for h in range(heads - 1):
+            cmds.append(IR.DotProduct(a=x, b=r[h + 1], res=r[h]))
+        cmds.append(IR.DotProduct(a=x, b=r[0], res=r[heads - 1]))   # ... and one that depends on a new value
+        keep += r
+    return IR.IRProcedure("main", cmds + [IR.EX()]), sorted(set(keep))

@@ -301,3 +301,27 @@ def test_code_object_cache_checks_the_source(tmp_path, monkeypatch):
     assert rc == 0, msg
     again = open(path, "rb").read()
     assert again.startswith(b"ADHC1\n") and b"adhip_sinX" not in again and abs(len(again) - good_size) < 4096
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_grouped_products_plan(seed, monkeypatch):
+    """Same-shape independent matrix products share grouped launches (at most 16 products each), every product is
+    still computed exactly once, and the switch ADHIP_GROUP_DOTS=0 restores one launch per product."""
+    from fuzz_control import random_grouped_products_program
+    from oracle.interp import OracleDevice
+    proc, keep = random_grouped_products_program(seed)
+    n_products = sum(1 for c in proc.main if isinstance(c, IR.DotProduct))
+    text = lower_describe(proc, set(keep))
+    grouped = [int(m) for m in re.findall(r"launch dots_\w+?_(\d+)x_", text)]
+    single = len(re.findall(r"launch dot_\w+ \[dot_", text))
+    assert grouped and all(2 <= g <= 16 for g in grouped), text
+    monkeypatch.setenv("ADHIP_GROUP_DOTS", "0")
+    text0 = lower_describe(proc, set(keep))
+    assert "launch dots_" not in text0
+    needed = len(re.findall(r"launch dot_\w+ \[dot_", text0))   # products nothing reads are not computed at all
+    assert 2 <= needed <= n_products
+    assert sum(grouped) + single == needed, text
+    # the program itself is valid: the oracle runs it
+    dev = OracleDevice()
+    dev.execute(proc, set(keep))
+    assert all(not dev.get_tensor(k).is_none for k in keep)

@@ -523,3 +523,23 @@ def test_enqueue_and_sync(hip_device):
     assert_exact(hip_device.get_tensor("x").data, x0 + 5, "four queued runs after one waited-for run")
     assert_exact(hip_device.get_tensor("s").data, (x0 + 5).reshape(3, 4).sum(1), "row sums of the last run")
     prog.close()
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_grouped_products_match_oracle(seed, hip_device):
+    """Independent same-shape matrix products that share one grouped launch (tests/fuzz_control.py::
+    random_grouped_products_program): offsets into packed weights, transposed operands, element-wise work between
+    two levels of products, and products that overwrite what others of their launch still read."""
+    print(f"[case] grouped products seed {seed}", flush=True)
+    from fuzz_control import random_grouped_products_program
+    from adhip.device import lower_describe
+    proc, keep = random_grouped_products_program(seed)
+    assert "launch dots_" in lower_describe(proc, set(keep))
+    ref_dev = OracleDevice()
+    ref_dev.execute(proc, set(keep))
+    hip_device.execute(proc, set(keep))
+    got = {k: hip_device.get_tensor(k) for k in keep}
+    for k in keep:
+        ref = ref_dev.get_tensor(k)
+        assert not got[k].is_none and got[k].dim == ref.dim, k
+        assert_close(got[k].data, ref.data, RED_RTOL * 16, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
