@@ -69,6 +69,42 @@ def test_malformed_program_is_an_error_not_a_crash():
         lower_describe(proc, {"y"})
 
 
+def test_damaged_command_streams_are_errors_not_crashes():
+    """Truncations, overwritten bytes and words, and single bit flips of valid command streams (nested control flow,
+    views, products): parsing and lowering either succeed or report an error.  Payload addresses inside a stream are
+    never dereferenced by the lowering, so damaged ones are harmless here."""
+    import numpy as np
+    from fuzz_control import random_control_program, random_grouped_products_program
+    lib = load_library()
+    cases = [random_control_program(seed)[:2] for seed in range(4)] + [random_grouped_products_program(0)]
+    rng = np.random.default_rng(7)
+    cap = 1 << 22
+    buf = ctypes.create_string_buffer(cap)
+    outcomes = set()
+    for it in range(800):
+        proc, keep = cases[it % len(cases)]
+        blob, keepalive = IR.serialize(proc)
+        b = bytearray(blob)
+        kind = it % 4
+        if kind == 0:
+            b = b[: int(rng.integers(0, len(b)))]
+        elif kind == 1:
+            for _ in range(int(rng.integers(1, 4))):
+                b[int(rng.integers(8, len(b)))] = int(rng.integers(256))
+        elif kind == 2:
+            i = int(rng.integers(8, len(b) - 4))
+            b[i:i + 4] = int(rng.integers(0, 2 ** 32)).to_bytes(4, "little")
+        else:
+            b[int(rng.integers(8, len(b)))] ^= 1 << int(rng.integers(8))
+        ids = [k.encode() for k in keep]
+        arr = (ctypes.c_char_p * len(ids))(*ids)
+        rc = lib.adhip_lower_describe(bytes(b), len(b), arr, len(ids), buf, cap)
+        outcomes.add(rc == 0)
+        assert rc == 0 or buf.value, "an error without a message"
+        del keepalive
+    assert outcomes == {True, False}
+
+
 @pytest.mark.parametrize("name", sorted(KATS))
 def test_kat_programs_lower_and_compile_for_gfx950(name):
     dev = Capture()
