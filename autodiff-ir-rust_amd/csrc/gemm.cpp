@@ -68,11 +68,15 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 // GROUPED: several independent products of one shape and one set of strides in a single launch; the block row
 // blockIdx.y works on problem y, whose three base pointers (operand offsets already applied) are parameters
 // c<y>, a<y>, b<y>.  For the same kind of product when there are many of them (the per-head projections of
-// multi-head attention), instead of cutting k.
+// multi-head attention).  With SPLITK the range of k is picked by blockIdx.z.
 extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
 #if GROUPED
     const int* __restrict__ guard, GROUP_PARAMS long long M, long long N, long long K, long long a_sm, long long a_sk,
-    long long b_sk, long long b_sn) {
+    long long b_sk, long long b_sn
+#if SPLITK
+    , long long k_chunk
+#endif
+    ) {
     if (guard && *guard == 0) return;
     float* __restrict__ C;
     const float* __restrict__ A;
@@ -90,9 +94,14 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     if (guard && *guard == 0) return;
 #endif
 #if SPLITK
-    const long long k_lo = (long long)blockIdx.y * k_chunk;
+#if GROUPED
+    const unsigned slice = blockIdx.z;  // c<y> points at problem y's own [gridDim.z][M][N] slices
+#else
+    const unsigned slice = blockIdx.y;
+#endif
+    const long long k_lo = (long long)slice * k_chunk;
     const long long k_hi = min(K, k_lo + k_chunk);
-    C += (long long)blockIdx.y * M * N;
+    C += (long long)slice * M * N;
 #else
     const long long k_lo = 0, k_hi = K;
 #endif

@@ -161,6 +161,42 @@ extern "C" __global__ __launch_bounds__(256) void adhip_sum_slices(const int* __
     }
 }
 
+// The same for up to 16 products that shared one launch: blockIdx.y picks the product, whose slices are
+// slices[y][count][n] and whose result goes to o<y>.
+#define ADHIP_O16 float* o0, float* o1, float* o2, float* o3, float* o4, float* o5, float* o6, float* o7, float* o8, float* o9, \
+                  float* o10, float* o11, float* o12, float* o13, float* o14, float* o15
+extern "C" __global__ __launch_bounds__(256) void adhip_sum_slices_grouped(const int* __restrict__ guard, ADHIP_O16,
+                                                                           const float* __restrict__ slices, long long count,
+                                                                           long long n) {
+    if (guard && *guard == 0) return;
+    float* __restrict__ out;
+    switch (blockIdx.y) {
+    case 0: out = o0; break; case 1: out = o1; break; case 2: out = o2; break; case 3: out = o3; break;
+    case 4: out = o4; break; case 5: out = o5; break; case 6: out = o6; break; case 7: out = o7; break;
+    case 8: out = o8; break; case 9: out = o9; break; case 10: out = o10; break; case 11: out = o11; break;
+    case 12: out = o12; break; case 13: out = o13; break; case 14: out = o14; break; case 15: out = o15; break;
+    default: return;
+    }
+    slices += (long long)blockIdx.y * count * n;
+    const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    if ((n & 3) == 0) {
+        float4 acc = *(const float4*)(slices + i);
+#pragma unroll 4
+        for (long long s = 1; s < count; ++s) {
+            const float4 v = *(const float4*)(slices + s * n + i);
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+        *(float4*)(out + i) = acc;
+    } else {
+        for (long long j = i; j < n && j < i + 4; ++j) {
+            float acc = slices[j];
+            for (long long s = 1; s < count; ++s) acc += slices[s * n + j];
+            out[j] = acc;
+        }
+    }
+}
+
 // One thread per output element, k ascending, one accumulator: the reference's dot kernel
 // (src/devices/opencl/kernels/dotprod.rs:23-53).  Used for small products.
 extern "C" __global__ __launch_bounds__(256) void adhip_dot_naive(const int* __restrict__ guard, float* __restrict__ c,
@@ -224,7 +260,7 @@ struct Lowerer {
     std::vector<std::unique_ptr<Node>> arena;
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
-    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sum_slices = -1;
+    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sum_slices = -1, fixed_sum_slices_grouped = -1;
     int dot_epilogue_counter = 0;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
 
@@ -1186,7 +1222,6 @@ struct Lowerer {
         // within a depth, puts everything such a set reads before all of it and everything that reads it after.
         // Dependencies are the values a kernel reads plus, for a kernel that overwrites an id's buffer, the earlier
         // kernels that still read the id's old contents.  Regions without such a set keep program order.
-        if (opt.fuse && opt.group_dots) group_products(groups, group_of, reads, home_of_early, reads_node);
         // ---- 6. generate code per group (no buffers needed yet)
         struct GK {
             GeneratedKernel k;
@@ -1227,6 +1262,19 @@ struct Lowerer {
             }
             return -1;
         };
+        if (opt.fuse && opt.group_dots) {
+            // a product that fills the chip by itself gives up an epilogue only for nothing: it stays out of grouped
+            // launches when an element-wise consumer could run on its accumulators
+            auto keeps_epilogue = [&](int g) {
+                Node* D = groups[g].members[0];
+                const int64_t M = D->shape[0], N = D->shape[1];
+                if (((M + 127) / 128) * ((N + 127) / 128) < 256) return false;
+                return find_epilogue((size_t)g, D, numel(D->shape)) >= 0;
+            };
+            group_products(groups, group_of, reads, home_of_early, reads_node, keeps_epilogue);
+            gks.resize(groups.size());  // dead groups were dropped if the region was reordered
+            greads.resize(groups.size());
+        }
         for (size_t g = 0; g < groups.size(); ++g) {
             Group& G = groups[g];
             if (G.dead) continue;
@@ -1284,7 +1332,15 @@ struct Lowerer {
                             if (rd.first != D && numel(rd.first->shape) * 2 >= numel(D->shape)) big.insert(rd.first);
                     if (big.size() > 8) nx = -1;
                 }
-                if (dpl.splits > 1) {
+                if (grouped) {
+                    const DotLaunchPlan gpl = plan_dot_group(D, (int)G.members.size());
+                    if (gpl.splits > 1) {
+                        Node* partial = new_node(Op::COPY, Shape{(int64_t)G.members.size() * gpl.splits, numel(D->shape)}, {},
+                                                 D->name + ".slices", 0.f, false);
+                        partial->root = true;
+                        gks[g].extra_nodes.push_back(partial);
+                    }
+                } else if (dpl.splits > 1) {
                     Node* partial = new_node(Op::COPY, Shape{dpl.splits, numel(D->shape)}, {}, D->name + ".slices", 0.f, false);
                     partial->root = true;
                     gks[g].extra_nodes.push_back(partial);
@@ -1460,7 +1516,7 @@ struct Lowerer {
             Group& G = groups[g];
             if (G.dead) continue;
             if (G.kind == Group::DOT) {
-                if (G.members.size() > 1) emit_dot_group(G.members, out);
+                if (G.members.size() > 1) emit_dot_group(G.members, out, gks[g].extra_nodes.empty() ? nullptr : gks[g].extra_nodes[0]);
                 else if (!G.epi.empty()) emit_dot(G.members[0], out, &gks[g].dot_epi, gks[g].dot_store);
                 else emit_dot(G.members[0], out, nullptr, true, gks[g].extra_nodes.empty() ? nullptr : gks[g].extra_nodes[0]);
                 continue;
@@ -1574,30 +1630,39 @@ struct Lowerer {
         push_launch(out, l, "transpose");
     }
 
+    // How a matrix-core product is launched: tile, bounds checking, and how many ranges of k it is split into.
+    struct DotLaunchPlan {
+        GemmConfig cfg;
+        int bn_tile = 128;
+        int64_t splits = 1, k_chunk = 0;
+    };
+
     // What must agree for products to share a grouped launch: sizes, strides and whether operands are 16-byte
-    // aligned.  False for products that fill the chip on their own or do not go to the matrix cores.
+    // aligned.  False for products that do not go to the matrix cores.
     static bool dot_group_key(const Node* n, std::array<int64_t, 8>& key) {
         if (!dot_uses_mfma(n)) return false;
         Affine2D a, b;
         tref_affine2d(n->in[0], a);
         tref_affine2d(n->in[1], b);
         const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
-        if (((M + 127) / 128) * ((N + 127) / 128) >= 256) return false;
         const int64_t a_ld = a.s1 == 1 ? a.s0 : a.s1, b_ld = b.s0 == 1 ? b.s1 : b.s0;
         const bool unaligned = (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
         key = {M, N, K, a.s0, a.s1, b.s0, b.s1, unaligned ? 1 : 0};
         return true;
     }
 
-    template <class ReadsNode>
+    template <class ReadsNode, class KeepsEpilogue>
     void group_products(std::vector<Group>& groups, std::map<Node*, int>& group_of, std::map<Node*, std::map<Node*, bool>>& reads,
-                        const std::map<Node*, std::string>& home_of_early, ReadsNode&& reads_node) {
+                        const std::map<Node*, std::string>& home_of_early, ReadsNode&& reads_node, KeepsEpilogue&& keeps_epilogue) {
         const int G = (int)groups.size();
         std::vector<std::array<int64_t, 8>> key(G);
         std::vector<char> cand(G, 0);
         int ncand = 0;
         for (int g = 0; g < G; ++g)
-            if (!groups[g].dead && groups[g].kind == Group::DOT && dot_group_key(groups[g].members[0], key[g])) { cand[g] = 1; ++ncand; }
+            if (!groups[g].dead && groups[g].kind == Group::DOT && dot_group_key(groups[g].members[0], key[g]) && !keeps_epilogue(g)) {
+                cand[g] = 1;
+                ++ncand;
+            }
         if (ncand < 2) return;
         // depth of every kernel
         std::vector<int> level(G, 0);
@@ -1682,30 +1747,64 @@ struct Lowerer {
         }
     }
 
-    // One launch for several products of the same shape (see group_products): problem y is block row y.
-    void emit_dot_group(const std::vector<Node*>& dots, std::vector<Step>& out) {
+    // Tile and k ranges of a grouped launch of `cnt` products shaped like `first`: by the number of blocks the whole
+    // launch has, as plan_dot does for a single product.
+    static DotLaunchPlan plan_dot_group(const Node* first, int cnt) {
+        std::array<int64_t, 8> key{};
+        ADHIP_CHECK(dot_group_key(first, key), "internal: grouped launch of a product that does not qualify");
+        const int64_t M = key[0], N = key[1], K = key[2];
+        DotLaunchPlan pl;
+        GemmConfig& cfg = pl.cfg;
+        cfg.a_kcontig = key[4] == 1;
+        cfg.b_kcontig = key[5] == 1;
+        cfg.grouped = true;
+        const int64_t blocks128 = ((M + 127) / 128) * ((N + 127) / 128) * cnt;
+        const int64_t max_splits = std::min<int64_t>(K / 256, 32);
+        auto splits_for = [&](int64_t blocks) {
+            if (blocks >= 256 || max_splits < 2) return (int64_t)1;
+            return std::max<int64_t>(std::min<int64_t>((512 + blocks - 1) / blocks, max_splits), 1);
+        };
+        // three 64x64 blocks per CU without cutting k beat 128x128 blocks with k cut and the slice sum that follows
+        // (12 x 2048x128x1024: 66 us against 77 + 8); with two per CU it is the other way round (8 x 2048x128x2048:
+        // 105-118 us against 80 + 7)
+        const int64_t blocks64 = ((M + 63) / 64) * ((N + 63) / 64) * cnt;
+        const bool small_whole = blocks128 < 256 && blocks64 >= 768;
+        cfg.bm = (!small_whole && blocks128 * splits_for(blocks128) >= 256) ? 128 : 64;
+        pl.bn_tile = cfg.bm == 64 ? 64 : 128;
+        if (cfg.bm == 128 && blocks128 < 512 && splits_for(blocks128) == 1) { pl.bn_tile = 64; cfg.bn = 64; }
+        cfg.edge = key[7] || (M % cfg.bm) || (N % pl.bn_tile);
+        const int64_t blocks = ((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile) * cnt;
+        const int64_t want = small_whole ? 1 : splits_for(blocks);
+        if (want > 1) {
+            pl.k_chunk = (((K + want - 1) / want) + 15) / 16 * 16;
+            pl.splits = (K + pl.k_chunk - 1) / pl.k_chunk;
+            cfg.split_k = pl.splits > 1;
+            if (!cfg.split_k) pl.splits = 1;
+        }
+        return pl;
+    }
+
+    // One launch for several products of the same shape (see group_products): problem y is block row y; with k cut
+    // into ranges, range z is block layer z and `partial` holds [problem][range][M*N] partial products, added by one
+    // grouped launch of the slice sum.
+    void emit_dot_group(const std::vector<Node*>& dots, std::vector<Step>& out, Node* partial) {
         const int cnt = (int)dots.size();
         ADHIP_CHECK(cnt >= 2 && cnt <= kGemmGroupSlots, "internal: grouped product launch of %d products", cnt);
         std::array<int64_t, 8> key0{};
         ADHIP_CHECK(dot_group_key(dots[0], key0), "internal: grouped launch of a product that does not qualify");
         const int64_t M = key0[0], N = key0[1], K = key0[2];
-        GemmConfig cfg;
-        cfg.a_kcontig = key0[4] == 1;
-        cfg.b_kcontig = key0[5] == 1;
-        cfg.grouped = true;
-        // tile by the number of blocks the whole launch has, as for a single product
-        const int64_t blocks128 = ((M + 127) / 128) * ((N + 127) / 128) * cnt;
-        cfg.bm = blocks128 >= 256 ? 128 : 64;
-        int bn_tile = cfg.bm == 64 ? 64 : 128;
-        if (cfg.bm == 128 && blocks128 < 512) { bn_tile = 64; cfg.bn = 64; }
-        cfg.edge = key0[7] || (M % cfg.bm) || (N % bn_tile);
-        std::string entry = strf("adhip_gemm_%c%c_%d%s%s_grouped", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
-                                 cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? "_edge" : "");
+        const DotLaunchPlan pl = plan_dot_group(dots[0], cnt);
+        const GemmConfig& cfg = pl.cfg;
+        ADHIP_CHECK(cfg.split_k == (partial != nullptr), "internal: split grouped product and its slice buffer disagree");
+        ADHIP_CHECK(!partial || numel(partial->shape) == (int64_t)cnt * pl.splits * M * N, "internal: slice buffer of the wrong size");
+        std::string entry = strf("adhip_gemm_%c%c_%d%s%s%s_grouped", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
+                                 cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? "_edge" : "", cfg.split_k ? "_splitk" : "");
         Launch l;
         l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
         l.block[0] = cfg.bm == 64 ? 256u : (unsigned)(cfg.bm * 2);
-        l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + bn_tile - 1) / bn_tile));
+        l.grid[0] = (unsigned)(((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile));
         l.grid[1] = (unsigned)cnt;
+        l.grid[2] = (unsigned)pl.splits;
         auto B = [&](Node* x, int64_t off) {
             Arg q;
             q.kind = Arg::BUF;
@@ -1716,22 +1815,40 @@ struct Lowerer {
         };
         auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
         for (int i = 0; i < kGemmGroupSlots; ++i) {
-            Node* n = dots[std::min(i, cnt - 1)];  // unused slots repeat the last problem; no block reads them
+            const int pi = std::min(i, cnt - 1);  // unused slots repeat the last problem; no block reads them
+            Node* n = dots[pi];
             std::array<int64_t, 8> key{};
             ADHIP_CHECK(dot_group_key(n, key) && key == key0, "internal: grouped products differ in shape or strides");
             Affine2D a, b;
             tref_affine2d(n->in[0], a);
             tref_affine2d(n->in[1], b);
-            l.args.push_back(B(n, 0));
+            l.args.push_back(partial ? B(partial, (int64_t)pi * pl.splits * M * N) : B(n, 0));
             l.args.push_back(B(a.base, a.offset));
             l.args.push_back(B(b.base, b.offset));
         }
-        for (int q = 0; q < 3; ++q) l.args.push_back(I(key0[q]));
-        for (int q = 3; q < 7; ++q) l.args.push_back(I(key0[q]));
+        for (int q = 0; q < 7; ++q) l.args.push_back(I(key0[q]));
+        if (cfg.split_k) l.args.push_back(I(pl.k_chunk));
         l.label = strf("dots_%s_%dx_%lldx%lldx%lld", dots[0]->name.c_str(), cnt, (long long)M, (long long)N, (long long)K);
-        l.bytes = 4.0 * cnt * ((double)M * K + (double)K * N + (double)M * N);
+        l.bytes = 4.0 * cnt * ((double)M * K + (double)K * N + (double)M * N * (double)pl.splits);
         l.flops = 2.0 * cnt * (double)M * (double)N * (double)K;
         push_launch(out, l, "dot_mfma");
+        if (cfg.split_k) {
+            if (fixed_sum_slices_grouped < 0)
+                fixed_sum_slices_grouped = add_kernel("adhip_sum_slices_grouped", fixed_kernels_source(), "sum_slices");
+            Launch lf;
+            lf.kernel = fixed_sum_slices_grouped;
+            lf.block[0] = 256;
+            lf.grid[0] = (unsigned)((M * N + 1023) / 1024);
+            lf.grid[1] = (unsigned)cnt;
+            for (int i = 0; i < kGemmGroupSlots; ++i) lf.args.push_back(B(dots[std::min(i, cnt - 1)], 0));
+            lf.args.push_back(B(partial, 0));
+            lf.args.push_back(I(pl.splits));
+            lf.args.push_back(I(M * N));
+            lf.label = l.label + "_sum";
+            lf.bytes = 4.0 * cnt * (double)M * (double)N * (double)(pl.splits + 1);
+            lf.flops = (double)cnt * (double)M * (double)N * (double)pl.splits;
+            push_launch(out, lf, "sum_slices");
+        }
     }
 
     // whether a product goes to the matrix-core kernel (else the one-thread-per-output kernel)
@@ -1743,12 +1860,6 @@ struct Lowerer {
         return M * N * K >= 64 * 64 * 64 && a_unit && b_unit;
     }
 
-    // How a matrix-core product is launched: tile, bounds checking, and how many ranges of k it is split into.
-    struct DotLaunchPlan {
-        GemmConfig cfg;
-        int bn_tile = 128;
-        int64_t splits = 1, k_chunk = 0;
-    };
     static DotLaunchPlan plan_dot(const Node* n) {
         Affine2D a, b;
         tref_affine2d(n->in[0], a);

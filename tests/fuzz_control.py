@@ -280,10 +280,11 @@ def random_grouped_products_program(seed: int):
     that are slices of one packed tensor (so the operands differ only by an offset), element-wise work between two
     levels of products, transposed operands, sums over the heads, and a rotation `w[h] = x . w[h+1]` in which every
     product overwrites a matrix that another product of the same level still reads.  Sizes are large enough for the
-    matrix-core kernel, with aligned and unaligned variants.  Returns (procedure, keep list)."""
+    matrix-core kernel, with aligned and unaligned variants and two with an inner dimension long enough to be cut
+    into ranges.  Returns (procedure, keep list)."""
     rng = np.random.default_rng(1000 + seed)
     heads = int(rng.integers(2, 21))
-    M, N, K = [(64, 64, 64), (128, 64, 96), (72, 80, 66), (96, 32, 160), (64, 128, 64)][seed % 5]
+    M, N, K = [(64, 64, 64), (128, 64, 96), (72, 80, 66), (96, 32, 160), (64, 128, 64), (64, 64, 512), (72, 40, 530)][seed % 7]
     cmds, keep = [], []
 
     def mat(name, shape, scale=1.0):

@@ -339,7 +339,7 @@ def test_code_object_cache_checks_the_source(tmp_path, monkeypatch):
     assert again.startswith(b"ADHC1\n") and b"adhip_sinX" not in again and abs(len(again) - good_size) < 4096
 
 
-@pytest.mark.parametrize("seed", range(20))
+@pytest.mark.parametrize("seed", range(28))
 def test_grouped_products_plan(seed, monkeypatch):
     """Same-shape independent matrix products share grouped launches (at most 16 products each), every product is
     still computed exactly once, and the switch ADHIP_GROUP_DOTS=0 restores one launch per product."""
@@ -348,7 +348,7 @@ def test_grouped_products_plan(seed, monkeypatch):
     proc, keep = random_grouped_products_program(seed)
     n_products = sum(1 for c in proc.main if isinstance(c, IR.DotProduct))
     text = lower_describe(proc, set(keep))
-    grouped = [int(m) for m in re.findall(r"launch dots_\w+?_(\d+)x_", text)]
+    grouped = [int(m) for m in re.findall(r"launch dots_\w+?_(\d+)x_\d+x\d+x\d+ \[dot_", text)]
     single = len(re.findall(r"launch dot_\w+ \[dot_", text))
     assert grouped and all(2 <= g <= 16 for g in grouped), text
     monkeypatch.setenv("ADHIP_GROUP_DOTS", "0")

@@ -525,7 +525,7 @@ def test_enqueue_and_sync(hip_device):
     prog.close()
 
 
-@pytest.mark.parametrize("seed", range(20))
+@pytest.mark.parametrize("seed", range(28))
 def test_grouped_products_match_oracle(seed, hip_device):
     """Independent same-shape matrix products that share one grouped launch (tests/fuzz_control.py::
     random_grouped_products_program): offsets into packed weights, transposed operands, element-wise work between
