@@ -862,8 +862,23 @@ struct Lowerer {
         walk(r, true);
     }
 
+    // Kernels are told apart by their text with the entry name blanked: the per-head kernels of multi-head attention
+    // (and the same epilogue generated for two layers) differ in nothing but the position in the program that their
+    // name carries, and then share the first one's code object instead of being compiled once each.
     int add_kernel(const std::string& entry, const std::string& source, const std::string& kind) {
-        std::string key = entry + "\n" + source;
+        std::string key;
+        key.reserve(source.size());
+        auto ident = [](char c) { return isalnum((unsigned char)c) || c == '_'; };
+        for (size_t pos = 0; pos < source.size();) {
+            const size_t hit = source.find(entry, pos);
+            if (hit == std::string::npos) { key.append(source, pos, std::string::npos); break; }
+            const size_t end = hit + entry.size();
+            const bool whole = (hit == 0 || !ident(source[hit - 1])) && (end >= source.size() || !ident(source[end]));
+            key.append(source, pos, hit - pos);
+            if (whole) key += "@entry@";
+            else key.append(source, hit, entry.size());
+            pos = end;
+        }
         auto it = kernel_by_source.find(key);
         if (it != kernel_by_source.end()) return it->second;
         KernelDef d;

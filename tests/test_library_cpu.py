@@ -361,3 +361,18 @@ def test_grouped_products_plan(seed, monkeypatch):
     dev = OracleDevice()
     dev.execute(proc, set(keep))
     assert all(not dev.get_tensor(k).is_none for k in keep)
+
+
+def test_kernels_differing_only_in_name_are_compiled_once():
+    """Every attention head runs the same generated kernels on other buffers; their names carry the position in the
+    program, but the plan holds (and the device compiles) one kernel for all of them: the number of kernels does not
+    grow with the number of heads, only the number of launches does."""
+    from oracle.interp import OracleDevice
+    counts = []
+    for heads in (2, 4, 8):
+        wl = W.encoder_layer(OracleDevice(), 64, 64, heads, 128, seed=1)
+        proc, deps = wl.finish()
+        text = lower_describe(proc, deps)
+        counts.append((int(re.search(r"kernels: (\d+)", text).group(1)), len(re.findall(r"^\s*launch", text, re.M))))
+    assert counts[0][0] == counts[1][0] == counts[2][0], counts
+    assert counts[0][1] < counts[1][1] < counts[2][1], counts
