@@ -296,3 +296,66 @@ def encoder_layer(dev, seq: int = 64, d_model: int = 32, heads: int = 4, ff_dim:
     fl += 2.0 * seq * d_model * d_model                     # output projection
     fl += 2 * 2.0 * seq * d_model * ff_dim                  # feed-forward
     return Workload("encoder_layer", outs, inputs, flops=fl * (3.0 if backward else 1.0))
+
+
+def encoder_train(dev, seq: int = 64, d_model: int = 32, heads: int = 4, ff_dim: int = 64, iters: int = 3,
+                  lr: float = 0.05, seed: int = 0) -> Workload:
+    """`iters` SGD steps on one TransformerEncoderLayer inside an IR for-loop: y = layer(x); loss = mean((y - t)^2);
+    zero_grad, forward, backward, step.  Every weight is updated in place while the next iteration's products read
+    it, which is what a training loop over the reference's modules does (src/tests/nn.rs:10-45 for the MLP)."""
+    autodiff.set_device(dev)
+    autodiff.eager_dep_opt()
+    rng = np.random.default_rng(seed)
+    inputs: Dict[str, np.ndarray] = {}
+    layer = nn.TransformerEncoderLayer(d_model, heads, ff_dim)
+    d_v = d_model // heads
+    named = {}
+
+    def mat(name, fan_in, fan_out):
+        w = (rng.standard_normal((fan_in, fan_out)) / np.sqrt(fan_in)).astype(np.float32)
+        inputs[name] = w
+        named[name] = autodiff.tensor(w, [fan_in, fan_out])
+        return named[name]
+
+    def vec(name, n):
+        b = (0.1 * rng.standard_normal(n)).astype(np.float32)
+        inputs[name] = b
+        named[name] = autodiff.tensor(b, [n])
+        return named[name]
+
+    for h in range(heads):
+        for kind, group in (("wq", layer.attention.wq), ("wk", layer.attention.wk), ("wv", layer.attention.wv)):
+            group[h].w = mat(f"{kind}{h}", d_model, d_v)
+    layer.attention.wo.w = mat("wo", d_model, d_model)
+    layer.ffwd.w_expand.w = mat("w1", d_model, ff_dim)
+    layer.ffwd.w_expand.b = vec("b1", ff_dim)
+    layer.ffwd.w_contract.w = mat("w2", ff_dim, d_model)
+    layer.ffwd.w_contract.b = vec("b2", d_model)
+    named["ln1_scale"] = layer.layer_norm_att.scale
+    named["ln2_scale"] = layer.layer_norm_ffwd.scale
+    xn = rng.standard_normal((seq, d_model)).astype(np.float32)
+    tn = rng.standard_normal((seq, d_model)).astype(np.float32)
+    inputs["x"], inputs["t"] = xn, tn
+    x = autodiff.tensor(xn, [seq, d_model])
+    t = autodiff.tensor(tn, [seq, d_model])
+    opt = nn.SGD(list(named.values()), lr)
+    scale = 1.0 / float(seq * d_model)
+    box = {}
+
+    def body(_):
+        y = layer.f(x)
+        d = y - t
+        loss = (d * d).sum(1).sum(0) * scale
+        opt.zero_grad()
+        loss.forward()
+        loss.backward()
+        opt.step()
+        box["loss"] = loss
+
+    autodiff.ir_for(range(0, iters), body)
+    outs = {"loss": box["loss"].val()}
+    for name, p in named.items():
+        outs[name] = p.val()
+    for v in outs.values():
+        v.keep()
+    return Workload("encoder_train", outs, inputs)

@@ -376,3 +376,15 @@ def test_kernels_differing_only_in_name_are_compiled_once():
         counts.append((int(re.search(r"kernels: (\d+)", text).group(1)), len(re.findall(r"^\s*launch", text, re.M))))
     assert counts[0][0] == counts[1][0] == counts[2][0], counts
     assert counts[0][1] < counts[1][1] < counts[2][1], counts
+
+
+def test_training_loop_body_groups_per_head_products():
+    """The loop body of an encoder training loop is a region like any other: its per-head products share launches, and
+    the weight updates are ordered behind the products of the same iteration that read the old weights."""
+    from oracle.interp import OracleDevice
+    wl = W.encoder_train(OracleDevice(), 128, 128, 2, 256, iters=3, lr=1.0, seed=1)
+    proc, deps = wl.finish()
+    text = lower_describe(proc, deps)
+    body = text[text.index("while "):]
+    assert "launch dots_" in body
+    assert "[counted:" in text

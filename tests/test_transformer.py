@@ -114,3 +114,26 @@ def test_norm_modules_at_scale_match_float64_autograd(kind, rows, cols, hip_devi
     tol = RED_RTOL * math.sqrt(cols)
     assert_close(got_y.data, yt.detach().numpy().reshape(-1), tol, "y")
     assert_close(got_dx.data, xt.grad.numpy().reshape(-1), 4 * tol, "dx")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seq,d_model,heads,ff", [(128, 128, 2, 256), (96, 144, 3, 200), (16, 16, 4, 32)])
+def test_encoder_training_loop_matches_oracle(seq, d_model, heads, ff, hip_device):
+    """Three SGD steps on an encoder layer inside an IR for-loop (workloads.encoder_train): grouped per-head products,
+    product epilogues and in-place weight updates inside a loop body, where every update must come after the last
+    product of the iteration that still reads the old weights.  What is compared is how far each weight moved, which
+    is a thousand times smaller than the weight itself."""
+    print(f"[case] encoder training loop {seq}x{d_model} heads {heads} ff {ff}", flush=True)
+    got = W.encoder_train(hip_device, seq, d_model, heads, ff, iters=3, lr=1.0, seed=seq).run()
+    wl = W.encoder_train(OracleDevice(), seq, d_model, heads, ff, iters=3, lr=1.0, seed=seq)
+    ref = wl.run()
+    assert_close(got["loss"].data, ref["loss"].data, 1e-4, "loss")
+    for k, rv in ref.items():
+        if k not in wl.inputs:
+            continue
+        w0 = wl.inputs[k].reshape(-1).astype(np.float64)
+        moved_ref = np.asarray(rv.data, dtype=np.float64) - w0
+        moved_got = np.asarray(got[k].data, dtype=np.float64) - w0
+        assert np.abs(moved_ref).max() > 1e-4, f"{k} did not train"
+        err = np.abs(moved_got - moved_ref).max()
+        assert err <= 2e-3 * np.abs(moved_ref).max() + 4e-7 * np.abs(w0).max(), (k, err, np.abs(moved_ref).max())
