@@ -245,6 +245,7 @@ struct Group {
     // element-wise values of the result's size that the reduction evaluates and stores right after summing
     std::vector<Node*> epi;
     bool dead = false;  // its only member was absorbed by another group
+    int lead = -1;      // >= 0: runs inside the launches of that group (same kernels on other buffers), which it follows directly
 };
 
 struct Lowerer {
@@ -260,6 +261,7 @@ struct Lowerer {
     std::vector<std::unique_ptr<Node>> arena;
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
+    std::map<std::pair<int, int>, int> layered_kernels;
     int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sum_slices = -1, fixed_sum_slices_grouped = -1;
     int dot_epilogue_counter = 0;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
@@ -890,6 +892,61 @@ struct Lowerer {
         return (int)plan->kernels.size() - 1;
     }
 
+    // The variant of a generated kernel that runs `cnt` instances of it in one launch: the kernel becomes a device
+    // function, and the new entry hands it the buffers of instance blockIdx.z.  Every parameter after `guard` is a
+    // pointer; the variant takes cnt of each, in the order p0_0 .. p0_<cnt-1>, p1_0 ...
+    int add_layered_kernel(int kernel, int cnt) {
+        auto it = layered_kernels.find({kernel, cnt});
+        if (it != layered_kernels.end()) return it->second;
+        const KernelDef base = plan->kernels[kernel];
+        const std::string& src = base.source;
+        const std::string head = "extern \"C\" __global__ __launch_bounds__(";
+        const size_t at = src.find(head);
+        ADHIP_CHECK(at != std::string::npos && src.find(head, at + 1) == std::string::npos, "internal: kernel '%s' has no single entry", base.entry.c_str());
+        const size_t lb_end = src.find(')', at + head.size());
+        const std::string bounds = src.substr(at + head.size(), lb_end - (at + head.size()));
+        const size_t open = src.find('(', lb_end + 1), close = src.find(") {", open);
+        ADHIP_CHECK(open != std::string::npos && close != std::string::npos, "internal: kernel '%s' has no parameter list", base.entry.c_str());
+        std::vector<std::pair<std::string, std::string>> params;  // (type, name) after guard
+        {
+            const std::string list = src.substr(open + 1, close - open - 1);
+            size_t pos = 0;
+            bool first = true;
+            while (pos < list.size()) {
+                size_t comma = list.find(',', pos);
+                if (comma == std::string::npos) comma = list.size();
+                std::string prm = list.substr(pos, comma - pos);
+                pos = comma + 1;
+                while (!prm.empty() && prm.front() == ' ') prm.erase(prm.begin());
+                while (!prm.empty() && prm.back() == ' ') prm.pop_back();
+                if (first) { first = false; continue; }  // guard
+                const size_t sp = prm.find_last_of(" *");
+                ADHIP_CHECK(sp != std::string::npos && prm.find('*') != std::string::npos, "internal: kernel '%s' takes a non-pointer argument", base.entry.c_str());
+                params.push_back({prm.substr(0, sp + 1), prm.substr(sp + 1)});
+            }
+        }
+        const std::string entry = base.entry + strf("_x%d", cnt);
+        std::string out = src.substr(0, at);
+        out += "static __device__ __forceinline__ void " + base.entry + "_one" + src.substr(open);
+        out += "\nextern \"C\" __global__ __launch_bounds__(" + bounds + ") void " + entry + "(const int* __restrict__ guard";
+        for (auto& pr : params)
+            for (int q = 0; q < cnt; ++q) out += ", " + pr.first + pr.second + strf("_%d", q);
+        out += ") {\n";
+        for (auto& pr : params) out += "    " + pr.first + pr.second + ";\n";
+        out += "    switch (blockIdx.z) {\n";
+        for (int q = 0; q < cnt; ++q) {
+            out += strf("    case %d:", q);
+            for (auto& pr : params) out += " " + pr.second + " = " + pr.second + strf("_%d;", q);
+            out += " break;\n";
+        }
+        out += "    default: return;\n    }\n    " + base.entry + "_one(guard";
+        for (auto& pr : params) out += ", " + pr.second;
+        out += ");\n}\n";
+        const int idx = add_kernel(entry, out, base.kind);
+        layered_kernels[{kernel, cnt}] = idx;
+        return idx;
+    }
+
     void push_launch(std::vector<Step>& out, Launch l, const std::string& kind) {
         KernelStat st;
         st.label = l.label;
@@ -1437,6 +1494,109 @@ struct Lowerer {
                 }
             }
         }
+        // ---- 6b. groups that run the same kernels on other buffers (every attention head's softmax passes) share
+        // their launches: block layer blockIdx.z works on member z.  A follower is moved up behind its lead, which
+        // needs everything it reads to exist before the lead runs; groups that update a live id's buffer in place
+        // stay where they are.
+        if (opt.fuse && opt.layer_kernels) {
+            const size_t n_groups = groups.size();
+            auto updates_in_place = [&](const Group& H) {
+                std::vector<Node*> produced = H.members;
+                for (Node* sd : H.side) produced.push_back(sd);
+                for (Node* ep : H.epi) produced.push_back(ep);
+                for (Node* m : produced) {
+                    auto ho = home_of_early.find(m);
+                    if (ho != home_of_early.end() && livein.count(ho->second)) return true;
+                }
+                return false;
+            };
+            std::map<std::vector<int64_t>, std::vector<size_t>> by_signature;
+            for (size_t g = 0; g < n_groups; ++g) {
+                Group& H = groups[g];
+                if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM) || !H.colsums.empty() || updates_in_place(H)) continue;
+                std::vector<int64_t> sig;
+                bool ok = true;
+                auto add = [&](const GeneratedKernel& k) {
+                    if (k.source.find("blockIdx.z") != std::string::npos || !k.int_args.empty()) ok = false;
+                    sig.push_back(add_kernel(k.entry, k.source, k.kind));
+                    for (int d = 0; d < 3; ++d) { sig.push_back(k.grid[d]); sig.push_back(k.block[d]); }
+                    sig.push_back(k.lds_bytes);
+                    sig.push_back((int64_t)k.buffer_args.size());
+                    sig.push_back(k.chunks);
+                };
+                add(gks[g].k);
+                for (const GeneratedKernel& e : gks[g].extra) add(e);
+                if (ok && gks[g].k.grid[2] == 1) by_signature[sig].push_back(g);
+            }
+            std::vector<std::vector<size_t>> followers(n_groups);
+            bool any = false;
+            // sets in the order of their first member, so that a set whose members read the results of another
+            // (the pass after each head's reduction) sees where those have moved to
+            std::vector<const std::pair<const std::vector<int64_t>, std::vector<size_t>>*> sets;
+            for (auto& kv : by_signature) sets.push_back(&kv);
+            std::sort(sets.begin(), sets.end(), [](auto* x, auto* y) { return x->second[0] < y->second[0]; });
+            std::vector<size_t> position(n_groups);  // the old index of the group a group will run behind (its own if it stays)
+            for (size_t g = 0; g < n_groups; ++g) position[g] = g;
+            for (auto* set : sets) {
+                auto& kv = *set;
+                if (kv.second.size() < 2) continue;
+                const size_t n_buf = (size_t)kv.first[8];
+                const size_t cap = std::max<size_t>(1, std::min<size_t>(16, 96 / std::max<size_t>(1, n_buf)));
+                std::vector<size_t> leads;
+                for (size_t f : kv.second) {
+                    bool placed = false;
+                    for (size_t h : leads) {
+                        if (followers[h].size() + 1 >= cap) continue;
+                        bool ready = true;
+                        for (auto& rd : greads[f]) {
+                            if (op_is_leaf(rd.first->op)) continue;
+                            auto it = group_of.find(rd.first);
+                            if (it != group_of.end() && position[it->second] >= h) { ready = false; break; }
+                        }
+                        if (!ready) continue;
+                        followers[h].push_back(f);
+                        position[f] = h;
+                        placed = any = true;
+                        break;
+                    }
+                    if (!placed) leads.push_back(f);
+                }
+            }
+            if (any) {
+                std::vector<char> is_follower(n_groups, 0);
+                for (auto& fs : followers)
+                    for (size_t f : fs) is_follower[f] = 1;
+                std::vector<int> new_index(n_groups, -1);
+                std::vector<Group> sorted;
+                std::vector<GK> sorted_gks;
+                std::vector<std::map<Node*, bool>> sorted_reads;
+                auto take = [&](size_t g, int lead) {
+                    new_index[g] = (int)sorted.size();
+                    sorted.push_back(std::move(groups[g]));
+                    sorted.back().lead = lead;
+                    sorted_gks.push_back(std::move(gks[g]));
+                    sorted_reads.push_back(std::move(greads[g]));
+                };
+                for (size_t g = 0; g < n_groups; ++g) {
+                    if (is_follower[g]) continue;
+                    take(g, -1);
+                    const int lead = new_index[g];
+                    for (size_t f : followers[g]) take(f, lead);
+                }
+                for (auto& kv : group_of) kv.second = new_index[kv.second];
+                groups.swap(sorted);
+                gks.swap(sorted_gks);
+                greads.swap(sorted_reads);
+            }
+        }
+        // the last group of the shared launches a group runs in (itself if it runs alone)
+        std::vector<int> set_end(groups.size());
+        for (size_t g = 0; g < groups.size(); ++g) {
+            set_end[g] = (int)g;
+            const int lead = groups[g].lead;
+            if (lead >= 0)
+                for (int q = lead; q <= (int)g; ++q) set_end[q] = (int)g;
+        }
         // ---- 7. buffers: homes, temporaries, in-place hazards
         std::map<Node*, std::string> home_of;
         for (auto& w : wanted) home_of[w.second] = w.first;
@@ -1448,6 +1608,7 @@ struct Lowerer {
         struct Commit { int dst, src; int64_t n; std::string id; };
         std::vector<Commit> commits;
         std::vector<std::vector<Node*>> free_after(groups.size());
+        std::vector<int> scratch_to_free;
         for (size_t g = 0; g < groups.size(); ++g) {
             if (groups[g].dead) continue;
             std::vector<Node*> produced = groups[g].members;
@@ -1496,7 +1657,7 @@ struct Lowerer {
                     m->buffer = alloc_temp(numel(m->shape), m->name + ".tmp");
                     auto lr = last_reader.find(m);
                     int when = lr == last_reader.end() ? (int)g : std::max(lr->second, (int)g);
-                    free_after[when].push_back(m);
+                    free_after[set_end[when]].push_back(m);  // groups that share launches run at the same time
                 }
             }
             // partial-sum scratch of chunked reductions lives only inside this group
@@ -1504,7 +1665,10 @@ struct Lowerer {
                 if (e->op == Op::COPY) e->buffer = alloc_temp(numel(e->shape), e->name);
             }
             for (Node* e : gks[g].extra_nodes)
-                if (e->op == Op::COPY) free_temp(e->buffer);
+                if (e->op == Op::COPY) scratch_to_free.push_back(e->buffer);
+            if (set_end[g] != (int)g) continue;
+            for (int b : scratch_to_free) free_temp(b);
+            scratch_to_free.clear();
             for (Node* f : free_after[g]) free_temp(f->buffer);
         }
         // ---- 8. launches
@@ -1526,6 +1690,42 @@ struct Lowerer {
             l2.flops = gk.flops;
             for (Node* n : gk.buffer_args) l2.args.push_back(buf_arg(n));
             push_launch(out, l2, gk.kind);
+        };
+        // the launches of an element-wise group without column sums or of a reduction, with their statistics kinds
+        auto group_launches = [&](size_t g) {
+            Group& G = groups[g];
+            GeneratedKernel& k = gks[g].k;
+            std::vector<std::pair<Launch, std::string>> ls;
+            Launch l;
+            l.kernel = add_kernel(k.entry, k.source, k.kind);
+            memcpy(l.grid, k.grid, sizeof l.grid);
+            memcpy(l.block, k.block, sizeof l.block);
+            l.lds_bytes = k.lds_bytes;
+            l.label = k.entry;
+            l.bytes = k.bytes;
+            l.flops = k.flops;
+            if (G.kind == Group::SUM && k.chunks > 1) {
+                Node* partial = gks[g].extra_nodes[0];
+                Node* fin = gks[g].extra_nodes[1];
+                fin->buffer = G.members[0]->buffer;
+                for (size_t i = 0; i < k.buffer_args.size(); ++i)
+                    l.args.push_back(buf_arg(i == 0 ? partial : k.buffer_args[i]));
+                ls.push_back({l, k.kind});
+                GeneratedKernel& k2 = gks[g].extra[0];
+                Launch l2;
+                l2.kernel = add_kernel(k2.entry, k2.source, k2.kind);
+                memcpy(l2.grid, k2.grid, sizeof l2.grid);
+                memcpy(l2.block, k2.block, sizeof l2.block);
+                l2.label = k2.entry;
+                l2.bytes = k2.bytes;
+                l2.flops = k2.flops;
+                for (Node* n : k2.buffer_args) l2.args.push_back(buf_arg(n));
+                ls.push_back({l2, k2.kind});
+            } else {
+                for (Node* n : k.buffer_args) l.args.push_back(buf_arg(n));
+                ls.push_back({l, k.kind});
+            }
+            return ls;
         };
         for (size_t g = 0; g < groups.size(); ++g) {
             Group& G = groups[g];
@@ -1571,35 +1771,34 @@ struct Lowerer {
                 }
                 continue;
             }
-            Launch l;
-            l.kernel = add_kernel(k.entry, k.source, k.kind);
-            memcpy(l.grid, k.grid, sizeof l.grid);
-            memcpy(l.block, k.block, sizeof l.block);
-            l.lds_bytes = k.lds_bytes;
-            l.label = k.entry;
-            l.bytes = k.bytes;
-            l.flops = k.flops;
-            if (G.kind == Group::SUM && k.chunks > 1) {
-                Node* partial = gks[g].extra_nodes[0];
-                Node* fin = gks[g].extra_nodes[1];
-                fin->buffer = G.members[0]->buffer;
-                for (size_t i = 0; i < k.buffer_args.size(); ++i)
-                    l.args.push_back(buf_arg(i == 0 ? partial : k.buffer_args[i]));
-                push_launch(out, l, k.kind);
-                GeneratedKernel& k2 = gks[g].extra[0];
-                Launch l2;
-                l2.kernel = add_kernel(k2.entry, k2.source, k2.kind);
-                memcpy(l2.grid, k2.grid, sizeof l2.grid);
-                memcpy(l2.block, k2.block, sizeof l2.block);
-                l2.label = k2.entry;
-                l2.bytes = k2.bytes;
-                l2.flops = k2.flops;
-                for (Node* n : k2.buffer_args) l2.args.push_back(buf_arg(n));
-                push_launch(out, l2, k2.kind);
-            } else {
-                for (Node* n : k.buffer_args) l.args.push_back(buf_arg(n));
-                push_launch(out, l, k.kind);
+            // groups that share their launches: one launch per kernel of the lead, block layer z for member z
+            size_t last = g;
+            while (last + 1 < groups.size() && groups[last + 1].lead == (int)g) ++last;
+            std::vector<std::vector<std::pair<Launch, std::string>>> per_member;
+            for (size_t q = g; q <= last; ++q) per_member.push_back(group_launches(q));
+            for (size_t j = 0; j < per_member[0].size(); ++j) {
+                if (last == g) {
+                    push_launch(out, per_member[0][j].first, per_member[0][j].second);
+                    continue;
+                }
+                Launch l = per_member[0][j].first;
+                const int cnt = (int)per_member.size();
+                l.kernel = add_layered_kernel(l.kernel, cnt);
+                l.grid[2] = (unsigned)cnt;
+                l.args.clear();
+                for (size_t a = 0; a < per_member[0][j].first.args.size(); ++a)
+                    for (int q = 0; q < cnt; ++q) {
+                        const Launch& lq = per_member[q][j].first;
+                        ADHIP_CHECK(lq.kernel == per_member[0][j].first.kernel && lq.args.size() == per_member[0][j].first.args.size() &&
+                                        lq.args[a].kind == Arg::BUF, "internal: groups that share a launch differ");
+                        l.args.push_back(lq.args[a]);
+                    }
+                l.bytes *= cnt;
+                l.flops *= cnt;
+                l.label += strf("_x%d", cnt);
+                push_launch(out, l, per_member[0][j].second);
             }
+            g = last;
         }
         for (auto& c : commits) emit_copy(out, c.dst, c.src, c.n, "commit_" + c.id);
         for (auto& c : commits) free_temp(c.src);
@@ -2262,6 +2461,7 @@ std::string Plan::describe() const {
 std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids, const LowerOptions& opt_in) {
     LowerOptions opt = opt_in;
     if (const char* e = getenv("ADHIP_GROUP_DOTS")) opt.group_dots = opt.group_dots && atoi(e) != 0;
+    if (const char* e = getenv("ADHIP_LAYER_KERNELS")) opt.layer_kernels = opt.layer_kernels && atoi(e) != 0;
     Lowerer l(prog, dep_ids, opt);
     return l.run();
 }

@@ -14,7 +14,8 @@ namespace adhip {
 
 struct LowerOptions {
     bool fuse = true;  // false: one kernel per compute command (diagnostic mode)
-    bool group_dots = true;  // same-shape independent matrix products that under-fill the chip share a launch
+    bool group_dots = true;  // same-shape independent matrix products share a launch
+    bool layer_kernels = true;  // groups that run the same generated kernels on other buffers share their launches
 };
 
 std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids,

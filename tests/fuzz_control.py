@@ -341,3 +341,60 @@ def random_grouped_products_program(seed: int):
         cmds.append(IR.DotProduct(a=x, b=r[0], res=r[heads - 1]))   # ... and one that depends on a new value
         keep += r
     return IR.IRProcedure("main", cmds + [IR.EX()]), sorted(set(keep))
+
+
+def random_layered_program(seed: int):
+    """The same short chain of reductions and element-wise passes applied to many tensors of one shape, one tensor
+    after the other, as a model with several heads or several same-sized layers does: the kernels of the chains are
+    the same code on other buffers, which the device may run as block layers of shared launches.  Chains read
+    slices of packed tensors and separate tensors, some results feed an accumulation across the chains, and some
+    chains update their input in place (those must keep their place in the order).  Returns (procedure, keep)."""
+    rng = np.random.default_rng(5000 + seed)
+    heads = int(rng.integers(2, 24))
+    R, C = [(64, 128), (33, 20), (256, 64), (128, 256), (7, 300)][seed % 5]
+    cmds, keep = [], []
+    packed = bool(rng.integers(2))
+    if packed:
+        cmds.append(IR.CreateMat(rng.uniform(-1, 1, heads * R * C).astype(np.float32), [heads, R, C], "xp"))
+    xs = []
+    for h in range(heads):
+        if packed:
+            cmds.append(IR.Index(a="xp", index=h, dim=0, res=f"x{h}"))
+        else:
+            cmds.append(IR.CreateMat(rng.uniform(-1, 1, R * C).astype(np.float32), [R, C], f"x{h}"))
+        xs.append(f"x{h}")
+    cmds.append(IR.CreateMat(rng.uniform(-1, 1, R * C).astype(np.float32), [R, C], "shared"))
+    cmds.append(IR.CreateConstant(0.0, "acc", [R, C]))
+    chain = int(rng.integers(3))
+    for h in range(heads):
+        x = xs[h]
+        if chain == 0:
+            # softmax-like: e = exp2(x); n = rowsum(e); p = e * (1/n broadcast over the columns)
+            cmds += [IR.Exp2(a=x, res=f"e{h}"), IR.Sum(a=f"e{h}", res=f"n{h}"), IR.Recip(a=f"n{h}", res=f"i{h}"),
+                     IR.View(a=f"i{h}", target_dim=[R, 1], res=f"iv{h}"), IR.Broadcast(a=f"iv{h}", dim=1, r=C, res=f"ib{h}"),
+                     IR.ElwMultiply(a=f"e{h}", b=f"ib{h}", res=f"p{h}")]
+        elif chain == 1:
+            # column statistics: m = colsum(x * shared); p = sin(x) + m broadcast over the rows
+            cmds += [IR.ElwMultiply(a=x, b="shared", res=f"t{h}"), IR.Permute(a=f"t{h}", p=[1, 0], res=f"tt{h}"),
+                     IR.Sum(a=f"tt{h}", res=f"n{h}"), IR.View(a=f"n{h}", target_dim=[1, C], res=f"nv{h}"),
+                     IR.Broadcast(a=f"nv{h}", dim=0, r=R, res=f"nb{h}"), IR.Sin(a=x, res=f"s{h}"),
+                     IR.ElwAdd(a=f"s{h}", b=f"nb{h}", res=f"p{h}")]
+        else:
+            # two reductions in a row: n = rowsum(x); total = sum(n); p = x * total
+            cmds += [IR.Sum(a=x, res=f"n{h}"), IR.View(a=f"n{h}", target_dim=[1, R], res=f"nr{h}"),
+                     IR.Sum(a=f"nr{h}", res=f"g{h}"), IR.View(a=f"g{h}", target_dim=[1, 1], res=f"gv{h}"),
+                     IR.Broadcast(a=f"gv{h}", dim=0, r=R, res=f"gb0{h}"), IR.Broadcast(a=f"gb0{h}", dim=1, r=C, res=f"gb{h}"),
+                     IR.ElwMultiply(a=x, b=f"gb{h}", res=f"p{h}")]
+        r = int(rng.integers(5))
+        if r == 0 and not packed:
+            cmds.append(IR.ElwAddEq(s=x, o=f"p{h}"))          # in-place update of this chain's input
+            keep.append(x)
+        elif r == 1:
+            cmds.append(IR.ElwAddEq(s="acc", o=f"p{h}"))      # accumulation across the chains
+        elif r == 2 and h + 1 < heads and not packed:
+            cmds.append(IR.ElwAddEq(s=xs[h + 1], o=f"p{h}"))  # the next chain depends on this one
+        elif r == 3:
+            keep.append(f"n{h}")
+        keep.append(f"p{h}")
+    keep.append("acc")
+    return IR.IRProcedure("main", cmds + [IR.EX()]), sorted(set(keep))

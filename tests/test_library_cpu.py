@@ -388,3 +388,31 @@ def test_training_loop_body_groups_per_head_products():
     body = text[text.index("while "):]
     assert "launch dots_" in body
     assert "[counted:" in text
+
+
+def test_layered_launches_plan_and_compile():
+    """Groups that run the same generated kernels on other buffers share launches (`<kernel>_x<count>`, block layer z
+    for member z).  Over the generator's seeds some programs must be layered, every program must lower, and a
+    layered program's kernels must compile for gfx950."""
+    from fuzz_control import random_layered_program
+    import __graft_entry__ as ge
+    layered = 0
+    compiled = False
+    for seed in range(30):
+        proc, keep = random_layered_program(seed)
+        text = lower_describe(proc, set(keep))
+        counts = [int(c) for c in re.findall(r"launch \w+_x(\d+) \[", text)]
+        assert all(2 <= c <= 16 for c in counts), text
+        for line in text.splitlines():
+            m = re.search(r"launch \w+_x(\d+) \[\w+\] grid=\((\d+),(\d+),(\d+)\)", line)
+            if m:
+                assert m.group(1) == m.group(4), line
+        layered += len(counts)
+        if counts and not compiled:
+            os.environ["ADHIP_CACHE_DIR"] = "off"
+            try:
+                assert "kernels compiled" in ge._compile_check(load_library(), proc, set(keep))
+            finally:
+                del os.environ["ADHIP_CACHE_DIR"]
+            compiled = True
+    assert layered >= 20 and compiled

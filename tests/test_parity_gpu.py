@@ -543,3 +543,20 @@ def test_grouped_products_match_oracle(seed, hip_device):
         ref = ref_dev.get_tensor(k)
         assert not got[k].is_none and got[k].dim == ref.dim, k
         assert_close(got[k].data, ref.data, RED_RTOL * 16, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_layered_launches_match_oracle(seed, hip_device):
+    """The same chain of reductions and element-wise passes on many tensors (tests/fuzz_control.py::
+    random_layered_program): chains whose kernels are the same code run as block layers of shared launches, chains that
+    update their input in place or feed the next chain keep their place."""
+    print(f"[case] layered launches seed {seed}", flush=True)
+    from fuzz_control import random_layered_program
+    proc, keep = random_layered_program(seed)
+    ref_dev = OracleDevice()
+    ref_dev.execute(proc, set(keep))
+    hip_device.execute(proc, set(keep))
+    for k in keep:
+        got, ref = hip_device.get_tensor(k), ref_dev.get_tensor(k)
+        assert not got.is_none and got.dim == ref.dim, k
+        assert_close(got.data, ref.data, RED_RTOL * 8, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
