@@ -1,6 +1,7 @@
 """Parity of the HIP device with the CPU oracle and with the reference's own known answers.
 Everything here goes through the C ABI (`adhip_execute` / `adhip_get_tensor`) on a real GPU."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -534,7 +535,8 @@ def test_grouped_products_match_oracle(seed, hip_device):
     from fuzz_control import random_grouped_products_program
     from adhip.device import lower_describe
     proc, keep = random_grouped_products_program(seed)
-    assert "launch dots_" in lower_describe(proc, set(keep))
+    if os.environ.get("ADHIP_GROUP_DOTS", "1") != "0":
+        assert "launch dots_" in lower_describe(proc, set(keep))
     ref_dev = OracleDevice()
     ref_dev.execute(proc, set(keep))
     hip_device.execute(proc, set(keep))
