@@ -2344,8 +2344,21 @@ struct Lowerer {
                 const int saved = cur_guard;
                 const bool predicated = cur_guard >= 0;  // inside a predicated loop the host cannot decide
                 if (predicated) s.taken_slot = plan->n_flags++;
+                // Bindings are threaded through the arms in program order (shapes follow the last definition in the
+                // text, as the reference's trackers do).  An arm drops the binding of an id that is dead after the
+                // branch; the next arm, which starts from the state before the branch, may still use it, and so may
+                // dead code after the branch: what was bound before the branch stays bound.
+                const std::unordered_map<std::string, Binding> before_branch = env;
+                auto rebind_dropped = [&]() {
+                    for (auto& kv : before_branch) {
+                        if (kv.second.kind == Binding::NONE) continue;
+                        auto it = env.find(kv.first);
+                        if (it == env.end() || it->second.kind == Binding::NONE) env[kv.first] = kv.second;
+                    }
+                };
                 for (auto& arm : c.conds) {
                     std::vector<Step> body;
+                    rebind_dropped();
                     int cb = cond_buffer(arm.first);
                     if (predicated) {
                         s.arm_slots.push_back(plan->n_flags++);
@@ -2360,9 +2373,11 @@ struct Lowerer {
                         s.else_slot = plan->n_flags++;
                         cur_guard = s.else_slot;
                     }
+                    rebind_dropped();
                     lower_block(*c.else_block, s.else_body, false);
                     cur_guard = saved;
                 }
+                rebind_dropped();
                 out.push_back(std::move(s));
             }
             i = j + 1;

@@ -380,9 +380,10 @@ def random_layered_program(seed: int):
                      IR.Broadcast(a=f"nv{h}", dim=0, r=R, res=f"nb{h}"), IR.Sin(a=x, res=f"s{h}"),
                      IR.ElwAdd(a=f"s{h}", b=f"nb{h}", res=f"p{h}")]
         else:
-            # two reductions in a row: n = rowsum(x); total = sum(n); p = x * total
-            cmds += [IR.Sum(a=x, res=f"n{h}"), IR.View(a=f"n{h}", target_dim=[1, R], res=f"nr{h}"),
-                     IR.Sum(a=f"nr{h}", res=f"g{h}"), IR.View(a=f"g{h}", target_dim=[1, 1], res=f"gv{h}"),
+            # two reductions in a row: n = rowsum(x * x); total = sum(n); p = x / total  (positive terms: a total that
+            # cancels to almost nothing would carry the rounding of the whole sum)
+            cmds += [IR.ElwMultiply(a=x, b=x, res=f"q{h}"), IR.Sum(a=f"q{h}", res=f"n{h}"), IR.View(a=f"n{h}", target_dim=[1, R], res=f"nr{h}"),
+                     IR.Sum(a=f"nr{h}", res=f"gs{h}"), IR.Recip(a=f"gs{h}", res=f"g{h}"), IR.View(a=f"g{h}", target_dim=[1, 1], res=f"gv{h}"),
                      IR.Broadcast(a=f"gv{h}", dim=0, r=R, res=f"gb0{h}"), IR.Broadcast(a=f"gb0{h}", dim=1, r=C, res=f"gb{h}"),
                      IR.ElwMultiply(a=x, b=f"gb{h}", res=f"p{h}")]
         r = int(rng.integers(5))

@@ -282,3 +282,36 @@ def predicated_loop_program(dev):
     autodiff.ir_while(pred, body)
     autodiff.execute()
     return {"y": y.val().get(), "z": z.val().get(), "i": i.val().get()}
+
+
+def branch_reads_id_dropped_by_earlier_arm(k_value: float):
+    """`f` is defined before a branch, redefined in the first arm, read in the second arm (which also updates it in
+    place inside a loop) and redefined after the branch, so it is dead once the branch is over: the first arm's
+    definition needs no memory, but the second arm must still find the value from before the branch.  Returns
+    (procedure, keep list, expected values) for a predicate input `k_value` (< 0: first arm, > 0: second arm, 0:
+    neither)."""
+    import numpy as np
+    from adhip import ir as IR
+
+    def mat(name, values, shape):
+        return IR.CreateMat(np.asarray(values, dtype=np.float32), list(shape), name)
+
+    def block(cmds):
+        return IR.IRProcedure("block", cmds)
+
+    f0 = np.array([1.0, 2.0, 3.0, 4.0], dtype=np.float32)
+    y0 = np.array([0.5, -1.0, 2.0, 8.0], dtype=np.float32)
+    top = [mat("f", f0, [4]), mat("y", y0, [4]), mat("g", [0, 0, 0, 0], [4]), mat("k", [k_value], [1]), mat("w", [1.0], [1]),
+           IR.LessZero(a="k", res="p"), IR.MoreZero(a="k", res="q")]
+    arm1 = [IR.CreateConstant(0.5, "c", [4]), IR.ElwMultiply(a="y", b="c", res="f"), IR.ElwAdd(a="f", b="y", res="g")]
+    body = [IR.ElwAddEq(s="f", o="y"), IR.CreateConstant(0.0, "z", [1]), IR.ElwMultiplyEq(s="w", o="z")]
+    arm2 = [IR.While(conditional_var="w", block=block(body)), IR.ElwAdd(a="f", b="f", res="g")]
+    tail = [IR.CreateConstant(3.0, "c3", [4]), IR.ElwMultiply(a="y", b="c3", res="f")]
+    proc = IR.IRProcedure("main", top + [IR.If(conditions=[("p", block(arm1)), ("q", block(arm2))], else_proc=None)] + tail + [IR.EX()])
+    if k_value < 0:
+        g = 0.5 * y0 + y0
+    elif k_value > 0:
+        g = 2.0 * (f0 + y0)
+    else:
+        g = np.zeros(4, dtype=np.float32)
+    return proc, ["f", "g"], {"f": 3.0 * y0, "g": g}

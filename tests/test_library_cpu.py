@@ -416,3 +416,20 @@ def test_layered_launches_plan_and_compile():
                 del os.environ["ADHIP_CACHE_DIR"]
             compiled = True
     assert layered >= 20 and compiled
+
+
+@pytest.mark.parametrize("k_value", [-1.0, 1.0, 0.0])
+def test_branch_arm_reads_id_that_an_earlier_arm_dropped(k_value):
+    """An id that is dead after a branch loses its binding at the end of the first arm; the second arm starts from the
+    state before the branch and must still find it (tests/programs.py::branch_reads_id_dropped_by_earlier_arm).  The
+    oracle agrees with the closed form, and the program lowers."""
+    from oracle.interp import OracleDevice
+    from programs import branch_reads_id_dropped_by_earlier_arm
+    import numpy as np
+    proc, keep, expect = branch_reads_id_dropped_by_earlier_arm(k_value)
+    dev = OracleDevice()
+    dev.execute(proc, set(keep))
+    for k in keep:
+        assert np.array_equal(np.asarray(dev.get_tensor(k).data, dtype=np.float32), expect[k].astype(np.float32)), k
+    text = lower_describe(proc, set(keep))
+    assert "else if" in text and "while" in text

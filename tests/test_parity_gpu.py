@@ -562,3 +562,15 @@ def test_layered_launches_match_oracle(seed, hip_device):
         got, ref = hip_device.get_tensor(k), ref_dev.get_tensor(k)
         assert not got.is_none and got.dim == ref.dim, k
         assert_close(got.data, ref.data, RED_RTOL * 8, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
+
+
+@pytest.mark.parametrize("k_value", [-1.0, 1.0, 0.0])
+def test_branch_arm_reads_id_that_an_earlier_arm_dropped(k_value, hip_device):
+    """tests/programs.py::branch_reads_id_dropped_by_earlier_arm on the device, every path of the branch, bit-exact
+    (small integers and halves only)."""
+    print(f"[case] branch arm reads dropped id, k = {k_value}", flush=True)
+    from programs import branch_reads_id_dropped_by_earlier_arm
+    proc, keep, expect = branch_reads_id_dropped_by_earlier_arm(k_value)
+    hip_device.execute(proc, set(keep))
+    for k in keep:
+        assert_exact(hip_device.get_tensor(k).data, expect[k], k)
