@@ -870,6 +870,8 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         if (epi) {
             auto memo = g.val_memo;
             g.val_memo.clear();
+            auto atom_memo = g.atom_memo;  // index pieces split off x inside the loop are declared in the loop's scope
+            g.atom_memo.clear();
             const int vec_saved = g.vec, lane_saved = g.lane_atom;
             g.vec = 1;
             g.lane_atom = -1;
@@ -886,6 +888,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
             g.vec = vec_saved;
             g.lane_atom = lane_saved;
             g.val_memo = memo;
+            g.atom_memo = atom_memo;
             k.epilogue_done = true;
         }
         // no __restrict__: the result (and a stored operand) may share a buffer with an input it replaces in place

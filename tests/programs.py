@@ -315,3 +315,20 @@ def branch_reads_id_dropped_by_earlier_arm(k_value: float):
     else:
         g = np.zeros(4, dtype=np.float32)
     return proc, ["f", "g"], {"f": 3.0 * y0, "g": g}
+
+
+def reduction_epilogue_with_split_row_index():
+    """y = a.permute(0, 2, 1).sum(-1) + v broadcast over the first dim, a [2,3,4], v [4]: the reduction walks a
+    permuted operand, so its row index is split into two pieces inside the loop, and the element-wise consumer that
+    runs as the reduction's epilogue needs one of the pieces again for v.  Returns (procedure, keep, expected)."""
+    import numpy as np
+    from adhip import ir as IR
+    rng = np.random.default_rng(11)
+    a = rng.integers(-4, 5, (2, 3, 4)).astype(np.float32)
+    v = rng.integers(-4, 5, 4).astype(np.float32)
+    cmds = [IR.CreateMat(a.reshape(-1), [2, 3, 4], "a"), IR.CreateMat(v, [4], "v"),
+            IR.Permute(a="a", p=[0, 2, 1], res="t"), IR.View(a="t", target_dim=[8, 3], res="tv"), IR.Sum(a="tv", res="s"),
+            IR.View(a="v", target_dim=[1, 4], res="vv"), IR.Broadcast(a="vv", dim=0, r=2, res="vb"),
+            IR.View(a="vb", target_dim=[8], res="vf"), IR.ElwAdd(a="s", b="vf", res="y"), IR.EX()]
+    expect = (a.transpose(0, 2, 1).sum(-1) + v[None, :]).reshape(-1)
+    return IR.IRProcedure("main", cmds), ["y"], {"y": expect.astype(np.float32)}

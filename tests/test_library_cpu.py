@@ -433,3 +433,24 @@ def test_branch_arm_reads_id_that_an_earlier_arm_dropped(k_value):
         assert np.array_equal(np.asarray(dev.get_tensor(k).data, dtype=np.float32), expect[k].astype(np.float32)), k
     text = lower_describe(proc, set(keep))
     assert "else if" in text and "while" in text
+
+
+def test_reduction_epilogue_redeclares_index_pieces():
+    """tests/programs.py::reduction_epilogue_with_split_row_index: the oracle matches the closed form, the consumer is
+    fused into the reduction (one kernel), and the kernel compiles for gfx950 (the pieces of the row index that the
+    loop declared are out of scope where the epilogue runs)."""
+    import numpy as np
+    import __graft_entry__ as ge
+    from oracle.interp import OracleDevice
+    from programs import reduction_epilogue_with_split_row_index
+    proc, keep, expect = reduction_epilogue_with_split_row_index()
+    dev = OracleDevice()
+    dev.execute(proc, set(keep))
+    assert np.array_equal(np.asarray(dev.get_tensor("y").data, dtype=np.float32), expect["y"].reshape(-1))
+    text = lower_describe(proc, set(keep))
+    assert len(re.findall(r"^\s*launch", text, re.M)) == 1, text
+    os.environ["ADHIP_CACHE_DIR"] = "off"
+    try:
+        assert "1 kernels compiled" in ge._compile_check(load_library(), proc, set(keep))
+    finally:
+        del os.environ["ADHIP_CACHE_DIR"]

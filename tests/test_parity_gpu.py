@@ -574,3 +574,12 @@ def test_branch_arm_reads_id_that_an_earlier_arm_dropped(k_value, hip_device):
     hip_device.execute(proc, set(keep))
     for k in keep:
         assert_exact(hip_device.get_tensor(k).data, expect[k], k)
+
+
+def test_reduction_epilogue_with_split_row_index(hip_device):
+    """tests/programs.py::reduction_epilogue_with_split_row_index on the device, bit-exact (small integers)."""
+    print("[case] reduction epilogue with split row index", flush=True)
+    from programs import reduction_epilogue_with_split_row_index
+    proc, keep, expect = reduction_epilogue_with_split_row_index()
+    hip_device.execute(proc, set(keep))
+    assert_exact(hip_device.get_tensor("y").data, expect["y"].reshape(-1), "y")
