@@ -123,9 +123,10 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "mlp"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "mlp", "reductions"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
-                         "the known-size reference that hardware byte counters are scaled by")
+                         "the known-size reference that hardware byte counters are scaled by; "
+                         "'reductions': only configs[2]; 'mlp': only configs[3]")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the device path is single-device (run with --gpus 1)", file=sys.stderr)
@@ -150,6 +151,13 @@ def main():
         print(json.dumps({"metric": "plain copy", "value": wlc.algorithmic_bytes / (msc * 1e-3) / 1e9, "unit": "GB/s",
                           "ms_per_step": msc, "bytes_read": 4.0 * rows * cols, "bytes_written": 4.0 * rows * cols,
                           "kernels": profile(pc, 3)}))
+        return
+    if args.workload == "reductions":
+        wl3 = W.reductions(dev, 16384, 4096, seed=0)
+        p3 = compile_resident(dev, wl3)
+        ms3 = timed_runs(p3, args.steps, args.warmup)
+        print(json.dumps({"metric": "reductions forward + backward, f32 [16384,4096]", "value": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
+                          "unit": "GB/s", "ms_per_step": ms3, "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}))
         return
     if args.workload == "mlp":
         print(json.dumps(dict(measure_mlp(dev, args.mlp_iters), metric="fp32 MLP train steps/s")))
