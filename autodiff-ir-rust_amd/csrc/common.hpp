@@ -33,9 +33,12 @@ inline std::string strf(const char* fmt, ...) {
         if (!(cond)) throw ::adhip::Error(::adhip::strf(__VA_ARGS__)); \
     } while (0)
 
+// Product of the dims; sizes come from the caller's command stream, so a product that does not fit is an error of
+// the program, not undefined behaviour here.
 inline int64_t numel(const Shape& s) {
     int64_t n = 1;
-    for (auto d : s) n *= d;
+    for (auto d : s)
+        if (__builtin_mul_overflow(n, d, &n)) throw ::adhip::Error("tensor size overflows 64 bits");
     return n;
 }
 

@@ -5,7 +5,15 @@
 namespace adhip {
 
 namespace {
+// Largest extent, index or repeat count a command may carry (2^40); products of extents are checked where they are formed.
+constexpr int64_t kMaxExtent = int64_t(1) << 40;
+
 struct Reader {
+    int64_t bounded() {
+        const int64_t v = (int64_t)u64();
+        ADHIP_CHECK(v >= -kMaxExtent && v <= kMaxExtent, "index or count %lld out of range", (long long)v);
+        return v;
+    }
     const uint8_t* p;
     const uint8_t* end;
     const uint8_t* base = nullptr;
@@ -26,7 +34,10 @@ struct Reader {
         uint32_t n = u32();
         ADHIP_CHECK(n <= 64, "tensor rank %u too large", n);
         Shape s(n);
-        for (uint32_t i = 0; i < n; ++i) s[i] = (int64_t)u64();
+        for (uint32_t i = 0; i < n; ++i) {
+            s[i] = (int64_t)u64();
+            ADHIP_CHECK(s[i] >= -1 && s[i] <= kMaxExtent, "tensor extent %lld out of range", (long long)s[i]);
+        }
         return s;
     }
 };
@@ -36,6 +47,7 @@ std::unique_ptr<Proc> parse_proc(Reader& r, int depth) {
     auto proc = std::make_unique<Proc>();
     proc->id = r.str();
     uint32_t n = r.u32();
+    ADHIP_CHECK((size_t)(r.end - r.p) >= n, "program stream truncated");  // every command takes at least one byte
     proc->cmds.reserve(n);
     for (uint32_t i = 0; i < n; ++i) {
         Cmd c;
@@ -73,16 +85,16 @@ std::unique_ptr<Proc> parse_proc(Reader& r, int depth) {
             c.a = r.str(); c.dims = r.dims(); c.res = r.str();
             break;
         case T_INDEX:
-            c.a = r.str(); c.i0 = (int64_t)r.u64(); c.i1 = (int64_t)r.u64(); c.res = r.str();
+            c.a = r.str(); c.i0 = r.bounded(); c.i1 = r.bounded(); c.res = r.str();
             break;
         case T_CONCAT:
-            c.a = r.str(); c.b = r.str(); c.i0 = (int64_t)r.u64(); c.res = r.str();
+            c.a = r.str(); c.b = r.str(); c.i0 = r.bounded(); c.res = r.str();
             break;
         case T_PERMUTE:
             c.a = r.str(); c.dims = r.dims(); c.res = r.str();
             break;
         case T_BROADCAST:
-            c.a = r.str(); c.i0 = (int64_t)r.u64(); c.i1 = (int64_t)r.u64(); c.res = r.str();
+            c.a = r.str(); c.i0 = r.bounded(); c.i1 = r.bounded(); c.res = r.str();
             break;
         case T_WHILE:
             c.a = r.str();

@@ -454,3 +454,30 @@ def test_reduction_epilogue_redeclares_index_pieces():
         assert "1 kernels compiled" in ge._compile_check(load_library(), proc, set(keep))
     finally:
         del os.environ["ADHIP_CACHE_DIR"]
+
+
+def test_absurd_sizes_in_a_stream_are_errors():
+    """Sizes in a command stream are the caller's: extents beyond 2^40, element counts that overflow 64 bits and a
+    command count larger than the stream itself are reported, not multiplied blindly or reserved."""
+    import struct
+    big = 1 << 40
+    cases = [
+        [IR.CreateConstant(1.0, "c", [big, big]), IR.CreateConstant(2.0, "d", [big, big]), IR.ElwAdd(a="c", b="d", res="y")],
+        [IR.CreateConstant(1.0, "c", [4, 1]), IR.Broadcast(a="c", dim=1, r=big, res="b1"), IR.View(a="b1", target_dim=[4, big, 1], res="v"),
+         IR.Broadcast(a="v", dim=2, r=big, res="b2"), IR.Exp2(a="b2", res="y")],
+        [IR.CreateConstant(1.0, "c", [big * 2]), IR.Exp2(a="c", res="y")],
+    ]
+    for cmds in cases:
+        with pytest.raises(RuntimeError, match="overflows|out of range|too large"):
+            lower_describe(IR.IRProcedure("main", cmds + [IR.EX()]), {"y"})
+    # a procedure that claims four billion commands
+    blob, keepalive = IR.serialize(IR.IRProcedure("main", [IR.EX()]))
+    name_len = struct.unpack_from("<I", blob, 8)[0]
+    at = 8 + 4 + name_len
+    assert struct.unpack_from("<I", blob, at)[0] == 1
+    forged = blob[:at] + struct.pack("<I", 0xFFFFFFFF) + blob[at + 4:]
+    lib = load_library()
+    buf = ctypes.create_string_buffer(4096)
+    arr = (ctypes.c_char_p * 1)()
+    assert lib.adhip_lower_describe(forged, len(forged), arr, 0, buf, 4096) != 0
+    assert b"truncated" in buf.value
