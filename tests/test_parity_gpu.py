@@ -209,7 +209,7 @@ def test_c_abi_from_cxx():
     assert "cabi_smoke ok" in r.stdout
 
 
-@pytest.mark.parametrize("seed", range(30))
+@pytest.mark.parametrize("seed", list(range(30)) + [369])   # 369: a reduction epilogue that re-uses a split row index
 def test_random_programs_match_oracle(seed, hip_device):
     """Differential test: random graphs of element-wise ops, sums, permutes, views, slices, concats and
     matmuls, forward and backward, device vs oracle."""
@@ -371,7 +371,7 @@ def test_repeated_execute_rebinds_payloads(hip_device):
         assert_close(out["s"].data, v.reshape(2, width).astype(np.float64).sum(1), RED_RTOL * math.sqrt(width), f"width {width}")
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", list(range(40)) + [257, 266, 290, 311])   # the last four: an arm reads an id an earlier arm dropped
 def test_random_control_flow_matches_oracle(seed, hip_device):
     """Random programs with nested counted loops, data-dependent loops and branches (tests/fuzz_control.py):
     integer-valued tensors (which drive every predicate) bit-exact, the others within the element-wise / reduction
