@@ -1,6 +1,8 @@
 #include "codegen.hpp"
 
 #include <algorithm>
+#include <climits>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 
@@ -61,6 +63,19 @@ static __device__ __forceinline__ float adhip_sinf(float x) {
 }
 
 namespace {
+
+// Buffers at least this large (elements) are read and written with non-temporal accesses: they cannot stay in the
+// 256 MiB last-level cache until their next use anyway, and streaming them through it evicts (and, for dirty lines,
+// writes back) whatever the neighbouring kernels could have reused.  ADHIP_NONTEMPORAL_MIB overrides the size in MiB;
+// 0 turns non-temporal accesses off.
+int64_t nontemporal_min_elems() {
+    static const int64_t v = [] {
+        int64_t mib = 256;
+        if (const char* e = getenv("ADHIP_NONTEMPORAL_MIB")) mib = atoll(e);
+        return mib <= 0 ? LLONG_MAX : mib * (int64_t(1) << 20) / 4;
+    }();
+    return v;
+}
 
 // ---------------------------------------------------------------------------------------
 // symbolic integer index arithmetic: c + sum(coef * atom), atoms with known ranges
@@ -329,6 +344,7 @@ struct Gen {
         std::string name = "l" + std::to_string(tmp++);
         Val v;
         const bool ilane = aff_lane(idx);
+        const bool nt = ne >= nontemporal_min_elems();
         if (!ilane && !plane) {
             if (pred.empty()) emit(false, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
             else emit(false, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
@@ -337,7 +353,8 @@ struct Gen {
             Aff base = idx;
             for (auto it2 = base.t.begin(); it2 != base.t.end(); ++it2)
                 if (it2->first == lane_atom) { base.t.erase(it2); break; }
-            std::string addr = strf("*(const float4_t*)(%s + %s)", bp.c_str(), aff_str(base).c_str());
+            std::string addr = nt ? strf("__builtin_nontemporal_load((const float4_t*)(%s + %s))", bp.c_str(), aff_str(base).c_str())
+                                  : strf("*(const float4_t*)(%s + %s)", bp.c_str(), aff_str(base).c_str());
             if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
             else emit(false, strf("float4_t %sv = {0.f, 0.f, 0.f, 0.f}; if (%s) %sv = %s;", name.c_str(), pred.c_str(), name.c_str(), addr.c_str()));
             emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
@@ -471,6 +488,13 @@ struct Gen {
     }
 };
 
+// statement that stores the four floats w[0..3] at `addr` (a float pointer expression), 128 bits wide
+std::string store4_stmt(const std::string& w, const std::string& addr, bool nontemporal) {
+    std::string q = strf("{ float4_t q = {%s[0], %s[1], %s[2], %s[3]}; ", w.c_str(), w.c_str(), w.c_str(), w.c_str());
+    if (nontemporal) return q + "__builtin_nontemporal_store(q, (float4_t*)(" + addr + ")); }";
+    return q + "*(float4_t*)(" + addr + ") = q; }";
+}
+
 std::string join(const std::vector<std::string>& v, const char* indent) {
     std::string s;
     for (auto& x : v) s += std::string(indent) + x + "\n";
@@ -585,17 +609,24 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
 
 }  // namespace
 
+// Rows one block of the column-sum layout covers: 16 (one per wavefront), times the number of rows each wavefront
+// walks, which is 1 until the partial sums would exceed 1024 rows.
+static int64_t elw_colsum_rows_per_wave(int64_t rows) { return std::max<int64_t>(1, (rows + 16 * 1024 - 1) / (16 * 1024)); }
+
 int64_t elw_colsum_tiles(int64_t rows, int64_t cols) {
-    const int64_t bx = (cols / 4 + 255) / 256;
-    int64_t tiles = (1024 + bx - 1) / bx;            // four blocks per CU on 256 CUs
-    tiles = std::min<int64_t>(tiles, 256);                             // bounds the partial sums the second pass reads
-    tiles = std::min<int64_t>(tiles, std::max<int64_t>(rows / 8, 1));  // and at least 8 rows per tile
-    return std::max<int64_t>(tiles, 1);
+    (void)cols;
+    const int64_t per_block = 16 * elw_colsum_rows_per_wave(rows);
+    return std::max<int64_t>(1, (rows + per_block - 1) / per_block);
 }
 
-// Element-wise pass over a [rows, cols] space that also accumulates column sums: a thread owns 4
-// adjacent columns and walks down a tile of rows, so the sums stay in registers; one partial row per
-// tile goes to memory and a small column reduction adds the tiles in a fixed order.
+// Element-wise pass over a [rows, cols] space that also accumulates column sums.  A block is 16 wavefronts; each
+// wavefront takes one row (lane = four adjacent columns, so a wavefront reads and writes 1 KiB runs) and the 16 row
+// results are added through LDS in a fixed order, which leaves one partial row per block row for a second pass.
+// There is no loop over rows in the common case: wavefronts are short-lived, the dispatcher hands out blocks in
+// address order (the 16-row bands of one block row are contiguous in memory), and the chip as a whole streams through
+// every operand front to back -- which is what keeps DRAM pages open for the four output streams.  A thread that
+// walks down a column tile instead (fewer partial rows) was measured 20 % slower on the 3-read + 4-write pass of
+// 8192 x 8192: long-lived loops drift apart and scatter the writes.
 static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members) {
     const int64_t R = spec.rows, C = spec.cols, N = R * C;
     ADHIP_CHECK(C % 4 == 0 && R > 0, "internal: column-sum fusion needs cols %% 4 == 0");
@@ -605,46 +636,54 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     const bool wide = needs_wide(all);
     ElwBody b = elw_body(spec, members, Shape{R, C}, 4, wide);
     Gen& g = b.g;
+    const int64_t K = elw_colsum_rows_per_wave(R);
     const int64_t tiles = elw_colsum_tiles(R, C);
-    const int64_t TR = (R + tiles - 1) / tiles;
     GeneratedKernel k;
     k.kind = "elw_colsum";
     k.entry = spec.name;
     std::string sig = "const int* __restrict__ guard";
     std::vector<Node*> order;
-    // no __restrict__ and no unrolling of the row loop: both make the compiler keep two rows of operands live, and
-    // the lower occupancy costs more than the earlier loads gain
+    // no __restrict__: an output may share its buffer with an input it replaces in place
     for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* o%zu", i); order.push_back(spec.outputs[i]); }
     for (size_t i = 0; i < spec.colsums.size(); ++i) { sig += strf(", float* q%zu", i); order.push_back(spec.colsums[i].partial); }
     for (auto& gb : g.bufs) { sig += strf(", const float* %s", gb.param.c_str()); order.push_back(gb.node); }
     const char* it = g.idx_t();
     const char* sfx = wide ? "ull" : "u";
+    const bool nt_out = N >= nontemporal_min_elems();
     std::string src = kernel_prelude();
-    src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+    src += strf("extern \"C\" __global__ __launch_bounds__(1024) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
     src += "    if (guard && *guard == 0) return;\n";
-    src += strf("    const %s c1 = (%s)blockIdx.x * 256u + threadIdx.x;\n", it, it);
-    src += strf("    if (c1 >= %lld%s) return;\n", (long long)(C / 4), sfx);
-    src += strf("    const %s row0 = (%s)blockIdx.y * %lld%s;\n", it, it, (long long)TR, sfx);
-    src += strf("    const %s row1 = min(row0 + %lld%s, (%s)%lld%s);\n", it, (long long)TR, sfx, it, (long long)R, sfx);
+    src += "    __shared__ float4_t part[16][64];\n";
+    src += "    const unsigned lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;\n";
+    src += strf("    const %s c1 = (%s)blockIdx.x * 64u + lane;\n", it, it);
+    src += strf("    const bool col_ok = c1 < %lld%s;\n", (long long)(C / 4), sfx);
     for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("    float cs%zu[4] = {0.f, 0.f, 0.f, 0.f};\n", i);
-    src += strf("    for (%s c0 = row0; c0 < row1; ++c0) {\n", it);
-    src += join(g.codeA, "        ");
-    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("        float w%zu[4];\n", i);
-    src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
-    src += join(g.codeB, "            ");
-    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
-    for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("            cs%zu[j] += %s;\n", i, b.cs_exprs[i].c_str());
-    src += "        }\n";
+    if (K == 1) src += strf("    {\n        const %s c0 = (%s)blockIdx.y * 16u + wv;\n", it, it);
+    else src += strf("#pragma unroll 1\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n",
+                     (long long)K, it, it, (long long)(16 * K), sfx);
+    src += strf("        if (col_ok && c0 < %lld%s) {\n", (long long)R, sfx);
+    src += join(g.codeA, "            ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            float w%zu[4];\n", i);
+    src += "#pragma unroll\n            for (int j = 0; j < 4; ++j) {\n";
+    src += join(g.codeB, "                ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("                w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
+    for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("                cs%zu[j] += %s;\n", i, b.cs_exprs[i].c_str());
+    src += "            }\n";
     for (size_t i = 0; i < spec.outputs.size(); ++i)
-        src += strf("        { float4_t q = {w%zu[0], w%zu[1], w%zu[2], w%zu[3]}; *(float4_t*)(o%zu + (c0 * %lld%s + c1 * 4u)) = q; }\n", i, i, i, i, i, (long long)C, sfx);
-    src += "    }\n";
-    for (size_t i = 0; i < spec.colsums.size(); ++i)
-        src += strf("    { float4_t q = {cs%zu[0], cs%zu[1], cs%zu[2], cs%zu[3]}; *(float4_t*)(q%zu + ((%s)blockIdx.y * %lld%s + c1 * 4u)) = q; }\n", i, i, i, i, i, it, (long long)C, sfx);
+        src += "            " + store4_stmt(strf("w%zu", i), strf("o%zu + (c0 * %lld%s + c1 * 4u)", i, (long long)C, sfx), nt_out) + "\n";
+    src += "        }\n    }\n";
+    // the 16 wavefronts' sums, added in wavefront order by wavefront (i mod 16) for sum i
+    for (size_t i = 0; i < spec.colsums.size(); ++i) {
+        if (i) src += "    __syncthreads();\n";
+        src += strf("    part[wv][lane] = float4_t{cs%zu[0], cs%zu[1], cs%zu[2], cs%zu[3]};\n    __syncthreads();\n", i, i, i, i);
+        src += strf("    if (wv == %zuu && col_ok) {\n        float4_t s = part[0][lane];\n#pragma unroll\n        for (int r = 1; r < 16; ++r) s += part[r][lane];\n", i % 16);
+        src += strf("        *(float4_t*)(q%zu + ((%s)blockIdx.y * %lld%s + c1 * 4u)) = s;\n    }\n", i, it, (long long)C, sfx);
+    }
     src += "}\n";
     k.source = src;
     k.buffer_args = order;
-    k.block[0] = 256;
-    k.grid[0] = (unsigned)((C / 4 + 255) / 256);
+    k.block[0] = 1024;
+    k.grid[0] = (unsigned)((C / 4 + 63) / 64);
     k.grid[1] = (unsigned)tiles;
     k.chunks = tiles;
     k.bytes = 4.0 * (double)N * (double)spec.outputs.size() + 4.0 * (double)tiles * C * spec.colsums.size();
@@ -717,7 +756,7 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
         src += strf("        w%zu[%s] = %s;\n", i, vec > 1 ? "j" : "0", b.out_exprs[i].c_str());
     src += "    }\n";
     for (size_t i = 0; i < spec.outputs.size(); ++i) {
-        if (vec == 4) src += strf("    { float4_t q = {w%zu[0], w%zu[1], w%zu[2], w%zu[3]}; *(float4_t*)(o%zu + t * 4u) = q; }\n", i, i, i, i, i);
+        if (vec == 4) src += "    " + store4_stmt(strf("w%zu", i), strf("o%zu + t * 4u", i), N >= nontemporal_min_elems()) + "\n";
         else src += strf("    o%zu[t] = w%zu[0];\n", i, i);
     }
     src += "}\n";
@@ -848,9 +887,9 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         Gen& g = b.g;
         k.side_done = side;
         const int64_t RV = R / vec;
-        // threads per row: one wavefront per row (no barrier, no LDS) up to 8192 elements, a whole
-        // block beyond that
-        int T = RV <= 2048 ? 64 : 256;
+        // threads per row: one wavefront per row (no barrier, no LDS) up to 2048 elements, a whole block beyond that
+        // (16384 x 4096: 41 us with a wavefront per row, 38 us with a block per row)
+        int T = RV <= 512 ? 64 : 256;
         if (V < 64 && RV >= 4096) T = 256;
         const int rows_per_block = 256 / T;
         // split long rows over several blocks when there are too few rows to fill the GPU
@@ -924,7 +963,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += strf("            acc[j] += %s;\n        }\n", b.value.c_str());
         if (side)
             for (size_t i = 0; i < b.side_exprs.size(); ++i)
-                src += strf("        { float4_t q = {sv%zu[0], sv%zu[1], sv%zu[2], sv%zu[3]}; *(float4_t*)(w%zu + (%lldu * x + 4u * yv)) = q; }\n", i, i, i, i, i, (long long)R);
+                src += "        " + store4_stmt(strf("sv%zu", i), strf("w%zu + (%lldu * x + 4u * yv)", i, (long long)R), V * R >= nontemporal_min_elems()) + "\n";
         src += "    }\n";
         if (vec == 4) src += "    float s = (acc[0] + acc[1]) + (acc[2] + acc[3]);\n";
         else src += "    float s = acc[0];\n";

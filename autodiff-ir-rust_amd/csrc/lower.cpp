@@ -26,21 +26,24 @@ extern "C" __global__ __launch_bounds__(256) void adhip_copy(const int* __restri
 
 // Dense copy of a strided view whose contiguous source dim (u) is not the innermost dim of the result (v):
 // a 64x64 tile goes through LDS so that both the reads (along u) and the writes (along v) are coalesced.
-// Up to three further dims are batch dims, given by extent and by source / result strides.
+// Up to three further dims are batch dims, given by extent and by source / result strides.  All tiles of all batches
+// are numbered along grid dimension x (the only one that is 2^31 wide).
 extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy(
     const int* __restrict__ guard, float* __restrict__ out, const float* __restrict__ in, long long in_off,
     long long nb0, long long nb1, long long nb2, long long ib0, long long ib1, long long ib2, long long ob0, long long ob1,
-    long long ob2, long long U, long long V, long long in_sv, long long out_su) {
+    long long ob2, long long U, long long V, long long in_sv, long long out_su, long long ut, long long vt) {
     if (guard && *guard == 0) return;
     __shared__ float tile[64][65];
-    long long b = blockIdx.z;
+    long long b = blockIdx.x;   // tile along u fastest, then tile along v, then the batch dims
+    const long long tu = b % ut; b /= ut;
+    const long long tv = b % vt; b /= vt;
     const long long b2 = b % nb2; b /= nb2;
     const long long b1 = b % nb1; b /= nb1;
     const long long b0 = b;
     const float* src = in + in_off + b0 * ib0 + b1 * ib1 + b2 * ib2;
     float* dst = out + b0 * ob0 + b1 * ob1 + b2 * ob2;
     const unsigned tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;
-    const long long u0 = (long long)blockIdx.x * 64, v0 = (long long)blockIdx.y * 64;
+    const long long u0 = tu * 64, v0 = tv * 64;
 #pragma unroll 4
     for (unsigned r = ty; r < 64u; r += 4u) {
         const long long u = u0 + tx, v = v0 + r;
@@ -58,18 +61,20 @@ extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy(
 extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy4(
     const int* __restrict__ guard, float* __restrict__ out, const float* __restrict__ in, long long in_off,
     long long nb0, long long nb1, long long nb2, long long ib0, long long ib1, long long ib2, long long ob0, long long ob1,
-    long long ob2, long long U, long long V, long long in_sv, long long out_su) {
+    long long ob2, long long U, long long V, long long in_sv, long long out_su, long long ut, long long vt) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     if (guard && *guard == 0) return;
     __shared__ float tile[64][65];
-    long long b = blockIdx.z;
+    long long b = blockIdx.x;   // tile along u fastest, then tile along v, then the batch dims
+    const long long tu = b % ut; b /= ut;
+    const long long tv = b % vt; b /= vt;
     const long long b2 = b % nb2; b /= nb2;
     const long long b1 = b % nb1; b /= nb1;
     const long long b0 = b;
     const float* src = in + in_off + b0 * ib0 + b1 * ib1 + b2 * ib2;
     float* dst = out + b0 * ob0 + b1 * ob1 + b2 * ob2;
     const unsigned c4 = threadIdx.x & 15u, rr = threadIdx.x >> 4;
-    const long long u0 = (long long)blockIdx.x * 64, v0 = (long long)blockIdx.y * 64;
+    const long long u0 = tu * 64, v0 = tv * 64;
 #pragma unroll
     for (unsigned r = rr; r < 64u; r += 16u) {
         const long long u = u0 + 4 * c4, v = v0 + r;
@@ -108,32 +113,33 @@ extern "C" __global__ void adhip_flag(int* __restrict__ flags, int slot, int par
 }
 
 // Second pass of column sums that rode along with an element-wise kernel: up to four sums, each the sum over
-// `tiles` rows of its dense partial buffer [tiles][cols], in one launch (blockIdx.y picks the sum).  A block is 64
-// columns x 16 row groups; the row groups are combined through LDS in a fixed order, so the result does not depend
-// on scheduling.
+// `tiles` rows of its dense partial buffer [tiles][cols] (cols a multiple of 4), in one launch (blockIdx.y picks the
+// sum).  A block is 16 four-column groups x 64 row groups; the row groups are combined through LDS by a tree of fixed
+// shape, so the result does not depend on scheduling.
 extern "C" __global__ __launch_bounds__(1024) void adhip_colsum_finalize(
     const int* __restrict__ guard, float* o0, float* o1, float* o2, float* o3, const float* p0, const float* p1,
     const float* p2, const float* p3, long long tiles, long long cols) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
     if (guard && *guard == 0) return;
-    __shared__ float part[16][64];
-    const unsigned lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;
+    __shared__ f4 part[64][16];
+    const unsigned lx = threadIdx.x & 15u, ly = threadIdx.x >> 4;
     const unsigned which = blockIdx.y;
     const float* p = which == 0 ? p0 : (which == 1 ? p1 : (which == 2 ? p2 : p3));
     float* o = which == 0 ? o0 : (which == 1 ? o1 : (which == 2 ? o2 : o3));
-    const long long x = (long long)blockIdx.x * 64 + lx;
-    float acc = 0.0f;
-    if (x < cols) {
-#pragma unroll 8
-        for (long long y = ly; y < tiles; y += 16) acc += p[y * cols + x];
+    const long long x = ((long long)blockIdx.x * 16 + lx) * 4;
+    const bool ok = x < cols;
+    f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (ok) {
+#pragma unroll 4
+        for (long long y = ly; y < tiles; y += 64) acc += *(const f4*)(p + y * cols + x);
     }
     part[ly][lx] = acc;
     __syncthreads();
-    if (ly == 0 && x < cols) {
-        float s4[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) s4[q] = (part[4 * q][lx] + part[4 * q + 1][lx]) + (part[4 * q + 2][lx] + part[4 * q + 3][lx]);
-        o[x] = (s4[0] + s4[1]) + (s4[2] + s4[3]);
-    }
+    if (ly < 16) part[ly][lx] = (part[ly][lx] + part[ly + 16][lx]) + (part[ly + 32][lx] + part[ly + 48][lx]);
+    __syncthreads();
+    if (ly < 4) part[ly][lx] = (part[ly][lx] + part[ly + 4][lx]) + (part[ly + 8][lx] + part[ly + 12][lx]);
+    __syncthreads();
+    if (ly == 0 && ok) *(f4*)(o + x) = (part[0][lx] + part[1][lx]) + (part[2][lx] + part[3][lx]);
 }
 
 // out[i] = slices[0][i] + slices[1][i] + ... in that order, i < n; four elements per thread when n allows.
@@ -1094,6 +1100,13 @@ struct Lowerer {
                         for (int d = 0; d < last; ++d)
                             if (d != u && st.shape[d] > 1) ++nbatch;
                         if (nbatch > 3) continue;
+                        {
+                            // every 64x64 tile of every batch is one block along grid dimension x
+                            int64_t blocks = ((st.shape[u] + 63) / 64) * ((st.shape[last] + 63) / 64);
+                            for (int d = 0; d < last; ++d)
+                                if (d != u && st.shape[d] > 1) blocks *= st.shape[d];
+                            if (blocks > 0x7fffffff) continue;
+                        }
                         TRef region;
                         region.shape = st.shape;
                         Piece whole;
@@ -1369,19 +1382,13 @@ struct Lowerer {
                 spec.rows = G.cs_rows;
                 spec.cols = G.cs_cols;
                 for (auto& cs : G.colsums) {
+                    // partial sums [tiles][cols], added by the fixed second-pass kernel
                     const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
                     Node* S = cs.second;
                     Node* partial = new_node(Op::COPY, Shape{tiles, G.cs_cols}, {}, S->name + ".partial", 0.f, false);
                     partial->root = true;
-                    Node* fin = new_node(Op::SUM, Shape{G.cs_cols}, {tr_permute(tr_node(partial, Shape{tiles, G.cs_cols}), Shape{1, 0})}, S->name, 0.f, false);
-                    fin->root = true;
                     spec.colsums.push_back({cs.first, partial});
-                    ReduceKernelSpec s2;
-                    s2.node = fin;
-                    s2.name = name + "_cs" + std::to_string(gks[g].extra.size());
-                    gks[g].extra.push_back(gen_reduce_kernel(s2, 1));
                     gks[g].extra_nodes.push_back(partial);
-                    gks[g].extra_nodes.push_back(fin);
                 }
                 gks[g].k = gen_elw_kernel(spec, members);
             } else if (G.kind == Group::DOT) {
@@ -1743,13 +1750,7 @@ struct Lowerer {
             GeneratedKernel& k = gks[g].k;
             if (G.kind == Group::ELW && !G.colsums.empty()) {
                 launch_generated(k);
-                if (G.colsums.size() == 1) {
-                    Node* fin = gks[g].extra_nodes[1];
-                    fin->buffer = G.colsums[0].second->buffer;
-                    launch_generated(gks[g].extra[0]);
-                    continue;
-                }
-                // several sums: one launch of the fixed second-pass kernel per four of them
+                // one launch of the fixed second-pass kernel per four sums
                 if (fixed_finalize < 0) fixed_finalize = add_kernel("adhip_colsum_finalize", fixed_kernels_source(), "colsum_finalize");
                 const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
                 for (size_t i0 = 0; i0 < G.colsums.size(); i0 += 4) {
@@ -1761,7 +1762,7 @@ struct Lowerer {
                     lf.grid[1] = (unsigned)cnt;
                     auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: column sum without buffer"); q.buf = x->buffer; return q; };
                     for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(G.colsums[i0 + std::min(j, cnt - 1)].second));
-                    for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(gks[g].extra_nodes[2 * (i0 + std::min(j, cnt - 1))]));
+                    for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(gks[g].extra_nodes[i0 + std::min(j, cnt - 1)]));
                     Arg t; t.kind = Arg::I64; t.iv = tiles; lf.args.push_back(t);
                     t.iv = G.cs_cols; lf.args.push_back(t);
                     lf.label = k.entry + "_cs";
@@ -1820,7 +1821,8 @@ struct Lowerer {
             if (d != u && st.shape[d] > 1) { nb[k] = st.shape[d]; ib[k] = st.stride[d]; ob[k] = dense[d]; ++k; }
         const int64_t U = st.shape[u], V = st.shape[last];
         const int64_t batches = nb[0] * nb[1] * nb[2];
-        ADHIP_CHECK(batches <= 65535 && (V + 63) / 64 <= 65535, "internal: transpose grid too large");
+        const int64_t ut = (U + 63) / 64, vt = (V + 63) / 64;
+        ADHIP_CHECK(ut * vt * batches <= 0x7fffffff, "internal: transpose grid too large");
         // the source region must lie inside the source buffer
         int64_t hi = st.offset;
         for (int d = 0; d < nd; ++d) hi += (st.shape[d] - 1) * st.stride[d];
@@ -1832,13 +1834,11 @@ struct Lowerer {
         Launch l;
         l.kernel = v4 ? fixed_transpose4 : fixed_transpose;
         l.block[0] = 256;
-        l.grid[0] = (unsigned)((U + 63) / 64);
-        l.grid[1] = (unsigned)((V + 63) / 64);
-        l.grid[2] = (unsigned)batches;
+        l.grid[0] = (unsigned)(ut * vt * batches);
         auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: transpose operand without buffer"); q.buf = x->buffer; return q; };
         auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
         l.args = {B(n), B(pc.src.node), I(st.offset), I(nb[0]), I(nb[1]), I(nb[2]), I(ib[0]), I(ib[1]), I(ib[2]),
-                  I(ob[0]), I(ob[1]), I(ob[2]), I(U), I(V), I(st.stride[last]), I(dense[u])};
+                  I(ob[0]), I(ob[1]), I(ob[2]), I(U), I(V), I(st.stride[last]), I(dense[u]), I(ut), I(vt)};
         l.label = "transpose_" + n->name;
         l.bytes = 8.0 * (double)numel(st.shape);
         push_launch(out, l, "transpose");
@@ -2283,11 +2283,46 @@ struct Lowerer {
         };
         if (!scan(body, true)) return false;
         if (!(pos_inc >= 0 && pos_inc < pos_add && pos_add < pos_lt)) return false;
-        // the constants must be the values in effect at those commands: both are defined by
-        // CreateConstant / folding only, checked by `consts` above
+        // The increment and the offset must have one value on every trip at the command that uses them: the id is
+        // either not defined in the body at all (the value it has before the loop), or defined only by CreateConstant
+        // at the top level, every definition with the same value, and -- when the first of them comes after the use --
+        // the same value as before the loop too.
+        auto invariant_constant = [&](const std::string& id, int use_pos, float& value) -> bool {
+            bool ok = true, have = false, defined_before_use = false;
+            float v = 0.f;
+            std::function<void(const Proc&, bool)> defs = [&](const Proc& p, bool top) {
+                for (size_t i = 0; i < p.cmds.size(); ++i) {
+                    const Cmd& c = p.cmds[i];
+                    if (c.tag == T_WHILE) { defs(*c.block, false); continue; }
+                    if (c.tag == T_IF) {
+                        for (auto& arm : c.conds) defs(*arm.second, false);
+                        if (c.else_block) defs(*c.else_block, false);
+                        continue;
+                    }
+                    if (c.res != id) continue;
+                    if (!top || c.tag != T_CREATE_CONSTANT) { ok = false; continue; }
+                    if (have && c.f != v) ok = false;
+                    have = true;
+                    v = c.f;
+                    if ((int)i < use_pos) defined_before_use = true;
+                }
+            };
+            defs(body, true);
+            if (!ok) return false;
+            if (!defined_before_use) {
+                auto it = env.find(id);
+                if (it == env.end() || it->second.kind != Binding::CONST) return false;
+                if (have && it->second.c != v) return false;
+                v = it->second.c;
+            }
+            value = v;
+            return true;
+        };
+        float inc_value = 0.f, add_value = 0.f;
+        if (!invariant_constant(inc->b, pos_inc, inc_value) || !invariant_constant(kadd, pos_add, add_value)) return false;
         step.counter_buf = home(x, 1);
-        step.counter_inc = consts[inc->b];
-        step.counter_add = consts[kadd];
+        step.counter_inc = inc_value;
+        step.counter_add = add_value;
         return true;
     }
 
@@ -2424,8 +2459,9 @@ void describe_steps(const std::vector<Step>& steps, const Plan& p, int indent, s
         switch (s.kind) {
         case Step::LAUNCH: {
             const Launch& l = s.launch;
-            o += pad + strf("launch %s [%s] grid=(%u,%u,%u) block=%u bytes=%.0f flops=%.0f args:", l.label.c_str(),
-                            p.kernels[l.kernel].kind.c_str(), l.grid[0], l.grid[1], l.grid[2], l.block[0], l.bytes, l.flops);
+            o += pad + strf("launch %s [%s] kernel=%s grid=(%u,%u,%u) block=%u bytes=%.0f flops=%.0f args:", l.label.c_str(),
+                            p.kernels[l.kernel].kind.c_str(), p.kernels[l.kernel].entry.c_str(), l.grid[0], l.grid[1], l.grid[2],
+                            l.block[0], l.bytes, l.flops);
             for (const Arg& a : l.args) {
                 if (a.kind == Arg::BUF) o += " " + p.buffers[a.buf].name + "#" + std::to_string(a.buf) + (a.off ? strf("+%lld", (long long)a.off) : std::string());
                 else if (a.kind == Arg::F32) o += strf(" %g", a.fv);

@@ -614,15 +614,18 @@ void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
                 }
                 break;
             }
-            for (size_t i = 0; i < s.arms.size() && i < 64; ++i) read_scalar(p, s.arms[i].first, (int)i);
-            HIP_OK(hipStreamSynchronize(ctx->stream));
+            // the predicates are read 64 at a time (the size of the pinned area); the first arm whose predicate is 1 runs
             bool ran = false;
-            for (size_t i = 0; i < s.arms.size(); ++i) {
-                float v = i < 64 ? ctx->pinned[i] : 0.f;
-                if (v == 1.0f) {
-                    exec_steps(p, s.arms[i].second);
-                    ran = true;
-                    break;
+            for (size_t i0 = 0; i0 < s.arms.size() && !ran; i0 += 64) {
+                const size_t i1 = std::min(s.arms.size(), i0 + 64);
+                for (size_t i = i0; i < i1; ++i) read_scalar(p, s.arms[i].first, (int)(i - i0));
+                HIP_OK(hipStreamSynchronize(ctx->stream));
+                for (size_t i = i0; i < i1; ++i) {
+                    if (ctx->pinned[i - i0] == 1.0f) {
+                        exec_steps(p, s.arms[i].second);
+                        ran = true;
+                        break;
+                    }
                 }
             }
             if (!ran) exec_steps(p, s.else_body);

@@ -27,7 +27,7 @@ def test_fused_elw_full_size(hip_device):
     assert_close(out["L"].data, [y.astype(np.float64).sum()], RED_RTOL * math.sqrt(rows * cols), "L vs sum(y)",
                  scale=float(np.abs(y).astype(np.float64).sum()))
     # sampled rows against the float64 formula
-    idx = np.array([0, 1, 17, 4095, 4096, 8190, 8191])
+    idx = np.array([0, 1, 15, 16, 17, 63, 64, 4095, 4096, 8175, 8176, 8190, 8191])   # block rows are 16 rows
     a64, b64, c64 = a[idx].astype(np.float64), b[idx].astype(np.float64), c[idx].astype(np.float64)
     t = a64 * b64 + c64 + bias.astype(np.float64)
     s = _sigmoid64(t)
@@ -38,7 +38,7 @@ def test_fused_elw_full_size(hip_device):
     assert_close(out["db"].numpy()[idx], ds * a64 + np.cos(b64) * np.cos(c64), 4 * ELW_RTOL, "db rows")
     assert_close(out["dc"].numpy()[idx], ds - np.sin(b64) * np.sin(c64), 4 * ELW_RTOL, "dc rows")
     # dbias = sum over rows of ds: check a few columns completely
-    cj = np.array([0, 5, 4097, 8191])
+    cj = np.array([0, 3, 4, 5, 255, 256, 4097, 8188, 8191])   # a wavefront covers 256 columns, a lane 4
     tcol = a[:, cj].astype(np.float64) * b[:, cj].astype(np.float64) + c[:, cj].astype(np.float64) + bias[cj].astype(np.float64)
     scol = _sigmoid64(tcol)
     assert_close(out["dbias"].numpy()[cj], (scol * (1 - scol)).sum(0), RED_RTOL * math.sqrt(rows), "dbias cols")
@@ -56,10 +56,52 @@ def test_reductions_full_size(hip_device):
     assert_close(out["dx"].data, (4 * x + 1).reshape(-1), 4 * ELW_RTOL, "dx")
 
 
+def _mlp_host_step(x, t, Ws, bs, lr):
+    """One training step of the three-layer network on the host, float32 BLAS products with float64 element-wise
+    arithmetic in between (the products are what the tolerance is sized for).  Returns the loss and the gradients."""
+    B, d3 = t.shape
+    h1 = x @ Ws[0] + bs[0]
+    a1 = (1.0 / (1.0 + np.exp(-h1.astype(np.float64)))).astype(np.float32)
+    h2 = a1 @ Ws[1] + bs[1]
+    a2 = (1.0 / (1.0 + np.exp(-h2.astype(np.float64)))).astype(np.float32)
+    y = a2 @ Ws[2] + bs[2]
+    d = (y - t).astype(np.float64)
+    loss = (d * d).sum() / (B * d3)
+    g = (2.0 * d / (B * d3)).astype(np.float32)                       # dL/dy
+    dW2, db2 = a2.T @ g, g.astype(np.float64).sum(0)
+    g2 = ((g @ Ws[2].T).astype(np.float64) * (a2.astype(np.float64) * (1 - a2.astype(np.float64)))).astype(np.float32)
+    dW1, db1 = a1.T @ g2, g2.astype(np.float64).sum(0)
+    g1 = ((g2 @ Ws[1].T).astype(np.float64) * (a1.astype(np.float64) * (1 - a1.astype(np.float64)))).astype(np.float32)
+    dW0, db0 = x.T @ g1, g1.astype(np.float64).sum(0)
+    dx = g1 @ Ws[0].T
+    return loss, [dW0, dW1, dW2], [db0, db1, db2], dx
+
+
+# rows and columns at the edges of the 256x128 block tile, the 64x64 wave tile and the 32x32 MFMA block
+_EDGE = np.array([0, 1, 31, 32, 63, 64, 127, 128, 255, 256, 257, 2047, 2048, 4000, 4094, 4095])
+
+
+def _check_update(name, got, before, grad, lr, tol, rows=None, cols=None):
+    """`got - before` against `-lr * grad` on the sampled rows x all columns and all rows x sampled columns."""
+    upd = got.astype(np.float64) - before.astype(np.float64)
+    want = -lr * grad.astype(np.float64)
+    scale = float(np.abs(want).max())
+    if upd.ndim == 1:
+        assert_close(upd, want, tol, name, scale=scale)
+        return
+    r = _EDGE[_EDGE < upd.shape[0]] if rows is None else rows
+    c = _EDGE[_EDGE < upd.shape[1]] if cols is None else cols
+    assert_close(upd[r, :], want[r, :], tol, name + " rows", scale=scale)
+    assert_close(upd[:, c], want[:, c], tol, name + " cols", scale=scale)
+
+
 def test_mlp_train_full_size_one_step(hip_device):
-    """One training step at batch 4096, 4096-4096-4096-1024: the loss against a float32 BLAS forward pass
-    on the host (tolerance 1e-5*sqrt(K)), and linearity of the weight update: W0_new - W0 = -lr * dW0 must
-    be reproduced by x^T . (gradient of the first pre-activation), checked on sampled entries."""
+    """One training step at batch 4096, 4096-4096-4096-1024 (the only size at which every product of the step
+    takes the 256x128 block tile: forward k-/n-contiguous, dX with W^T read in place, dW with x^T read in place, the
+    weight updates as epilogues on the accumulators).  Checked against a host step: the loss, and for every weight and
+    bias the update `new - old = -lr * gradient`, on rows and columns at the tile edges; dx likewise.  The update is
+    1e-6 of the weight, so it is compared with the float32 rounding of the sum `old + update` in mind: tolerance
+    2^-23 * |W|_max / |update|_max relative to the update's largest entry, plus 1e-5*sqrt(k) for the product."""
     print("[case] full mlp_train 1 step", flush=True)
     batch, dims, lr = 4096, (4096, 4096, 4096, 1024), 0.01
     wl = W.mlp_train(hip_device, batch, dims, 1, lr=lr, seed=13)
@@ -67,23 +109,49 @@ def test_mlp_train_full_size_one_step(hip_device):
     x, t = wl.inputs["x"], wl.inputs["t"]
     Ws = [wl.inputs[f"W{i}"] for i in range(3)]
     bs = [wl.inputs[f"b{i}"] for i in range(3)]
-    h1 = x @ Ws[0] + bs[0]
-    a1 = 1.0 / (1.0 + np.exp(-h1.astype(np.float64))).astype(np.float32)
-    h2 = a1 @ Ws[1] + bs[1]
-    a2 = 1.0 / (1.0 + np.exp(-h2.astype(np.float64))).astype(np.float32)
-    y = a2 @ Ws[2] + bs[2]
-    d = (y - t).astype(np.float64)
-    loss = (d * d).sum() / (batch * dims[-1])
+    loss, dWs, dbs, dx = _mlp_host_step(x, t, Ws, bs, lr)
     assert_close(out["loss"].data, [loss], RED_RTOL * math.sqrt(4096), "loss")
-    # backward, sampled: dW2 = a2^T . g, g = 2 * d / (B*d3) * 2?  (d*d backward visits both factors)
-    g = (2.0 * d / (batch * dims[-1]))
-    rows_s, cols_s = np.array([0, 100, 4095]), np.array([0, 77, 1023])
-    dW2 = a2[:, rows_s].astype(np.float64).T @ g[:, cols_s]
-    upd = out["W2"].numpy()[np.ix_(rows_s, cols_s)].astype(np.float64) - Ws[2][np.ix_(rows_s, cols_s)].astype(np.float64)
-    assert_close(upd, -lr * dW2, 50 * RED_RTOL * math.sqrt(4096), "W2 update", scale=float(np.abs(lr * dW2).max()))
-    db2 = g.sum(0)
-    updb = out["b2"].numpy().astype(np.float64) - bs[2].astype(np.float64)
-    assert_close(updb, -lr * db2, 50 * RED_RTOL * math.sqrt(4096), "b2 update", scale=float(np.abs(lr * db2).max()))
+    ktol = RED_RTOL * math.sqrt(4096)
+    for li in range(3):
+        for name, got, before, grad in ((f"W{li}", out[f"W{li}"].numpy(), Ws[li], dWs[li]), (f"b{li}", out[f"b{li}"].numpy(), bs[li], dbs[li])):
+            rounding = 2.0 ** -23 * float(np.abs(before).max()) / float(np.abs(lr * grad).max())
+            _check_update(name + " update", got, before, grad, lr, ktol + rounding)
+    got_dx = out["dx"].numpy().astype(np.float64)
+    scale = float(np.abs(dx).max())
+    assert_close(got_dx[_EDGE, :], dx[_EDGE, :], ktol, "dx rows", scale=scale)
+    assert_close(got_dx[:, _EDGE], dx[:, _EDGE], ktol, "dx cols", scale=scale)
+
+
+def test_mlp_train_full_size_ten_iterations(hip_device):
+    """The benchmarked configuration itself: 10 iterations inside the IR for-loop at full size (the unrolled loop
+    replayed as a graph, weights updated in place by product epilogues while the next iteration reads them), against
+    10 host steps.  Weights move by ~1e-5 of their size in total, so they are compared through their total update."""
+    print("[case] full mlp_train 10 iterations", flush=True)
+    batch, dims, lr, iters = 4096, (4096, 4096, 4096, 1024), 0.01, 10
+    wl = W.mlp_train(hip_device, batch, dims, iters, lr=lr, seed=14)
+    out = wl.run()
+    x, t = wl.inputs["x"], wl.inputs["t"]
+    W0 = [wl.inputs[f"W{i}"] for i in range(3)]
+    b0 = [wl.inputs[f"b{i}"] for i in range(3)]
+    Ws = [w.copy() for w in W0]
+    bs = [b.copy() for b in b0]
+    loss = None
+    for it in range(iters):
+        print(f"  host step {it}", flush=True)
+        loss, dWs, dbs, dx = _mlp_host_step(x, t, Ws, bs, lr)
+        for li in range(3):
+            Ws[li] = (Ws[li] - np.float32(lr) * dWs[li]).astype(np.float32)
+            bs[li] = (bs[li].astype(np.float64) - lr * dbs[li]).astype(np.float32)
+    ktol = RED_RTOL * math.sqrt(4096) * iters
+    assert_close(out["loss"].data, [loss], ktol, "loss after 10 iterations")
+    for li in range(3):
+        for name, got, before, after in ((f"W{li}", out[f"W{li}"].numpy(), W0[li], Ws[li]), (f"b{li}", out[f"b{li}"].numpy(), b0[li], bs[li])):
+            total = after.astype(np.float64) - before.astype(np.float64)
+            rounding = iters * 2.0 ** -23 * float(np.abs(before).max()) / float(np.abs(total).max())
+            _check_update(name + " total update", got, before, -total / lr, lr, ktol + rounding)
+    got_dx = out["dx"].numpy().astype(np.float64)
+    scale = float(np.abs(dx).max())
+    assert_close(got_dx[_EDGE, :], dx[_EDGE, :], ktol, "dx of the last iteration, rows", scale=scale)
 
 
 def test_manip_loop_full_size(hip_device):

@@ -1,0 +1,105 @@
+"""Every variant of the 256x128 block tile of the matrix-core kernel, value-checked.
+
+The lowering picks that tile only for outputs of at least 4096 x 4096 (512 tiles), so these cases use such an output
+with a short inner dimension (k = 256 keeps the float64 reference cheap): the four operand layouts (k- or m-contiguous
+A, k- or n-contiguous B: the forward product and the two backward products of reference
+src/graph/ops/dot_product.rs:34-42 read their operands that way), each plain and with an element-wise epilogue on the
+accumulators.  The kernel each case runs is asserted from the plan, so a change of the selection rule cannot turn the
+test into one of another tile without notice.  Tolerance: 1e-5 * sqrt(k) of the largest |a|.|b| dot product."""
+import math
+import re
+
+import numpy as np
+import pytest
+
+from adhip import ir as IR
+from adhip.device import lower_describe
+from parity import RED_RTOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+M = N = 4096
+
+
+def _operands(layout, k, rng):
+    """IR commands that define `a` [M,k] and `b` [k,N] with the requested contiguity, and the arrays as float64."""
+    cmds = []
+    if layout[0] == "k":
+        a = rng.standard_normal((M, k), dtype=np.float32)
+        cmds.append(IR.CreateMat(a.reshape(-1), [M, k], "a"))
+        a64 = a.astype(np.float64)
+    else:
+        at = rng.standard_normal((k, M), dtype=np.float32)
+        cmds += [IR.CreateMat(at.reshape(-1), [k, M], "at"), IR.Permute(a="at", p=[1, 0], res="a")]
+        a64 = at.T.astype(np.float64)
+    if layout[1] == "n":
+        b = rng.standard_normal((k, N), dtype=np.float32)
+        cmds.append(IR.CreateMat(b.reshape(-1), [k, N], "b"))
+        b64 = b.astype(np.float64)
+    else:
+        bt = rng.standard_normal((N, k), dtype=np.float32)
+        cmds += [IR.CreateMat(bt.reshape(-1), [N, k], "bt"), IR.Permute(a="bt", p=[1, 0], res="b")]
+        b64 = bt.T.astype(np.float64)
+    return cmds, a64, b64
+
+
+def _kernels(proc, keep):
+    return re.findall(r"launch dot_\w+ \[dot_mfma\] kernel=(\w+)", lower_describe(proc, set(keep)))
+
+
+@pytest.mark.parametrize("layout", ["kn", "kk", "mn", "mk"])
+@pytest.mark.parametrize("k", [256, 272])
+def test_256_tile_plain(layout, k, hip_device):
+    print(f"[case] 256x128 tile, layout {layout}, k {k}", flush=True)
+    rng = np.random.default_rng(100 + k + sum(map(ord, layout)))
+    cmds, a64, b64 = _operands(layout, k, rng)
+    cmds += [IR.DotProduct(a="a", b="b", res="c"), IR.EX()]
+    proc = IR.IRProcedure("main", cmds)
+    assert _kernels(proc, ["c"]) == [f"adhip_gemm_{layout}_256"]
+    hip_device.execute(proc, {"c"})
+    got = hip_device.get_tensor("c")
+    assert got.dim == [M, N]
+    ref = a64 @ b64
+    scale = float((np.abs(a64) @ np.abs(b64)).max())
+    assert_close(got.data, ref.reshape(-1), RED_RTOL * math.sqrt(k), f"c ({layout})", scale=scale)
+
+
+@pytest.mark.parametrize("layout", ["kn", "kk", "mn", "mk"])
+@pytest.mark.parametrize("kind", ["update", "activation"])
+def test_256_tile_epilogue(layout, kind, hip_device):
+    """`update`: W += -0.01 * (A.B), the product itself never stored (the SGD step on a weight gradient);
+    `activation`: y = sigmoid-like 1 / (1 + exp2(-(A.B + bias))) with the product also kept."""
+    print(f"[case] 256x128 tile epilogue, layout {layout}, {kind}", flush=True)
+    k = 256
+    rng = np.random.default_rng(200 + sum(map(ord, layout + kind)))
+    cmds, a64, b64 = _operands(layout, k, rng)
+    d = a64 @ b64
+    scale = float((np.abs(a64) @ np.abs(b64)).max())
+    tol = RED_RTOL * math.sqrt(k)
+    if kind == "update":
+        w = rng.standard_normal((M, N), dtype=np.float32)
+        cmds += [IR.CreateMat(w.reshape(-1), [M, N], "w"), IR.DotProduct(a="a", b="b", res="d"),
+                 IR.CreateConstant(-0.01, "c", [M, N]), IR.ElwMultiply(a="d", b="c", res="t"), IR.ElwAddEq(s="w", o="t"), IR.EX()]
+        keep = ["w"]
+        proc = IR.IRProcedure("main", cmds)
+        names = _kernels(proc, keep)
+        assert len(names) == 1 and re.fullmatch(rf"adhip_gemm_{layout}_256_e\d+", names[0]), names
+        hip_device.execute(proc, set(keep))
+        got = hip_device.get_tensor("w")
+        assert_close(got.data, (w.astype(np.float64) - 0.01 * d).reshape(-1), tol, "w", scale=scale)
+    else:
+        bias = rng.standard_normal(N).astype(np.float32)
+        cmds += [IR.CreateMat(bias, [N], "bias"), IR.DotProduct(a="a", b="b", res="p"),
+                 IR.View(a="bias", target_dim=[1, N], res="b1"), IR.Broadcast(a="b1", dim=0, r=M, res="bb"),
+                 IR.ElwAdd(a="p", b="bb", res="h"), IR.CreateConstant(-1.0 / 64.0, "m1", [M, N]), IR.ElwMultiply(a="h", b="m1", res="nh"),
+                 IR.Exp2(a="nh", res="e"), IR.CreateConstant(1.0, "one", [M, N]), IR.ElwAdd(a="e", b="one", res="den"),
+                 IR.Recip(a="den", res="y"), IR.EX()]
+        keep = ["y", "p"]
+        proc = IR.IRProcedure("main", cmds)
+        names = _kernels(proc, keep)
+        assert len(names) == 1 and re.fullmatch(rf"adhip_gemm_{layout}_256_e\d+", names[0]), names
+        hip_device.execute(proc, set(keep))
+        assert_close(hip_device.get_tensor("p").data, d.reshape(-1), tol, "p", scale=scale)
+        y = 1.0 / (1.0 + np.exp2(-(d + bias) / 64.0))
+        # |dy/dh| <= 1/64 * 1/4: the product's error is damped; the chain adds a few roundings of its own
+        assert_close(hip_device.get_tensor("y").data, y.reshape(-1), tol * scale / 256.0 + 4e-7, "y", scale=1.0)

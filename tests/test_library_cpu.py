@@ -404,7 +404,7 @@ def test_layered_launches_plan_and_compile():
         counts = [int(c) for c in re.findall(r"launch \w+_x(\d+) \[", text)]
         assert all(2 <= c <= 16 for c in counts), text
         for line in text.splitlines():
-            m = re.search(r"launch \w+_x(\d+) \[\w+\] grid=\((\d+),(\d+),(\d+)\)", line)
+            m = re.search(r"launch \w+_x(\d+) \[\w+\] kernel=\w+ grid=\((\d+),(\d+),(\d+)\)", line)
             if m:
                 assert m.group(1) == m.group(4), line
         layered += len(counts)
