@@ -19,11 +19,17 @@ from .core import STATE, Tensor, Value, concat, constant
 
 class Workload:
     def __init__(self, name: str, outputs: Dict[str, Value], inputs: Dict[str, np.ndarray],
-                 algorithmic_bytes: Optional[float] = None, flops: Optional[float] = None):
+                 algorithmic_bytes: Optional[float] = None, flops: Optional[float] = None,
+                 unfused_bytes: Optional[float] = None):
         self.name = name
         self.outputs = outputs
         self.inputs = inputs
+        # bytes one run has to move when every tensor the caller can observe is read or written exactly once and
+        # nothing else touches memory (the figure throughput is quoted on)
         self.algorithmic_bytes = algorithmic_bytes
+        # the same workload priced pass by pass (forward and backward as separate sweeps over the inputs): not a
+        # bandwidth when divided by the time of a fused run, kept as a named secondary figure only
+        self.unfused_bytes = unfused_bytes
         self.flops = flops
 
     def finish(self):
@@ -99,12 +105,15 @@ def fused_elw(dev, rows: int = 8192, cols: int = 8192, seed: int = 0, backward: 
     L.val().keep()
     outs = {"y": y.val(), "L": L.val()}
     n = rows * cols
-    nbytes = 4.0 * (4 * n + cols)          # forward: read a,b,c,bias; write y
+    unfused = 4.0 * (4 * n + cols)          # forward on its own: read a,b,c,bias; write y
+    fused = unfused + 4.0                   # ... and L
     if backward:
         L.backward()
         outs.update({"da": a.grad(), "db": b.grad(), "dc": c.grad(), "dbias": bias.grad()})
-        nbytes += 4.0 * (6 * n + 2 * cols)  # backward: read a,b,c,bias; write da,db,dc,dbias
-    return Workload("fused_elw", outs, {"a": an, "b": bn, "c": cn, "bias": biasn}, algorithmic_bytes=nbytes)
+        unfused += 4.0 * (6 * n + 2 * cols)  # backward on its own: read a,b,c,bias again; write da,db,dc,dbias
+        fused += 4.0 * (3 * n + cols)        # one pass: the inputs are read once, da,db,dc,dbias written
+    return Workload("fused_elw", outs, {"a": an, "b": bn, "c": cn, "bias": biasn}, algorithmic_bytes=fused,
+                    unfused_bytes=unfused)
 
 
 # ---- config 3: reductions ---------------------------------------------------------------
@@ -124,14 +133,17 @@ def reductions(dev, rows: int = 16384, cols: int = 4096, seed: int = 0, backward
         s.val().keep()
         outs[name] = s.val()
     n = rows * cols
-    nbytes = 3 * 4.0 * n + 4.0 * (rows + cols + 1)
+    small = 4.0 * (rows + cols + 1)
+    unfused = 3 * 4.0 * n + small           # three reductions, x read once by each
+    fused = 4.0 * n + small                 # forward alone: one pass over x yields all three (s2 is the sum of s0)
     if backward:
         s0.backward()
         s1.backward()
         s2.backward()
         outs["dx"] = x.grad()
-        nbytes += 2 * 4.0 * n
-    return Workload("reductions", outs, {"x": xn}, algorithmic_bytes=nbytes)
+        unfused += 2 * 4.0 * n              # read x, write dx
+        fused += 2 * 4.0 * n                # as lowered: a second pass reads x and writes dx (x.sum(0) rides along with it)
+    return Workload("reductions", outs, {"x": xn}, algorithmic_bytes=fused, unfused_bytes=unfused)
 
 
 # ---- config 4: dense MLP training -------------------------------------------------------

@@ -653,7 +653,7 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     std::string src = kernel_prelude();
     src += strf("extern \"C\" __global__ __launch_bounds__(1024) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
     src += "    if (guard && *guard == 0) return;\n";
-    src += "    __shared__ float4_t part[16][64];\n";
+    src += "    __shared__ float4_t part[2][16][64];\n";
     src += "    const unsigned lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;\n";
     src += strf("    const %s c1 = (%s)blockIdx.x * 64u + lane;\n", it, it);
     src += strf("    const bool col_ok = c1 < %lld%s;\n", (long long)(C / 4), sfx);
@@ -672,12 +672,17 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     for (size_t i = 0; i < spec.outputs.size(); ++i)
         src += "            " + store4_stmt(strf("w%zu", i), strf("o%zu + (c0 * %lld%s + c1 * 4u)", i, (long long)C, sfx), nt_out) + "\n";
     src += "        }\n    }\n";
-    // the 16 wavefronts' sums, added in wavefront order by wavefront (i mod 16) for sum i
-    for (size_t i = 0; i < spec.colsums.size(); ++i) {
-        if (i) src += "    __syncthreads();\n";
-        src += strf("    part[wv][lane] = float4_t{cs%zu[0], cs%zu[1], cs%zu[2], cs%zu[3]};\n    __syncthreads();\n", i, i, i, i);
-        src += strf("    if (wv == %zuu && col_ok) {\n        float4_t s = part[0][lane];\n#pragma unroll\n        for (int r = 1; r < 16; ++r) s += part[r][lane];\n", i % 16);
-        src += strf("        *(float4_t*)(q%zu + ((%s)blockIdx.y * %lld%s + c1 * 4u)) = s;\n    }\n", i, it, (long long)C, sfx);
+    // the 16 wavefronts' sums, added in wavefront order; two sums per round through LDS (wavefronts 0 and 1 add them)
+    for (size_t i0 = 0; i0 < spec.colsums.size(); i0 += 2) {
+        const size_t cnt = std::min<size_t>(2, spec.colsums.size() - i0);
+        if (i0) src += "    __syncthreads();\n";
+        for (size_t q = 0; q < cnt; ++q)
+            src += strf("    part[%zu][wv][lane] = float4_t{cs%zu[0], cs%zu[1], cs%zu[2], cs%zu[3]};\n", q, i0 + q, i0 + q, i0 + q, i0 + q);
+        src += "    __syncthreads();\n";
+        src += strf("    if (wv < %zuu && col_ok) {\n        float4_t s = part[wv][0][lane];\n#pragma unroll\n        for (int r = 1; r < 16; ++r) s += part[wv][r][lane];\n", cnt);
+        if (cnt == 2) src += strf("        float* q = wv ? q%zu : q%zu;\n", i0 + 1, i0);
+        else src += strf("        float* q = q%zu;\n", i0);
+        src += strf("        *(float4_t*)(q + ((%s)blockIdx.y * %lld%s + c1 * 4u)) = s;\n    }\n", it, (long long)C, sfx);
     }
     src += "}\n";
     k.source = src;

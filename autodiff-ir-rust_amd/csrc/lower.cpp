@@ -1081,6 +1081,8 @@ struct Lowerer {
         // of the consumer) are first copied densely by the tiled transposing kernel
         if (opt.fuse) {
             std::vector<Node*> work = topo;
+            std::stable_sort(work.begin(), work.end(), [](Node* a, Node* b) { return a->order < b->order; });
+            std::map<std::string, Node*> transposed;  // region of a source node -> its dense copy
             bool added = false;
             for (Node* n : work) {
                 if (!op_is_elw(n->op) || n->transpose) continue;
@@ -1107,19 +1109,36 @@ struct Lowerer {
                                 if (d != u && st.shape[d] > 1) blocks *= st.shape[d];
                             if (blocks > 0x7fffffff) continue;
                         }
-                        TRef region;
-                        region.shape = st.shape;
-                        Piece whole;
-                        whole.lo.assign(st.shape.size(), 0);
-                        whole.hi = st.shape;
-                        whole.view.st = {st};
-                        whole.src = pc.src;
-                        region.pieces.push_back(whole);
-                        Node* T = new_node(Op::COPY, st.shape, {region}, pc.src.node->name + ".t", 0.f, true);
-                        T->root = true;
-                        T->transpose = true;
-                        T->transpose_u = u;
-                        T->order = std::min(T->order, n->order - 0.25);
+                        // a dense copy of exactly this region that must be in memory anyway (Contigious, a kept view)
+                        // is written by the transposing kernel itself; later readers of the region read that copy
+                        const std::string region_key = std::to_string(pc.src.node->id) + "@" + stage_str(st);
+                        Node* T = nullptr;
+                        auto known = transposed.find(region_key);
+                        if (known != transposed.end() && known->second->order < n->order) T = known->second;
+                        if (!T && n->root && n->op == Op::COPY && t.single_full() && pc.view.st.size() == 1 && t.shape == st.shape &&
+                            n->shape == st.shape) {
+                            n->transpose = true;
+                            n->transpose_u = u;
+                            transposed[region_key] = n;
+                            added = true;
+                            continue;
+                        }
+                        if (!T) {
+                            TRef region;
+                            region.shape = st.shape;
+                            Piece whole;
+                            whole.lo.assign(st.shape.size(), 0);
+                            whole.hi = st.shape;
+                            whole.view.st = {st};
+                            whole.src = pc.src;
+                            region.pieces.push_back(whole);
+                            T = new_node(Op::COPY, st.shape, {region}, pc.src.node->name + ".t", 0.f, true);
+                            T->root = true;
+                            T->transpose = true;
+                            T->transpose_u = u;
+                            T->order = std::min(T->order, n->order - 0.25);
+                            transposed[region_key] = T;
+                        }
                         pc.view.st.back() = contiguous_stage(st.shape);
                         pc.src = Src();
                         pc.src.kind = Src::NODE;

@@ -34,6 +34,12 @@
 
 using namespace adhip;
 
+// Scratch memory of adhip_program_enqueue_noalloc: the temporaries of a program (partial sums, slices of split
+// products, intermediate tensors) and its control-flow flags live here instead of in allocations of the program's
+// own.  Every GPU the library runs on holds its own copy of the array, at its own address, until the process ends;
+// host code never uses the array's name as an address, only what hipGetSymbolAddress returned for the current device.
+static __device__ __align__(256) unsigned char adhip_static_scratch[ADHIP_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local std::string g_tls_error;
@@ -97,6 +103,8 @@ struct adhip_ctx {
     std::map<std::string, HostResult> results;
     float* pinned = nullptr;  // small pinned area for predicate read-back
     char* stage = nullptr;    // pinned staging area for small uploads and read-backs
+    unsigned char* static_scratch = nullptr;  // this device's copy of adhip_static_scratch (device address)
+    std::string static_scratch_error;         // why it could not be located, if so
     double compile_ms = 0;
     // Programs kept from earlier adhip_execute calls, most recently used first: a caller that executes the same
     // program again (a training loop) skips lowering, module loading and allocation.
@@ -127,6 +135,12 @@ struct adhip_program {
     std::vector<int> payload_of;         // per plan buffer: index into `payloads`, -1 if none
     size_t device_bytes = 0;
     int* flags = nullptr;            // device flags of predicated blocks
+    // the same buffer table with every temporary, and the flags, placed in the device's static scratch area
+    // (adhip_program_enqueue_noalloc); static_need is what the program takes of it
+    std::vector<void*> static_buf_ptr;
+    int* static_flags = nullptr;
+    size_t static_need = 0;
+    bool use_static = false;         // set for the duration of a run that uses the static area
     hipFunction_t flag_fn = nullptr;
     uint64_t flag_launches = 0;
     std::vector<std::pair<int, std::pair<hipEvent_t, hipEvent_t>>> pending;  // stat index, (start, stop)
@@ -389,6 +403,24 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
             p->device_bytes += (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float);
             p->buf_ptr[i] = q;
         }
+        // where the temporaries and the flags would sit in the static scratch area (256-byte aligned slots)
+        {
+            std::vector<size_t> slot_off(plan.slot_elems.size(), 0);
+            size_t need = 0;
+            for (size_t s = 0; s < plan.slot_elems.size(); ++s) {
+                slot_off[s] = need;
+                need += (((size_t)std::max<int64_t>(plan.slot_elems[s], 1) * sizeof(float)) + 255) & ~size_t(255);
+            }
+            const size_t flags_off = need;
+            need += (((size_t)plan.n_flags * sizeof(int)) + 255) & ~size_t(255);
+            p->static_need = need;
+            if (ctx->static_scratch && need <= (size_t)ADHIP_STATIC_SCRATCH_BYTES) {
+                p->static_buf_ptr = p->buf_ptr;
+                for (size_t i = 0; i < plan.buffers.size(); ++i)
+                    if (plan.buffers[i].kind == PlanBuffer::TEMP) p->static_buf_ptr[i] = ctx->static_scratch + slot_off[(size_t)plan.buffers[i].slot];
+                p->static_flags = (int*)(ctx->static_scratch + flags_off);
+            }
+        }
     } catch (...) {
         program_free(p.release());
         throw;
@@ -449,20 +481,33 @@ void drain_events(adhip_program* p) {
     p->pending.clear();
 }
 
+int* cur_flags(adhip_program* p) { return p->use_static ? p->static_flags : p->flags; }
+void* cur_buf(adhip_program* p, int buf) { return p->use_static ? p->static_buf_ptr[(size_t)buf] : p->buf_ptr[(size_t)buf]; }
+
 void launch(adhip_program* p, const Launch& l) {
     adhip_ctx* ctx = p->ctx;
-    // argument block: guard pointer, then the plan's arguments
-    const void* guard = l.guard >= 0 ? (const void*)(p->flags + l.guard) : nullptr;
-    std::vector<void*> ptrs;
-    std::vector<std::unique_ptr<char[]>> store;
-    ptrs.reserve(l.args.size() + 1);
-    ptrs.push_back((void*)&guard);
-    std::vector<uint64_t> vals(l.args.size());
+    // argument block: guard pointer, then the plan's arguments; on the stack for all but the widest launches, so
+    // that a run allocates nothing on the host either
+    const void* guard = l.guard >= 0 ? (const void*)(cur_flags(p) + l.guard) : nullptr;
+    constexpr size_t kStackArgs = 192;
+    void* ptr_stack[kStackArgs + 1];
+    uint64_t val_stack[kStackArgs];
+    std::vector<void*> ptr_heap;
+    std::vector<uint64_t> val_heap;
+    void** ptrs = ptr_stack;
+    uint64_t* vals = val_stack;
+    if (l.args.size() > kStackArgs) {
+        ptr_heap.resize(l.args.size() + 1);
+        val_heap.resize(l.args.size());
+        ptrs = ptr_heap.data();
+        vals = val_heap.data();
+    }
+    ptrs[0] = (void*)&guard;
     for (size_t i = 0; i < l.args.size(); ++i) {
         const Arg& a = l.args[i];
         switch (a.kind) {
         case Arg::BUF: {
-            char* base = (char*)p->buf_ptr[a.buf];
+            char* base = (char*)cur_buf(p, a.buf);
             void* q = base + a.off * (int64_t)sizeof(float);
             memcpy(&vals[i], &q, sizeof q);
             break;
@@ -471,9 +516,9 @@ void launch(adhip_program* p, const Launch& l) {
         case Arg::I64: { long long v = a.iv; memcpy(&vals[i], &v, sizeof v); break; }
         case Arg::F32: { memcpy(&vals[i], &a.fv, sizeof a.fv); break; }
         }
-        ptrs.push_back(&vals[i]);
+        ptrs[i + 1] = &vals[i];
     }
-    if (p->profiling) {
+    if (p->profiling && !p->use_static) {
         // the launch carries its own start and stop events, which take the kernel's begin and end on the device
         // (events recorded around the launch would include the dispatch gap before it)
         hipEvent_t e0 = get_event(p), e1 = get_event(p);
@@ -481,25 +526,25 @@ void launch(adhip_program* p, const Launch& l) {
                        gz = (uint64_t)l.grid[2] * l.block[2];
         if (gx <= 0xffffffffull && gy <= 0xffffffffull && gz <= 0xffffffffull) {
             HIP_OK(hipExtModuleLaunchKernel(p->fn[l.kernel], (uint32_t)gx, (uint32_t)gy, (uint32_t)gz, l.block[0], l.block[1],
-                                            l.block[2], l.lds_bytes, ctx->stream, ptrs.data(), nullptr, e0, e1, 0));
+                                            l.block[2], l.lds_bytes, ctx->stream, ptrs, nullptr, e0, e1, 0));
         } else {
             HIP_OK(hipEventRecord(e0, ctx->stream));
             HIP_OK(hipModuleLaunchKernel(p->fn[l.kernel], l.grid[0], l.grid[1], l.grid[2], l.block[0], l.block[1], l.block[2],
-                                         l.lds_bytes, ctx->stream, ptrs.data(), nullptr));
+                                         l.lds_bytes, ctx->stream, ptrs, nullptr));
             HIP_OK(hipEventRecord(e1, ctx->stream));
         }
         p->pending.push_back({l.stat, {e0, e1}});
         if (p->pending.size() > 4096) drain_events(p);
     } else {
         HIP_OK(hipModuleLaunchKernel(p->fn[l.kernel], l.grid[0], l.grid[1], l.grid[2], l.block[0], l.block[1], l.block[2],
-                                     l.lds_bytes, ctx->stream, ptrs.data(), nullptr));
+                                     l.lds_bytes, ctx->stream, ptrs, nullptr));
     }
     p->plan->stats[l.stat].launches++;
 }
 
 void launch_flag(adhip_program* p, int slot, int parent, int cond_buf, int mode, int taken) {
-    int* flags = p->flags;
-    const float* cond = cond_buf >= 0 ? (const float*)p->buf_ptr[cond_buf] : nullptr;
+    int* flags = cur_flags(p);
+    const float* cond = cond_buf >= 0 ? (const float*)cur_buf(p, cond_buf) : nullptr;
     void* args[] = {&flags, &slot, &parent, &cond, &mode, &taken};
     HIP_OK(hipModuleLaunchKernel(p->flag_fn, 1, 1, 1, 64, 1, 1, 0, p->ctx->stream, args, nullptr));
     p->flag_launches++;
@@ -507,7 +552,7 @@ void launch_flag(adhip_program* p, int slot, int parent, int cond_buf, int mode,
 
 float read_scalar(adhip_program* p, int buf, int slot) {
     adhip_ctx* ctx = p->ctx;
-    HIP_OK(hipMemcpyAsync(ctx->pinned + slot, p->buf_ptr[buf], sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    HIP_OK(hipMemcpyAsync(ctx->pinned + slot, cur_buf(p, buf), sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
     return 0.f;
 }
 
@@ -515,7 +560,7 @@ float read_scalar(adhip_program* p, int buf, int slot) {
 // single submission afterwards (kernel arguments are fixed device pointers and constants, so the captured
 // nodes never need updating).  Per-kernel profiling and ADHIP_GRAPHS=0 bypass this.
 bool replay_run(adhip_program* p, const std::vector<Step>& steps, size_t first, size_t last) {
-    if (!p->use_graphs || p->profiling || last - first < 8) return false;
+    if (!p->use_graphs || p->profiling || p->use_static || last - first < 8) return false;
     adhip_ctx* ctx = p->ctx;
     auto key = std::make_pair((const void*)&steps, first);
     auto it = p->graphs.find(key);
@@ -583,7 +628,7 @@ void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
                         exec_steps(p, s.body);
                     }
                     read_scalar(p, s.cond_buf, 0);
-                    HIP_OK(hipMemcpyAsync(ctx->pinned + 1, p->flags + s.flag_slot, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+                    HIP_OK(hipMemcpyAsync(ctx->pinned + 1, cur_flags(p) + s.flag_slot, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
                     HIP_OK(hipStreamSynchronize(ctx->stream));
                     int flag;
                     memcpy(&flag, ctx->pinned + 1, sizeof flag);
@@ -735,6 +780,14 @@ int adhip_create(int device_ordinal, adhip_ctx** out) {
         HIP_OK(hipStreamCreate(&ctx->stream));
         HIP_OK(hipHostMalloc((void**)&ctx->pinned, 64 * sizeof(float), hipHostMallocDefault));
         HIP_OK(hipHostMalloc((void**)&ctx->stage, kStageBytes, hipHostMallocDefault));
+        // this device's copy of the static scratch area (the device is current, see hipSetDevice above)
+        void* sp = nullptr;
+        const hipError_t se = hipGetSymbolAddress(&sp, HIP_SYMBOL(adhip_static_scratch));
+        if (se == hipSuccess && sp) ctx->static_scratch = (unsigned char*)sp;
+        else {
+            ctx->static_scratch_error = strf("hipGetSymbolAddress(adhip_static_scratch) failed: %s", hipGetErrorString(se));
+            (void)hipGetLastError();  // the failure concerns adhip_program_enqueue_noalloc only; do not leave it pending
+        }
         *out = ctx.release();
     });
 }
@@ -885,6 +938,24 @@ int adhip_program_run(adhip_program* p) {
 int adhip_program_enqueue(adhip_program* p) {
     if (!p) return 2;
     return guarded(p->ctx, [&] { program_run(p, false); });
+}
+
+int adhip_program_enqueue_noalloc(adhip_program* p) {
+    if (!p) return 2;
+    return guarded(p->ctx, [&] {
+        adhip_ctx* ctx = p->ctx;
+        ADHIP_CHECK(ctx->static_scratch, "adhip_program_enqueue_noalloc: the static scratch area is not available on this device (%s)",
+                    ctx->static_scratch_error.c_str());
+        ADHIP_CHECK(p->static_need <= (size_t)ADHIP_STATIC_SCRATCH_BYTES && !p->static_buf_ptr.empty(),
+                    "adhip_program_enqueue_noalloc: the program needs %zu bytes of scratch memory, the static area holds %zu",
+                    p->static_need, (size_t)ADHIP_STATIC_SCRATCH_BYTES);
+        struct Restore {
+            adhip_program* q;
+            ~Restore() { q->use_static = false; }
+        } restore{p};
+        p->use_static = true;
+        program_run(p, false);
+    });
 }
 
 int adhip_program_sync(adhip_program* p) {

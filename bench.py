@@ -21,10 +21,14 @@ for p in (ROOT, os.path.join(ROOT, "autodiff-ir-rust_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
-# HBM bytes per launch of the fused forward+backward kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
-# plain copy kernel (profiles/fused_elw_8192x8192.hbm_traffic_pmc.txt).  Valid for the 8192x8192 workload only.
-FUSED_ELW_TRAFFIC_BYTES = 805459399 + 1082131484
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
+# Bytes per launch between the L2 caches and the memory fabric, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a plain
+# copy kernel of known size (the summaries under profiles/ give the runs).  These counters sit in front of the 256 MiB
+# last-level cache, so they bound HBM traffic from above.  Valid for the full-size workloads only.
+TRAFFIC_BYTES = {
+    "fused_elw": {"elw_colsum": None},
+    "reductions": {"reduce_row": None, "elw_colsum": None},
+}
 
 
 def timed_runs(prog, steps, warmup):
@@ -57,6 +61,16 @@ def profile(prog, runs):
     return out
 
 
+def hbm_roofline(kernel, algorithmic_bytes, traffic=None, note=None):
+    """Roofline block of one HBM-bound launch site: algorithmic bytes over its average duration."""
+    achieved = algorithmic_bytes / (kernel["avg_ms"] * 1e-3) / 1e9
+    out = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+           "traffic": traffic, "kernel": kernel["kernel"], "avg_ms": kernel["avg_ms"], "algorithmic_bytes": algorithmic_bytes}
+    if note:
+        out["note"] = note
+    return out
+
+
 def compile_resident(dev, workload):
     proc, deps = workload.finish()
     prog = dev.compile(proc, deps)
@@ -75,7 +89,8 @@ def cpu_baseline_fused_elw(rows, cols):
     dt = time.perf_counter() - t0
     out = {"value": wl.algorithmic_bytes / dt / 1e9, "unit": "GB/s", "cores": int(c_kernels().ref_num_threads()),
            "kind": "port", "sample": f"fused_elw forward+backward on {rows}x{cols} f32 ({rows}/8192 of the rows), "
-           f"{dt:.2f} s wall", "seconds": dt}
+           f"{dt:.2f} s wall; rate on the same {wl.algorithmic_bytes:.0f} bytes as the GPU figure (the port itself stores "
+           f"every intermediate, as the reference does)", "seconds": dt}
     # the other two rooflines, on bounded samples: configs[2] whole, and one 2048^3 product of configs[3]'s kind
     import numpy as np
     from oracle.interp import ref_dot
@@ -109,10 +124,16 @@ def measure_mlp(dev, iters):
     dot_ms = sum(k["avg_ms"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
     dot_fl = sum(k["flops"] * k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))
     p4.close()
-    return {"steps_per_s": iters / dt4, "ms_per_train_step": dt4 * 1e3 / iters,
-            "matmul_TFLOPs": dot_fl / (dot_ms * 1e-3) / 1e12 if dot_ms else None,
-            "matmul_frac_of_fp32_mfma_peak": dot_fl / (dot_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS if dot_ms else None,
-            "flops_per_train_step": wl4.flops / iters}
+    tf = dot_fl / (dot_ms * 1e-3) / 1e12 if dot_ms else None
+    out = {"steps_per_s": iters / dt4, "ms_per_train_step": dt4 * 1e3 / iters, "matmul_TFLOPs": tf,
+           "matmul_frac_of_fp32_mfma_peak": tf / FP32_MFMA_PEAK_TFLOPS if tf else None,
+           "flops_per_train_step": wl4.flops / iters}
+    if tf:
+        # all matrix-product launches of the run together: flops over the sum of their durations
+        out["roofline"] = {"bound": "mfma", "achieved": tf, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                           "frac": tf / FP32_MFMA_PEAK_TFLOPS, "traffic": None, "kernel": "dot_mfma (all launches)",
+                           "avg_ms": dot_ms / sum(k["launches_per_run"] for k in k4 if k["kernel"].startswith("dot"))}
+    return out
 
 
 def main():
@@ -123,9 +144,11 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "mlp", "reductions"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by; "
+                         "'streammix': only a bare 3-reads + 4-writes kernel over 8192x8192 f32 (the stream mix of the "
+                         "headline pass with trivial arithmetic and no column sums: what the memory system gives that mix); "
                          "'reductions': only configs[2]; 'mlp': only configs[3]")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -152,6 +175,24 @@ def main():
                           "ms_per_step": msc, "bytes_read": 4.0 * rows * cols, "bytes_written": 4.0 * rows * cols,
                           "kernels": profile(pc, 3)}))
         return
+    if args.workload == "streammix":
+        import numpy as np
+        from adhip import autodiff
+        autodiff.set_device(dev)
+        a, b, c = (autodiff.tensor(np.zeros(rows * cols, dtype=np.float32), [rows, cols]) for _ in range(3))
+        outs = {}
+        for name, t in (("o0", a + b), ("o1", b + c), ("o2", a + c), ("o3", a * b)):
+            t.forward()
+            t.val().keep()
+            outs[name] = t.val()
+        wlm = W.Workload("streammix", outs, {}, algorithmic_bytes=7 * 4.0 * rows * cols)
+        pm = compile_resident(dev, wlm)
+        msm = timed_runs(pm, args.steps, args.warmup)
+        ks = profile(pm, 5)
+        print(json.dumps({"metric": "bare 3-read + 4-write stream mix, f32 [8192,8192]", "value": wlm.algorithmic_bytes / (msm * 1e-3) / 1e9,
+                          "unit": "GB/s", "ms_per_step": msm, "frac_of_hbm_peak": wlm.algorithmic_bytes / (msm * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                          "kernels": ks}))
+        return
     if args.workload == "reductions":
         wl3 = W.reductions(dev, 16384, 4096, seed=0)
         p3 = compile_resident(dev, wl3)
@@ -171,12 +212,7 @@ def main():
     n = rows * cols
     # algorithmic bytes of the dominant launch: a, b, c, bias read once; y, da, db, dc written once
     dom_alg = 4.0 * (7 * n + cols) if dom["kernel"].startswith("elw") else dom["bytes"]
-    achieved = dom_alg / (dom["avg_ms"] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS,
-                "traffic": FUSED_ELW_TRAFFIC_BYTES if dom["kernel"].startswith("elw_colsum") else None,
-                "kernel": dom["kernel"],
-                "avg_ms": dom["avg_ms"], "algorithmic_bytes": dom_alg}
+    roofline = hbm_roofline(dom, dom_alg, TRAFFIC_BYTES["fused_elw"]["elw_colsum"] if dom["kernel"].startswith("elw_colsum") else None)
     prog.close()
 
     extra = {"fused_elw_kernels": kstats}
@@ -204,8 +240,19 @@ def main():
         wl3 = W.reductions(dev, 16384, 4096, seed=0)
         p3 = compile_resident(dev, wl3)
         ms3 = timed_runs(p3, max(5, args.steps // 2), 2)
+        k3 = profile(p3, 3)
+        n3 = 16384 * 4096
         extra["reductions"] = {"ms_per_step": ms3, "GBps": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
-                               "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}
+                               "frac_of_hbm_peak": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                               "algorithmic_bytes": wl3.algorithmic_bytes,
+                               "accounting": "bytes the lowered step moves: x read by the row reduction, x read again and dx "
+                                             "written by the backward pass (x.sum(0) rides along with it), results",
+                               "kernels": k3, "roofline": []}
+        for k in k3:
+            if k["kernel"].startswith("reduce_row:") and k["bytes"] > 1e8:
+                extra["reductions"]["roofline"].append(hbm_roofline(k, 4.0 * (n3 + 16384), TRAFFIC_BYTES["reductions"]["reduce_row"]))
+            if k["kernel"].startswith("elw_colsum:"):
+                extra["reductions"]["roofline"].append(hbm_roofline(k, 4.0 * (2 * n3 + 4096), TRAFFIC_BYTES["reductions"]["elw_colsum"]))
         p3.close()
         # config 5: tensor manipulation + data-dependent loop
         wl5 = W.manip_loop(dev)
@@ -213,7 +260,17 @@ def main():
         t0 = time.perf_counter()
         p5.run()
         ms5 = (time.perf_counter() - t0) * 1e3
-        extra["manip_loop"] = {"ms_total": ms5, "kernels": profile_once(p5)}
+        k5 = profile_once(p5)
+        for k in k5:
+            # r is 151 MB and is rewritten every iteration: it stays in the 256 MiB last-level cache, so the loop
+            # kernels' rates are cache rates, not HBM rates
+            k["GBps"] = k["bytes"] / (k["avg_ms"] * 1e-3) / 1e9
+            k["memory"] = "LLC-resident" if k["launches"] > 1 else "HBM"
+        extra["manip_loop"] = {"ms_total": ms5, "kernels": k5,
+                               "gather_stage": {"algorithmic_bytes": 301989888 + 150994944, "note": "p and q regions read, r and the kept "
+                                                "copy of the gathered tensor written",
+                                                "moved_bytes": sum(k["bytes"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce")),
+                                                "ms": sum(k["avg_ms"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce"))}}
         p5.close()
         # config 4: dense MLP training
         extra["mlp_train"] = measure_mlp(dev, args.mlp_iters)
@@ -239,7 +296,12 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "configs[1]: fused element-wise + broadcast, forward + backward, a,b,c f32 [8192,8192], bias [8192]",
-                   "algorithmic_bytes_per_step": wl.algorithmic_bytes, "frac_of_hbm_peak": value / HBM_PEAK_GBS},
+                   "algorithmic_bytes_per_step": wl.algorithmic_bytes,
+                   "accounting": "a, b, c, bias read once; y, da, db, dc, dbias, L written once (forward and backward are one pass)",
+                   "frac_of_hbm_peak": value / HBM_PEAK_GBS,
+                   "unfused_accounting_bytes": wl.unfused_bytes,
+                   "unfused_accounting_note": "forward and backward priced as separate sweeps; divided by the fused step's time "
+                                              "this is not a bandwidth and is not reported as one"},
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(line))

@@ -155,11 +155,13 @@ class OracleDevice(Device):
         self.result: Dict[str, np.ndarray] = {}
         self.result_shape: Dict[str, List[int]] = {}
         self.op_count = 0
+        self.max_terms = 1   # most terms any single Sum or DotProduct of the last program added up
 
     # -- Device interface ---------------------------------------------------------------
     def execute(self, proc: IR.IRProcedure, dep_ids: Iterable[str]) -> None:
         self.result.clear()
         self.result_shape.clear()
+        self.max_terms = 1
         self.buf: Dict[str, np.ndarray] = {}      # id -> flat f32 buffer
         self.shape: Dict[str, List[int]] = {}     # id -> logical shape (shape tracker)
         self.const: Dict[str, np.float32] = {}    # id -> inline constant
@@ -271,10 +273,12 @@ class OracleDevice(Device):
         elif t == IR.T_SUM:
             a = self._value(cmd.a)
             assert a.ndim == 2, "Sum needs a 2-D operand"
+            self.max_terms = max(self.max_terms, int(a.shape[-1]))
             self._store(cmd.res, list(a.shape[:-1]), ref_reduce_sum(a))
         elif t == IR.T_DOT_PRODUCT:
             a, b = self._value(cmd.a), self._value(cmd.b)
             assert a.ndim == 2 and b.ndim == 2 and a.shape[1] == b.shape[0]
+            self.max_terms = max(self.max_terms, int(a.shape[1]))
             self._store(cmd.res, [a.shape[0], b.shape[1]], ref_dot(a, b))
         elif t == IR.T_CONTIGIOUS:
             self._store(cmd.res, self.shape[cmd.a], self._value(cmd.a))

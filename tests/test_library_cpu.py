@@ -481,3 +481,58 @@ def test_absurd_sizes_in_a_stream_are_errors():
     arr = (ctypes.c_char_p * 1)()
     assert lib.adhip_lower_describe(forged, len(forged), arr, 0, buf, 4096) != 0
     assert b"truncated" in buf.value
+
+
+def _counter_loop(body_extra_before, body_extra_after, k_before=1.0):
+    """x = 0; while (x + (-3)) < 0: <before>; x += k; <after>; with k defined before the loop."""
+    import numpy as np
+    body = body_extra_before + [IR.ElwAddEq(s="x", o="k")] + body_extra_after + [IR.ElwAdd(a="x", b="lim", res="t"), IR.LessZero(a="t", res="cond")]
+    return IR.IRProcedure("main", [
+        IR.CreateMat(np.zeros(1, dtype="float32"), [1], "x"), IR.CreateConstant(k_before, "k", [1]), IR.CreateConstant(-3.0, "lim", [1]),
+        IR.ElwAdd(a="x", b="lim", res="t"), IR.LessZero(a="t", res="cond"),
+        IR.While(conditional_var="cond", block=IRProcBody(body)), IR.EX()])
+
+
+def IRProcBody(cmds):
+    return IR.IRProcedure("body", cmds)
+
+
+def test_counted_loop_needs_an_invariant_increment():
+    """The trip count of a counted loop is computed on the host from the increment; an increment whose constant is
+    redefined inside the body with another value (first trip adds 1, later trips add 2) must not take that form."""
+    plain = _counter_loop([], [])
+    assert "[counted: x += 1;" in lower_describe(plain, {"x"})
+    same_value = _counter_loop([IR.CreateConstant(1.0, "k", [1])], [])
+    assert "[counted: x += 1;" in lower_describe(same_value, {"x"})
+    redefined_after_use = _counter_loop([], [IR.CreateConstant(2.0, "k", [1])])
+    assert "[counted" not in lower_describe(redefined_after_use, {"x"})
+    redefined_before_use = _counter_loop([IR.CreateConstant(2.0, "k", [1])], [])
+    assert "[counted: x += 2;" in lower_describe(redefined_before_use, {"x"})
+    two_values = _counter_loop([IR.CreateConstant(2.0, "k", [1])], [IR.CreateConstant(5.0, "k", [1])])
+    assert "[counted" not in lower_describe(two_values, {"x"})
+    in_a_branch = _counter_loop([], [IR.If(conditions=[("cond", IRProcBody([IR.CreateConstant(2.0, "k", [1])]))], else_proc=None)])
+    assert "[counted" not in lower_describe(in_a_branch, {"x"})
+
+
+@pytest.mark.parametrize("shape,perm,extra", [([5000000, 16], [1, 0], False), ([70000, 16, 16], [0, 2, 1], False),
+                                              ([300, 300, 16, 16], [0, 1, 3, 2], False), ([1024, 128, 16, 16], [0, 1, 3, 2], True)])
+def test_transposing_copies_with_many_batches_lower(shape, perm, extra):
+    """Dense copies of permuted tensors whose batch count or tile count exceeds 65535 (the width of grid dimensions y
+    and z): every tile of every batch is a block along grid dimension x."""
+    import numpy as np
+    n = int(np.prod(shape))
+    cmds = [IR.CreateMat(np.zeros(n, dtype="float32"), shape, "a"), IR.Permute(a="a", p=perm, res="at")]
+    if extra:
+        cmds += [IR.CreateMat(np.zeros(n, dtype="float32"), [shape[i] for i in perm], "b"), IR.ElwAdd(a="at", b="b", res="y")]
+    else:
+        cmds += [IR.Contigious(a="at", res="y")]
+    cmds.append(IR.EX())
+    text = lower_describe(IR.IRProcedure("main", cmds), {"y"})
+    grids = re.findall(r"launch transpose_\S+ \[transpose\] kernel=\w+ grid=\((\d+),(\d+),(\d+)\)", text)
+    assert len(grids) == 1, text
+    gx, gy, gz = map(int, grids[0])
+    assert gy == 1 and gz == 1 and gx < 2 ** 31
+    tiles = 1
+    for d in shape[:-2]:
+        tiles *= d
+    assert gx == tiles * ((shape[-1] + 63) // 64) * ((shape[-2] + 63) // 64)
