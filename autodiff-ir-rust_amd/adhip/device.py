@@ -77,8 +77,8 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.adhip_dot_prod_shape.restype = i32
     lib.adhip_program_create.argtypes = [vp, c.c_char_p, sz, c.POINTER(c.c_char_p), sz, c.POINTER(vp)]
     lib.adhip_program_create.restype = i32
-    for name in ("adhip_program_upload", "adhip_program_run", "adhip_program_enqueue", "adhip_program_sync",
-                 "adhip_program_readback"):
+    for name in ("adhip_program_upload", "adhip_program_run", "adhip_program_enqueue", "adhip_program_enqueue_noalloc",
+                 "adhip_program_sync", "adhip_program_readback"):
         getattr(lib, name).argtypes = [vp]
         getattr(lib, name).restype = i32
     lib.adhip_program_destroy.argtypes = [vp]
@@ -159,6 +159,10 @@ class Program:
     def enqueue(self):
         """Queue one run without waiting for it; `sync()` waits for everything queued."""
         self._call("adhip_program_enqueue")
+
+    def enqueue_noalloc(self):
+        """`enqueue()` with the program's temporaries in the library's static device array: allocates nothing."""
+        self._call("adhip_program_enqueue_noalloc")
 
     def sync(self):
         self._call("adhip_program_sync")
