@@ -425,7 +425,15 @@ class Tensor:
         return self * self.more_than(constant(0.0, self.dim()))
 
     def softmax(self, dim: int):
-        return self.exp() / self.exp().sum(dim)
+        """exp(x - max) / sum(exp(x - max)) along `dim`.  The reference writes `x.exp() / x.exp().sum(dim)`
+        (src/nn/activations/softmax.rs:28-30): its sum loses `dim` and is broadcast back by the trailing-dim rule, so
+        element (i, j) of a square matrix is divided by the sum of row j and any other shape fails to broadcast, and
+        exp overflows beyond x = 88.  The evident intent is followed: normalise along `dim`, with the maximum along
+        `dim` subtracted first.  The maximum carries no gradient: a shift of the argument cancels in the quotient."""
+        d = len(self.dim()) + dim if dim < 0 else dim
+        m = self.max(d).stop_grad().unsqueeze(d)
+        e = (self - m).exp()
+        return e / e.sum(d).unsqueeze(d)
 
     # -- comparisons (src/graph/ops/equality.rs) --------------------------------------
     def equal(self, b: "Tensor"):
@@ -459,6 +467,28 @@ class Tensor:
         node = node.view(list(new_dim))
         permute_to = permute_to[:dim] + permute_to[dim + 1:]
         return node.permute(permute_to)
+
+    def max(self, dim: int):
+        """Largest element along `dim`: the decomposition of `sum` (permute the dim last, view as 2-D, reduce, view
+        and permute back) around the `Max` command.  The reference declares this reduction and never emits it
+        (src/kernel/kernel_decl.rs:75-78, "add max, min" in src/core/ir.rs:49)."""
+        p_dim = len(self.dim())
+        dim = p_dim + dim if dim < 0 else dim
+        permute_to = list(range(p_dim))
+        permute_to[-1] = dim
+        permute_to[dim] = p_dim - 1
+        node = self.permute(permute_to)
+        new_dim = node.dim()
+        node = node.view([-1, new_dim[-1]])
+        node = Tensor(MaxNode(node))
+        new_dim = new_dim[:-1]
+        node = node.view(list(new_dim))
+        permute_to = permute_to[:dim] + permute_to[dim + 1:]
+        return node.permute(permute_to)
+
+    def stop_grad(self):
+        """The same value, as a constant of the backward pass (nothing is propagated to what it was computed from)."""
+        return Tensor(StopGradNode(self))
 
     def mean(self, dim: int):
         p_dim = self.dim()
@@ -846,6 +876,60 @@ class SumNode(Node):
         if self.parent.val() is None:
             return None
         return self._val
+
+
+class MaxNode(Node):
+    """2-D maximum over the last dim: the `Max` command.  Backward: the gradient goes to the positions that hold the
+    maximum, in equal shares when several do."""
+
+    def __init__(self, parent: Tensor):
+        self.parent = parent
+        self._val: Optional[Value] = None
+
+    def forward(self):
+        v = self.val()
+        if v is not None:
+            return v
+        a = self.parent.forward()
+        assert len(self.parent.dim()) == 2, "Reduce (max) node needs dim=2"
+        id = self._val.id if self._val is not None else ir_b_id()
+        ir_b_add(IR.Max(a=a.id, res=id))
+        self._val = Value(a.dim[:-1], id)
+        return self._val.clone()
+
+    def dim(self):
+        return self.parent.dim()[:-1]
+
+    def backward(self, grad: Value):
+        n = self.parent.dim()[-1]
+        m = self._val.to_node().unsqueeze(-1).broadcast(-1, n)
+        at_max = self.parent.equal(m)
+        share = at_max / Tensor(SumNode(at_max)).unsqueeze(-1).broadcast(-1, n)
+        self.parent.n.backward((grad.to_node().unsqueeze(-1).broadcast(-1, n) * share).forward())
+
+    def val(self):
+        if self.parent.val() is None:
+            return None
+        return self._val
+
+
+class StopGradNode(Node):
+    """Passes its parent's value through and ends the backward pass there."""
+
+    def __init__(self, parent: Tensor):
+        self.parent = parent
+
+    def forward(self):
+        return self.parent.forward()
+
+    def dim(self):
+        return self.parent.dim()
+
+    def backward(self, grad: Value):
+        return None
+
+    def val(self):
+        return self.parent.val()
 
 
 class DotProductNode(Node):

@@ -27,6 +27,8 @@ T_SUM, T_DOT_PRODUCT = 9, 10
 T_VIEW, T_INDEX, T_CONCAT, T_PERMUTE, T_BROADCAST, T_CONTIGIOUS = 11, 12, 13, 14, 15, 16
 T_EXP2, T_LOG2, T_SIN, T_RECIP, T_SQRT = 17, 18, 19, 20, 21
 T_WHILE, T_IF, T_EX, T_HEADING = 22, 23, 24, 25
+# not in the reference's enum: the reduction it declares (`ReduceOp::Max`, kernel_decl.rs:75-78) but never emits
+T_MAX = 26
 
 
 class IRCmd:
@@ -106,6 +108,14 @@ class Sum(IRCmd):
     a: str
     res: str
     tag = T_SUM
+
+
+@dataclass
+class Max(IRCmd):
+    """Largest element of every row of a 2-D tensor (same operand rules as `Sum`); NaN only where a whole row is NaN."""
+    a: str
+    res: str
+    tag = T_MAX
 
 
 @dataclass
@@ -318,7 +328,7 @@ def _dims(out: bytearray, dims) -> None:
         out += struct.pack("<Q", int(d))
 
 
-def _proc(out: bytearray, proc: IRProcedure, keepalive: list) -> None:
+def _proc(out: bytearray, proc: IRProcedure, keepalive: list, offsets: Optional[list] = None) -> None:
     _s(out, proc.id)
     out += struct.pack("<I", len(proc.main))
     for cmd in proc.main:
@@ -329,6 +339,8 @@ def _proc(out: bytearray, proc: IRProcedure, keepalive: list) -> None:
             keepalive.append(arr)
             _s(out, cmd.id)
             _dims(out, cmd.dim)
+            if offsets is not None:
+                offsets.append(len(out))
             out += struct.pack("<QQ", arr.ctypes.data if arr.size else 0, arr.size)
         elif t == T_CREATE_CONSTANT:
             out += struct.pack("<f", np.float32(cmd.contents))
@@ -338,7 +350,7 @@ def _proc(out: bytearray, proc: IRProcedure, keepalive: list) -> None:
             _s(out, cmd.a); _s(out, cmd.b); _s(out, cmd.res)
         elif t in (T_ELW_MULTIPLY_EQ, T_ELW_ADD_EQ):
             _s(out, cmd.s); _s(out, cmd.o)
-        elif t in (T_EQUAL_ZERO, T_MORE_ZERO, T_LESS_ZERO, T_SUM, T_CONTIGIOUS,
+        elif t in (T_EQUAL_ZERO, T_MORE_ZERO, T_LESS_ZERO, T_SUM, T_MAX, T_CONTIGIOUS,
                    T_EXP2, T_LOG2, T_SIN, T_RECIP, T_SQRT):
             _s(out, cmd.a); _s(out, cmd.res)
         elif t == T_VIEW:
@@ -353,15 +365,15 @@ def _proc(out: bytearray, proc: IRProcedure, keepalive: list) -> None:
             _s(out, cmd.a); out += struct.pack("<QQ", cmd.dim, cmd.r); _s(out, cmd.res)
         elif t == T_WHILE:
             _s(out, cmd.conditional_var)
-            _proc(out, cmd.block, keepalive)
+            _proc(out, cmd.block, keepalive, offsets)
         elif t == T_IF:
             out += struct.pack("<I", len(cmd.conditions))
             for cond, p in cmd.conditions:
                 _s(out, cond)
-                _proc(out, p, keepalive)
+                _proc(out, p, keepalive, offsets)
             out.append(1 if cmd.else_proc is not None else 0)
             if cmd.else_proc is not None:
-                _proc(out, cmd.else_proc, keepalive)
+                _proc(out, cmd.else_proc, keepalive, offsets)
         elif t == T_EX:
             pass
         elif t == T_HEADING:
@@ -370,14 +382,16 @@ def _proc(out: bytearray, proc: IRProcedure, keepalive: list) -> None:
             raise ValueError(f"unknown IR command {cmd!r}")
 
 
-def serialize(proc: IRProcedure):
+def serialize(proc: IRProcedure, payload_offsets: Optional[list] = None):
     """Return (bytes, keepalive).  `keepalive` holds the float32 arrays whose addresses are
-    embedded in the stream; the caller must keep it alive until `adhip_execute` returns."""
+    embedded in the stream; the caller must keep it alive until `adhip_execute` returns.
+    `payload_offsets`, when given, receives the byte offset of every CreateMat pointer field (the only
+    bytes of the stream that differ from run to run)."""
     out = bytearray()
     out += WIRE_MAGIC
     out += struct.pack("<I", WIRE_VERSION)
     keepalive: list = []
-    _proc(out, proc, keepalive)
+    _proc(out, proc, keepalive, payload_offsets)
     return bytes(out), keepalive
 
 

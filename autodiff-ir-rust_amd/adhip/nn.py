@@ -57,7 +57,7 @@ class Softmax(Module):
         self.dim = dim
 
     def f(self, x):
-        return x.exp() / x.exp().sum(self.dim)
+        return x.softmax(self.dim)
 
 
 class RMS(Module):
@@ -130,9 +130,9 @@ class SGD:
 
 
 # ---- attention / transformer encoder (reference src/nn/transformer.rs) ------------------------------
-# Everything works on 2-D tensors [sequence, features]: DotProduct is 2-D in the IR.  `softmax` is the
-# reference's composition (core.Tensor.softmax: exp(x) / exp(x).sum(dim), the sum broadcast back by the usual
-# trailing-dim rule, no maximum subtracted).
+# Everything works on 2-D tensors [sequence, features]: DotProduct is 2-D in the IR.  `softmax` normalises along the
+# given dim with the maximum subtracted first (core.Tensor.softmax, which also says where the reference's own
+# composition differs).
 
 def Attention(Q: Tensor, K: Tensor, V: Tensor, d_model: int) -> Tensor:
     """dot(softmax(dot(Q, K^T) / sqrt(d_model), -1), V)  (transformer.rs:10-18)."""

@@ -25,6 +25,7 @@ const char* op_name(Op o) {
     case Op::COPY: return "copy";
     case Op::FILL: return "fill";
     case Op::SUM: return "sum";
+    case Op::MAX: return "max";
     case Op::DOT: return "dot";
     }
     return "?";
@@ -38,6 +39,11 @@ static __device__ __forceinline__ float u2f(unsigned u) { return __builtin_bit_c
 static __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+static __device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
 }
 // sin(x) for |x| <= 2^15 in ~15 instructions: x = k*pi + r with pi split in three floats (each fma is exact or rounds
@@ -857,7 +863,17 @@ RedBody red_body(const Node* n, RedLayout layout, int vec, bool wide, const std:
 
 GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks) {
     const Node* n = spec.node;
-    ADHIP_CHECK(n->op == Op::SUM && n->in.size() == 1 && n->in[0].shape.size() == 2, "internal: malformed reduction");
+    ADHIP_CHECK(op_is_reduce(n->op) && n->in.size() == 1 && n->in[0].shape.size() == 2, "internal: malformed reduction");
+    // Sum and Max share everything but the combining step: `acc (+)= v`, the identity lanes start from, and how two
+    // partial results are merged.  fmaxf returns the other operand when one is NaN, so a row's maximum is NaN only
+    // if all of it is.
+    const bool mx = n->op == Op::MAX;
+    const char* ident = mx ? "-__builtin_inff()" : "0.0f";
+    auto comb = [&](const std::string& a, const std::string& b) { return mx ? "fmaxf(" + a + ", " + b + ")" : a + " + " + b; };
+    auto comb4 = [&](const std::string& a, const std::string& b, const std::string& c, const std::string& d) {
+        return mx ? "fmaxf(fmaxf(" + a + ", " + b + "), fmaxf(" + c + ", " + d + "))" : "(" + a + " + " + b + ") + (" + c + " + " + d + ")";
+    };
+    const char* wave_comb = mx ? "wave_max" : "wave_sum";
     const int64_t V = n->in[0].shape[0], R = n->in[0].shape[1];
     ADHIP_CHECK(V > 0 && R > 0, "internal: empty reduction");
     std::vector<Node*> roots{const_cast<Node*>(n)};
@@ -949,7 +965,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += strf("    const %s x = (%s)blockIdx.x * %du + threadIdx.x / %du;\n", g.idx_t(), g.idx_t(), rows_per_block, T);
         src += "    const unsigned chunk = blockIdx.y;\n";
         src += strf("    const bool row_ok = x < %lld%s;\n", (long long)V, wide ? "ull" : "u");
-        src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = 0.0f;\n", vec, vec);
+        src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = %s;\n", vec, vec, ident);
         if (chunks == 1) {
             // constant trip count: the loads of several iterations can be in flight together
             src += strf("    if (row_ok)\n#pragma unroll 8\n    for (%s yv = lane; yv < %lldu; yv += %du) {\n", g.idx_t(), (long long)RV, T);
@@ -965,12 +981,12 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += join(g.codeB, "            ");
         if (side)
             for (size_t i = 0; i < b.side_exprs.size(); ++i) src += strf("            sv%zu[j] = %s;\n", i, b.side_exprs[i].c_str());
-        src += strf("            acc[j] += %s;\n        }\n", b.value.c_str());
+        src += strf("            acc[j] = %s;\n        }\n", comb("acc[j]", b.value).c_str());
         if (side)
             for (size_t i = 0; i < b.side_exprs.size(); ++i)
                 src += "        " + store4_stmt(strf("sv%zu", i), strf("w%zu + (%lldu * x + 4u * yv)", i, (long long)R), V * R >= nontemporal_min_elems()) + "\n";
         src += "    }\n";
-        if (vec == 4) src += "    float s = (acc[0] + acc[1]) + (acc[2] + acc[3]);\n";
+        if (vec == 4) src += "    float s = " + comb4("acc[0]", "acc[1]", "acc[2]", "acc[3]") + ";\n";
         else src += "    float s = acc[0];\n";
         std::string epilogue;
         if (epi) {
@@ -978,14 +994,14 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
             for (size_t i = 0; i < epi_exprs.size(); ++i) epilogue += strf("        e%zu[x] = %s;\n", i, epi_exprs[i].c_str());
         }
         if (T == 64) {
-            src += "    s = wave_sum(s);\n";
+            src += strf("    s = %s(s);\n", wave_comb);
             src += "    if (lane == 0 && row_ok) {\n        const float sum_value = s;\n";
             src += strf("        out[(%s)chunk * %lldu + x] = sum_value;\n", g.idx_t(), (long long)V);
             src += epilogue + "    }\n";
         } else {
-            src += "    __shared__ float part[4];\n    s = wave_sum(s);\n";
+            src += strf("    __shared__ float part[4];\n    s = %s(s);\n", wave_comb);
             src += "    if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = s;\n    __syncthreads();\n";
-            src += "    if (threadIdx.x == 0 && row_ok) {\n        const float sum_value = (part[0] + part[1]) + (part[2] + part[3]);\n";
+            src += "    if (threadIdx.x == 0 && row_ok) {\n        const float sum_value = " + comb4("part[0]", "part[1]", "part[2]", "part[3]") + ";\n";
             src += strf("        out[(%s)chunk * %lldu + x] = sum_value;\n", g.idx_t(), (long long)V);
             src += epilogue + "    }\n";
         }
@@ -1028,23 +1044,23 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += strf("    const %s xv = (%s)blockIdx.x * 64u + lx;\n", g.idx_t(), g.idx_t());
         src += "    const unsigned chunk = blockIdx.y;\n";
         src += strf("    const bool col_ok = xv < %lld%s;\n", (long long)XV, wide ? "ull" : "u");
-        src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = 0.0f;\n", vec, vec);
+        src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = %s;\n", vec, vec, ident);
         src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)R);
         src += strf("    if (col_ok)\n#pragma unroll 8\n    for (%s y = (%s)chunk * %lldu + ly; y < y_end; y += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, YG);
         src += join(g.codeA, "        ");
         if (vec > 1) src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
         else src += "        { const int j = 0;\n";
         src += join(g.codeB, "            ");
-        src += strf("            acc[j] += %s;\n        }\n    }\n", b.value.c_str());
+        src += strf("            acc[j] = %s;\n        }\n    }\n", comb("acc[j]", b.value).c_str());
         src += strf("#pragma unroll\n    for (int j = 0; j < %d; ++j) part[ly][lx][j] = acc[j];\n    __syncthreads();\n", vec);
         src += "    if (ly == 0 && col_ok) {\n";
         src += strf("#pragma unroll\n        for (int j = 0; j < %d; ++j) {\n", vec);
         if (YG == 4)
-            src += "            float s = (part[0][lx][j] + part[1][lx][j]) + (part[2][lx][j] + part[3][lx][j]);\n";
+            src += "            float s = " + comb4("part[0][lx][j]", "part[1][lx][j]", "part[2][lx][j]", "part[3][lx][j]") + ";\n";
         else {
             src += "            float s4[4];\n#pragma unroll\n            for (int q = 0; q < 4; ++q)\n";
-            src += "                s4[q] = (part[4 * q][lx][j] + part[4 * q + 1][lx][j]) + (part[4 * q + 2][lx][j] + part[4 * q + 3][lx][j]);\n";
-            src += "            float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);\n";
+            src += "                s4[q] = " + comb4("part[4 * q][lx][j]", "part[4 * q + 1][lx][j]", "part[4 * q + 2][lx][j]", "part[4 * q + 3][lx][j]") + ";\n";
+            src += "            float s = " + comb4("s4[0]", "s4[1]", "s4[2]", "s4[3]") + ";\n";
         }
         src += strf("            out[(%s)chunk * %lldu + xv * %du + j] = s;\n        }\n    }\n}\n", g.idx_t(), (long long)V, vec);
         k.buffer_args = order;

@@ -23,11 +23,13 @@ enum class Op : uint8_t {
     ADD, MUL, EXP2, LOG2, SIN, RECIP, SQRT, EQ0, GT0, LT0, COPY, FILL,
     // kernels of their own
     SUM,  // [V,R] -> [V]
+    MAX,  // [V,R] -> [V], the largest element of every row (NaN only where a whole row is NaN)
     DOT,  // [M,K] x [K,N] -> [M,N]
 };
 
 inline bool op_is_leaf(Op o) { return o == Op::LIVEIN || o == Op::UPLOAD; }
 inline bool op_is_elw(Op o) { return o >= Op::ADD && o <= Op::FILL; }
+inline bool op_is_reduce(Op o) { return o == Op::SUM || o == Op::MAX; }
 inline bool op_is_transcendental(Op o) { return o == Op::EXP2 || o == Op::LOG2 || o == Op::SIN; }
 const char* op_name(Op o);
 

@@ -77,7 +77,7 @@ std::unique_ptr<Proc> parse_proc(Reader& r, int depth) {
         case T_ELW_MULTIPLY_EQ: case T_ELW_ADD_EQ:
             c.a = r.str(); c.b = r.str(); c.res = c.a;
             break;
-        case T_EQUAL_ZERO: case T_MORE_ZERO: case T_LESS_ZERO: case T_SUM: case T_CONTIGIOUS:
+        case T_EQUAL_ZERO: case T_MORE_ZERO: case T_LESS_ZERO: case T_SUM: case T_MAX: case T_CONTIGIOUS:
         case T_EXP2: case T_LOG2: case T_SIN: case T_RECIP: case T_SQRT:
             c.a = r.str(); c.res = r.str();
             break;
@@ -138,7 +138,7 @@ const char* tag_name(Tag t) {
     static const char* names[] = {"CreateMat", "CreateConstant", "ElwMultiply", "ElwAdd", "ElwMultiplyEq",
                                   "ElwAddEq", "EqualZero", "MoreZero", "LessZero", "Sum", "DotProduct", "View",
                                   "Index", "Concat", "Permute", "Broadcast", "Contigious", "Exp2", "Log2", "Sin",
-                                  "Recip", "Sqrt", "While", "If", "EX", "Heading"};
+                                  "Recip", "Sqrt", "While", "If", "EX", "Heading", "Max"};
     return t < T_COUNT ? names[t] : "?";
 }
 

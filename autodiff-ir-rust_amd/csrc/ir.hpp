@@ -13,6 +13,9 @@ enum Tag : uint8_t {
     T_CREATE_MAT = 0, T_CREATE_CONSTANT, T_ELW_MULTIPLY, T_ELW_ADD, T_ELW_MULTIPLY_EQ, T_ELW_ADD_EQ,
     T_EQUAL_ZERO, T_MORE_ZERO, T_LESS_ZERO, T_SUM, T_DOT_PRODUCT, T_VIEW, T_INDEX, T_CONCAT, T_PERMUTE,
     T_BROADCAST, T_CONTIGIOUS, T_EXP2, T_LOG2, T_SIN, T_RECIP, T_SQRT, T_WHILE, T_IF, T_EX, T_HEADING,
+    // Not a variant of the reference's enum: the reduction it declares but never emits (ReduceOp::Max, reference
+    // src/kernel/kernel_decl.rs:75-78; "add max, min" in src/core/ir.rs:49).  Same operand rules as Sum.
+    T_MAX,
     T_COUNT
 };
 

@@ -387,7 +387,7 @@ struct Lowerer {
             st.views[c.res] = e;
             return;
         }
-        case T_SUM: case T_DOT_PRODUCT: {
+        case T_SUM: case T_MAX: case T_DOT_PRODUCT: {
             AvEntry a = av_canon(st, c.a);
             std::string key = std::string(tag_name(c.tag)) + "(" + a.text;
             std::set<std::string> roots = a.roots;
@@ -747,11 +747,12 @@ struct Lowerer {
             bind_val(c.res, n, sh);
             return;
         }
-        case T_SUM: {
+        case T_SUM: case T_MAX: {
             TRef ta = operand(c.a);
-            ADHIP_CHECK(ta.shape.size() == 2, "Sum: operand '%s' has shape %s, expected 2-D", c.a.c_str(), shape_str(ta.shape).c_str());
+            ADHIP_CHECK(ta.shape.size() == 2, "%s: operand '%s' has shape %s, expected 2-D", tag_name(c.tag), c.a.c_str(), shape_str(ta.shape).c_str());
+            ADHIP_CHECK(c.tag == T_SUM || ta.shape[1] > 0, "Max: operand '%s' has no elements to take the largest of", c.a.c_str());
             Shape sh{ta.shape[0]};
-            Node* n = new_node(Op::SUM, sh, {ta}, c.res);
+            Node* n = new_node(c.tag == T_SUM ? Op::SUM : Op::MAX, sh, {ta}, c.res);
             bind_val(c.res, n, sh);
             return;
         }
@@ -1046,7 +1047,7 @@ struct Lowerer {
         for (auto& w : wanted) w.second->root = true;
         for (size_t i = 0; i < topo.size(); ++i) {
             Node* n = topo[i];
-            if (n->op == Op::SUM || n->op == Op::DOT || n->force_root) n->root = true;
+            if (op_is_reduce(n->op) || n->op == Op::DOT || n->force_root) n->root = true;
             if (!opt.fuse && op_is_elw(n->op)) n->root = true;
             if (numel(n->shape) == 0) n->root = false;
         }
@@ -1217,7 +1218,7 @@ struct Lowerer {
             if (chosen < 0) {
                 Group g;
                 g.n = numel(r->shape);
-                g.kind = r->op == Op::SUM ? Group::SUM : (r->op == Op::DOT ? Group::DOT : (r->transpose ? Group::TRANSPOSE : Group::ELW));
+                g.kind = op_is_reduce(r->op) ? Group::SUM : (r->op == Op::DOT ? Group::DOT : (r->transpose ? Group::TRANSPOSE : Group::ELW));
                 groups.push_back(g);
                 chosen = (int)groups.size() - 1;
             }
@@ -1510,7 +1511,7 @@ struct Lowerer {
                     const int64_t V = n->shape[0], C = gks[g].k.chunks;
                     Node* partial = new_node(Op::COPY, Shape{C, V}, {}, n->name + ".partial", 0.f, false);
                     partial->root = true;
-                    Node* fin = new_node(Op::SUM, Shape{V}, {tr_permute(tr_node(partial, Shape{C, V}), Shape{1, 0})}, n->name, 0.f, false);
+                    Node* fin = new_node(n->op, Shape{V}, {tr_permute(tr_node(partial, Shape{C, V}), Shape{1, 0})}, n->name, 0.f, false);
                     fin->root = true;
                     ReduceKernelSpec s2;
                     s2.node = fin;
@@ -1665,7 +1666,7 @@ struct Lowerer {
                                 // at the position it is about to write (s = Sum(f(x, s broadcast along the reduced
                                 // dim))): the block that owns an output element loads before it stores, and a
                                 // chunked reduction stores in its second pass
-                                const bool own_sum = groups[g].kind == Group::SUM && m == groups[g].members[0] && m->op == Op::SUM &&
+                                const bool own_sum = groups[g].kind == Group::SUM && m == groups[g].members[0] && op_is_reduce(m->op) &&
                                                      m->in[0].shape.size() == 2 &&
                                                      reads_at_kept_coordinate_only(m, old, m->in[0].shape[0], m->in[0].shape[1]);
                                 if (!own_sum) direct = false;

@@ -22,7 +22,10 @@ namespace adhip_host {
 
 enum Tag : uint8_t {
     CreateMat = 0, CreateConstant, ElwMultiply, ElwAdd, ElwMultiplyEq, ElwAddEq, EqualZero, MoreZero, LessZero, Sum,
-    DotProduct, View, Index, Concat, Permute, Broadcast, Contigious, Exp2, Log2, Sin, Recip, Sqrt, While, If, EX, Heading
+    DotProduct, View, Index, Concat, Permute, Broadcast, Contigious, Exp2, Log2, Sin, Recip, Sqrt, While, If, EX, Heading,
+    // not a variant of the reference's enum: the row maximum it declares (ReduceOp::Max, reference
+    // src/kernel/kernel_decl.rs:75-78) but never emits; same fields as Sum
+    Max
 };
 
 struct IRProcedure;
@@ -90,6 +93,13 @@ inline IRCmd if_(std::string cond, IRProcedure then_block, const IRProcedure* el
     if (else_block) c.else_proc = std::make_shared<IRProcedure>(*else_block);
     return c;
 }
+inline IRCmd if_arms(std::vector<std::pair<std::string, IRProcedure>> arms, const IRProcedure* else_block = nullptr) {
+    IRCmd c; c.tag = If;
+    for (auto& arm : arms) c.conditions.emplace_back(std::move(arm.first), std::make_shared<IRProcedure>(std::move(arm.second)));
+    if (else_block) c.else_proc = std::make_shared<IRProcedure>(*else_block);
+    return c;
+}
+inline IRCmd heading(std::string cmt) { IRCmd c; c.tag = Heading; c.cmt = std::move(cmt); return c; }
 inline IRCmd ex() { IRCmd c; c.tag = EX; return c; }
 
 namespace detail {
@@ -98,13 +108,17 @@ inline void u32(std::vector<uint8_t>& o, uint32_t v) { put(o, &v, 4); }
 inline void u64(std::vector<uint8_t>& o, uint64_t v) { put(o, &v, 8); }
 inline void str(std::vector<uint8_t>& o, const std::string& s) { u32(o, (uint32_t)s.size()); put(o, s.data(), s.size()); }
 inline void dims(std::vector<uint8_t>& o, const std::vector<uint64_t>& d) { u32(o, (uint32_t)d.size()); for (auto v : d) u64(o, v); }
-inline void proc(std::vector<uint8_t>& o, const IRProcedure& p) {
+inline void proc(std::vector<uint8_t>& o, const IRProcedure& p, std::vector<size_t>* payload_offsets) {
     str(o, p.id);
     u32(o, (uint32_t)p.main.size());
     for (const IRCmd& c : p.main) {
         o.push_back((uint8_t)c.tag);
         switch (c.tag) {
-        case CreateMat: str(o, c.res); dims(o, c.dim); u64(o, (uint64_t)(uintptr_t)c.contents->data()); u64(o, c.contents->size()); break;
+        case CreateMat:
+            str(o, c.res); dims(o, c.dim);
+            if (payload_offsets) payload_offsets->push_back(o.size());
+            u64(o, (uint64_t)(uintptr_t)c.contents->data()); u64(o, c.contents->size());
+            break;
         case CreateConstant: put(o, &c.constant, 4); str(o, c.res); dims(o, c.dim); break;
         case ElwMultiply: case ElwAdd: case DotProduct: str(o, c.a); str(o, c.b); str(o, c.res); break;
         case ElwMultiplyEq: case ElwAddEq: str(o, c.a); str(o, c.b); break;
@@ -112,12 +126,12 @@ inline void proc(std::vector<uint8_t>& o, const IRProcedure& p) {
         case Index: str(o, c.a); u64(o, c.index); u64(o, c.dim_index); str(o, c.res); break;
         case Concat: str(o, c.a); str(o, c.b); u64(o, c.dim_index); str(o, c.res); break;
         case Broadcast: str(o, c.a); u64(o, c.dim_index); u64(o, c.r); str(o, c.res); break;
-        case While: str(o, c.a); proc(o, *c.block); break;
+        case While: str(o, c.a); proc(o, *c.block, payload_offsets); break;
         case If:
             u32(o, (uint32_t)c.conditions.size());
-            for (auto& arm : c.conditions) { str(o, arm.first); proc(o, *arm.second); }
+            for (auto& arm : c.conditions) { str(o, arm.first); proc(o, *arm.second, payload_offsets); }
             o.push_back(c.else_proc ? 1 : 0);
-            if (c.else_proc) proc(o, *c.else_proc);
+            if (c.else_proc) proc(o, *c.else_proc, payload_offsets);
             break;
         case EX: break;
         case Heading: str(o, c.cmt); break;
@@ -128,11 +142,12 @@ inline void proc(std::vector<uint8_t>& o, const IRProcedure& p) {
 }  // namespace detail
 
 // Flat little-endian stream understood by adhip_execute.  CreateMat payloads are referenced by pointer: the
-// procedure must stay alive (and unmodified) until the call returns.
-inline std::vector<uint8_t> serialize(const IRProcedure& p) {
+// procedure must stay alive (and unmodified) until the call returns.  `payload_offsets`, when given, receives the byte
+// offset of every such pointer field (the only bytes of the stream that differ from run to run).
+inline std::vector<uint8_t> serialize(const IRProcedure& p, std::vector<size_t>* payload_offsets = nullptr) {
     std::vector<uint8_t> o{'A', 'D', 'I', 'R'};
     detail::u32(o, 1);
-    detail::proc(o, p);
+    detail::proc(o, p, payload_offsets);
     return o;
 }
 

@@ -27,6 +27,8 @@ Pinned by (tests/test_oracle_kats.py, tests/test_oracle_math.py):
   * closed forms: tree-sum and sequential-k dot against float64 sums, bit-exact integer cases,
     permute/view/index/concat against brute-force index arithmetic written independently of numpy's
     reshape/transpose.
+  * `Max` (an extension: declared, never implemented by the reference): brute-force loops over small matrices
+    including NaN, infinities and signed zeros.
 Parity unpinned: the exact last-ulp behaviour of exp2/log2/sin of whichever OpenCL runtime the
 reference ran on (libm's float functions are used here), and random initial weights (`randn`
 draws from an unseeded generator in the reference).
@@ -110,6 +112,16 @@ def ref_reduce_sum(a: np.ndarray) -> np.ndarray:
     isz = 4
     c_kernels().ref_reduce_sum(_ptr(a), a.strides[0] // isz, a.strides[1] // isz, _ptr(out), vec, red)
     return out
+
+
+def ref_reduce_max(a: np.ndarray) -> np.ndarray:
+    """[vec,red] -> [vec], the largest element of every row.  The reference only declares this reduction
+    (`ReduceOp::Max`, src/kernel/kernel_decl.rs:75-78; "add max, min", src/core/ir.rs:49) and has no kernel for it,
+    so there is no algorithm of its to restate: the result is order-independent (maximum is associative and
+    commutative and rounds nothing) and is taken with C's `fmax` rule, which OpenCL C's `fmax`/`max` share: a NaN
+    operand is ignored unless both are NaN.  Pinned by brute force in tests/test_oracle_math.py."""
+    a = np.asarray(a, dtype=np.float32)
+    return np.fmax.reduce(a, axis=1).astype(np.float32)
 
 
 _UNARY_OPS = {IR.T_EXP2: 0, IR.T_LOG2: 1, IR.T_SIN: 2, IR.T_RECIP: 4, IR.T_SQRT: 5,
@@ -275,6 +287,10 @@ class OracleDevice(Device):
             assert a.ndim == 2, "Sum needs a 2-D operand"
             self.max_terms = max(self.max_terms, int(a.shape[-1]))
             self._store(cmd.res, list(a.shape[:-1]), ref_reduce_sum(a))
+        elif t == IR.T_MAX:
+            a = self._value(cmd.a)
+            assert a.ndim == 2 and a.shape[1] > 0, "Max needs a 2-D operand with a non-empty last dim"
+            self._store(cmd.res, list(a.shape[:-1]), ref_reduce_max(a))
         elif t == IR.T_DOT_PRODUCT:
             a, b = self._value(cmd.a), self._value(cmd.b)
             assert a.ndim == 2 and b.ndim == 2 and a.shape[1] == b.shape[0]

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from adhip import ir as IR
-from oracle.interp import OracleDevice, ref_dot, ref_reduce_sum, ref_unary
+from oracle.interp import OracleDevice, ref_dot, ref_reduce_max, ref_reduce_sum, ref_unary
 
 
 # ---- reductions and matmul ----------------------------------------------------------------
@@ -29,6 +29,84 @@ def test_tree_sum_matches_float64_and_is_exact_on_integers(vec, red):
 def test_tree_sum_reads_strided_input():
     a = np.arange(24, dtype=np.float32).reshape(4, 6)
     assert np.array_equal(ref_reduce_sum(a.T), a.sum(0))
+
+
+def test_row_max_by_brute_force():
+    """`Max` against plain loops with explicit comparisons (no numpy reduction): the largest element of every row;
+    a NaN is passed over unless the whole row is NaN; -0.0 and +0.0 compare equal (either may come back); rows of
+    -inf stay -inf; position of the maximum does not matter."""
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((9, 37)).astype(np.float32)
+    a[1, 5] = np.nan
+    a[2, :] = np.nan
+    a[3, :] = -np.inf
+    a[4, 7] = np.inf
+    a[5, :] = -0.0
+    a[5, 3] = 0.0
+    a[6, 0] = 1e30            # first position
+    a[7, 36] = 1e30           # last position
+    got = ref_reduce_max(a)
+    for i in range(a.shape[0]):
+        best = None
+        for j in range(a.shape[1]):
+            v = float(a[i, j])
+            if v != v:
+                continue
+            if best is None or v > best:
+                best = v
+        if best is None:
+            assert got[i] != got[i], f"row {i}: all NaN must give NaN"
+        else:
+            assert float(got[i]) == best, (i, got[i], best)
+    assert np.array_equal(ref_reduce_max(a[:1, :1]), a[:1, 0])
+    # strided input (a transposed view)
+    b = np.arange(24, dtype=np.float32).reshape(4, 6)
+    assert np.array_equal(ref_reduce_max(b.T), b.max(0))
+
+
+def test_max_command_and_softmax_through_the_oracle():
+    """`Tensor.max(dim)` on every dim of a 3-D tensor against loops, its backward (equal shares among ties), and the
+    shifted softmax against float64 at arguments where exp alone overflows."""
+    from adhip import autodiff
+    dev = OracleDevice()
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(9)
+    xn = rng.integers(-3, 4, size=(3, 4, 5)).astype(np.float32)
+    x = autodiff.tensor(xn, [3, 4, 5])
+    outs = []
+    for d in range(3):
+        m = x.max(d)
+        m.forward()
+        m.val().keep()
+        outs.append(m)
+    total = outs[2].sum(0).sum(0)
+    total.forward()
+    total.backward()
+    x.grad().keep()
+    s = (x * 40.0).softmax(-1)
+    s.forward()
+    s.val().keep()
+    autodiff.execute()
+    for d in range(3):
+        got = outs[d].val().get().numpy()
+        exp = np.empty([n for i, n in enumerate(xn.shape) if i != d], dtype=np.float32)
+        for idx in itertools.product(*[range(n) for n in exp.shape]):
+            full = list(idx)
+            full.insert(d, slice(None))
+            exp[idx] = max(float(v) for v in xn[tuple(full)])
+        assert np.array_equal(got, exp), d
+    g = x.grad().get().numpy()
+    for i in range(3):
+        for j in range(4):
+            row = xn[i, j]
+            ties = [k for k in range(5) if row[k] == row.max()]
+            for k in range(5):
+                assert abs(g[i, j, k] - (1.0 / len(ties) if k in ties else 0.0)) < 1e-6
+    z = xn.astype(np.float64) * 40.0
+    e = np.exp(z - z.max(-1, keepdims=True))
+    ref = e / e.sum(-1, keepdims=True)
+    got = s.val().get().numpy()
+    assert np.isfinite(got).all() and np.abs(got - ref).max() < 2e-6
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 1, 1), (2, 5, 3), (17, 33, 9), (64, 128, 32)])

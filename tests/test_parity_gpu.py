@@ -623,3 +623,74 @@ def test_if_with_more_arms_than_one_predicate_batch(hip_device):
     cmds.append(IR.If(conditions=arms, else_proc=IR.IRProcedure("else", [IR.CreateConstant(-1.0, "k", [4]), IR.ElwAddEq(s="x", o="k")])))
     got = _run_ir(hip_device, cmds, ["x"])
     assert_exact(got["x"].data, np.full(4, 66.0, dtype=np.float32), "x")
+
+
+@pytest.mark.parametrize("V,R", [(7, 5), (64, 256), (300, 1000), (33, 4096), (4, 70000), (2048, 64), (3, 1)])
+def test_max_rows_and_columns(V, R, hip_device):
+    """The Max reduction over rows (contiguous) and over columns (strided operand) of the same matrix, with NaN,
+    infinities and ties placed in it: bit-exact against the oracle and against numpy's fmax."""
+    print(f"[case] max {V}x{R}", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(V * 31 + R)
+    x = rng.standard_normal((V, R)).astype(np.float32)
+    x[0, R // 2] = np.inf
+    if R > 1:
+        x[V - 1, 0] = np.nan
+        x[V // 2, :] = -np.inf
+    cmds = [IR.CreateMat(x.reshape(-1), [V, R], "x"), IR.Max(a="x", res="rows"),
+            IR.Permute(a="x", p=[1, 0], res="xt"), IR.Max(a="xt", res="cols")]
+    got = _run_ir(hip_device, cmds, ["rows", "cols"])
+    ref_dev = OracleDevice()
+    ref_dev.execute(IR.IRProcedure("main", cmds + [IR.EX()]), {"rows", "cols"})
+    assert got["rows"].dim == [V] and got["cols"].dim == [R]
+    for k in ("rows", "cols"):
+        assert_exact(got[k].data, ref_dev.get_tensor(k).data, k + " vs oracle")
+    assert_exact(got["rows"].data, np.fmax.reduce(x, axis=1), "rows vs numpy")
+    assert_exact(got["cols"].data, np.fmax.reduce(x, axis=0), "cols vs numpy")
+
+
+@pytest.mark.parametrize("shape,dim", [((6, 10), 1), ((6, 10), 0), ((3, 5, 7), 1), ((40, 300), -1)])
+def test_max_forward_backward_and_stable_softmax(shape, dim, hip_device):
+    """Tensor.max(dim) forward and backward and the shifted softmax, device against oracle, and the softmax against
+    float64 at arguments up to +-100 (exp alone overflows at 88)."""
+    print(f"[case] max/softmax {shape} dim {dim}", flush=True)
+    from adhip import autodiff
+    rng = np.random.default_rng(sum(shape) + dim)
+    xn = (rng.standard_normal(shape) * 30).astype(np.float32)
+    xn.reshape(-1)[0] = 100.0
+    xn.reshape(-1)[1] = -100.0
+    wn = rng.standard_normal(shape).astype(np.float32)
+
+    def build(dev):
+        autodiff.set_device(dev)
+        x = autodiff.tensor(xn, list(shape))
+        w = autodiff.tensor(wn, list(shape))
+        m = x.max(dim)
+        s = x.softmax(dim)
+        L = (s * w)
+        for _ in shape:
+            L = L.sum(0)
+        t = m
+        for _ in m.dim():
+            t = t.sum(0)
+        total = L + t
+        total.forward()
+        total.backward()
+        for v in (m.val(), s.val(), x.grad()):
+            v.keep()
+        autodiff.execute()
+        return {"m": m.val().get(), "s": s.val().get(), "dx": x.grad().get()}
+
+    got, ref = build(hip_device), build(OracleDevice())
+    assert_exact(got["m"].data, ref["m"].data, "max")
+    n = shape[dim]
+    compare_outputs(got, ref, {"m": ("exact",)}, ("close", RED_RTOL * math.sqrt(n)))
+    z = xn.astype(np.float64)
+    e = np.exp(z - z.max(dim, keepdims=True))
+    s64 = e / e.sum(dim, keepdims=True)
+    assert np.isfinite(got["s"].data).all()
+    assert_close(got["s"].data, s64.reshape(-1), RED_RTOL * math.sqrt(n), "softmax vs float64")
+    # d/dx of sum(softmax * w) + sum(max): softmax part s * (w - sum(s * w)) along dim, max part one-hot (no ties here)
+    sw = (s64 * wn).sum(dim, keepdims=True)
+    dmax = (z == z.max(dim, keepdims=True)).astype(np.float64)
+    assert_close(got["dx"].data, (s64 * (wn - sw) + dmax).reshape(-1), 4 * RED_RTOL * math.sqrt(n), "dx vs float64")

@@ -1,7 +1,7 @@
 """A float64 restatement of `workloads.encoder_layer` in torch (CPU autograd), used to check the oracle and the
-device on a whole encoder layer.  It restates the reference's compositions literally, including its softmax
-(exp(x) / exp(x).sum(-1) with the sum broadcast back along the trailing dim, no maximum subtracted) and its LayerNorm
-(biased variance, eps 1e-9, scale trainable, bias fixed at zero)."""
+device on a whole encoder layer.  It restates the reference's compositions: attention with a softmax over the last
+dim (the evident intent of reference src/nn/activations/softmax.rs:28-30, whose own broadcast divides by the wrong
+row's sum) and its LayerNorm (biased variance, eps 1e-9, scale trainable, bias fixed at zero)."""
 import math
 
 import torch
@@ -13,8 +13,7 @@ def encoder_layer_reference(inputs, heads):
     seq, d_model = x.shape
 
     def softmax_ref(s):
-        e = torch.exp(s)
-        return e / e.sum(-1)          # [S,S] / [S]: trailing-dim broadcast, as the reference's try_broadcast does
+        return torch.softmax(s, -1)
 
     def layer_norm(v, scale):
         mean = v.mean(-1, keepdim=True)
