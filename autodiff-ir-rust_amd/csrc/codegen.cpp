@@ -1,6 +1,7 @@
 #include "codegen.hpp"
 
 #include <algorithm>
+#include <cctype>
 #include <climits>
 #include <cstdlib>
 #include <cstring>
@@ -91,6 +92,7 @@ struct Atom {
     std::string name;
     int64_t range = 1;  // value in [0, range) whenever the access it feeds is selected
     bool lane = false;  // differs between the lanes of one thread's vector
+    std::string code;   // derived atoms: the expression (over earlier atoms) that defines them
 };
 
 struct Aff {
@@ -140,6 +142,7 @@ struct LoadRec {
     const Node* node;
     Aff idx;
     bool predicated;
+    std::string key;
 };
 
 struct Gen {
@@ -157,6 +160,16 @@ struct Gen {
     std::map<const Node*, std::string> preset;  // nodes whose value is a variable the kernel already holds
     std::vector<LoadRec> loads;
     std::vector<Aff> recorded;  // every index expression over base atoms, for dim merging
+    // Tiled element-wise kernels: loads whose key is in `stage_keys` are not issued by the thread that needs the value;
+    // the block reads the 64x64 tile they come from through LDS (see gen_elw_tiled_kernel).  `index_code` collects, in
+    // order, every statement that defines an index atom or a predicate (no loads, no arithmetic on values), so that
+    // the staging phase can evaluate the same index at other coordinates.
+    std::set<std::string> stage_keys;
+    struct Staged { std::string key, param, index, pred; int slot; };
+    std::vector<Staged> staged;
+    std::vector<std::string> index_code;
+    std::string tile_row_origin, tile_col_origin;  // expressions of the tile's first row / first column
+    int row_atom = -1;
     int tmp = 0;
     double flops = 0;  // per lane element
 
@@ -178,6 +191,24 @@ struct Gen {
         for (auto& x : a.t)
             if (x.second < 0) m += x.second * (atoms[x.first].range - 1);
         return m;
+    }
+    // whether atom `a` is atom `base` or is computed from it
+    bool atom_depends_on(int a, int base) const {
+        if (a == base) return true;
+        const std::string& code = atoms[(size_t)a].code;
+        if (code.empty()) return false;
+        auto mentions = [&](const std::string& name) {
+            for (size_t pos = code.find(name); pos != std::string::npos; pos = code.find(name, pos + 1)) {
+                const bool left = pos == 0 || !(isalnum((unsigned char)code[pos - 1]) || code[pos - 1] == '_');
+                const size_t end = pos + name.size();
+                const bool right = end >= code.size() || !(isalnum((unsigned char)code[end]) || code[end] == '_');
+                if (left && right) return true;
+            }
+            return false;
+        };
+        for (int b = 0; b < a; ++b)
+            if (mentions(atoms[(size_t)b].name) && atom_depends_on(b, base)) return true;
+        return false;
     }
     bool aff_lane(const Aff& a) const {
         for (auto& x : a.t)
@@ -208,7 +239,9 @@ struct Gen {
         if (it != atom_memo.end()) return it->second;
         std::string name = "a" + std::to_string(tmp++);
         emit(lane, strf("const %s %s = %s;", idx_t(), name.c_str(), code.c_str()));
+        index_code.push_back(strf("const %s %s = %s;", idx_t(), name.c_str(), code.c_str()));
         int id = add_atom(name, range, lane);
+        atoms[(size_t)id].code = code;
         atom_memo[code] = id;
         return id;
     }
@@ -345,12 +378,24 @@ struct Gen {
         ADHIP_CHECK(aff_min(idx) >= 0 && aff_max(idx) < ne,
                     "internal: generated load of node %d (%s) spans [%lld,%lld] outside its %lld elements", n->id,
                     n->name.c_str(), (long long)aff_min(idx), (long long)aff_max(idx), (long long)ne);
-        loads.push_back({n, idx, !pred.empty()});
+        loads.push_back({n, idx, !pred.empty(), key});
         const std::string& bp = bufs[buffer_of(n)].param;
         std::string name = "l" + std::to_string(tmp++);
         Val v;
         const bool ilane = aff_lane(idx);
         const bool nt = ne >= nontemporal_min_elems();
+        if (stage_keys.count(key)) {
+            // the value was put into LDS by the staging phase: tile[column within the tile][row within the tile]
+            ADHIP_CHECK(lane_atom >= 0 && row_atom >= 0 && vec == 4, "internal: staged load outside a tiled kernel");
+            const int slot = (int)staged.size();
+            staged.push_back({key, bp, aff_str(idx), pred, slot});
+            const std::string& last = atoms[(size_t)lane_atom - 1].name;  // the atom of the innermost dim (float4 index)
+            emit(true, strf("const float %s = tile%d[(4u * %s + %s) - %s][%s - %s];", name.c_str(), slot, last.c_str(),
+                            atoms[lane_atom].name.c_str(), tile_col_origin.c_str(), atoms[row_atom].name.c_str(), tile_row_origin.c_str()));
+            v = {name, true};
+            val_memo[key] = v;
+            return v;
+        }
         if (!ilane && !plane) {
             if (pred.empty()) emit(false, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
             else emit(false, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
@@ -381,6 +426,7 @@ struct Gen {
         std::string name = "p" + std::to_string(tmp++);
         bool lane = cond_lane || (!pred.empty() && pred_lane[pred]);
         emit(lane, strf("const bool %s = %s%s;", name.c_str(), pred.empty() ? "" : (pred + " && ").c_str(), cond.c_str()));
+        index_code.push_back(strf("const bool %s = %s%s;", name.c_str(), pred.empty() ? "" : (pred + " && ").c_str(), cond.c_str()));
         pred_lane[name] = lane;
         val_memo[key] = {name, lane};
         return name;
@@ -579,13 +625,14 @@ struct ElwBody {
 };
 
 ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members, const Shape& iter_shape, int vec,
-                 bool wide) {
+                 bool wide, const std::function<void(Gen&)>& setup = nullptr) {
     ElwBody b;
     b.iter_shape = iter_shape;
     Gen& g = b.g;
     g.vec = vec;
     g.wide = wide;
     g.members = members;
+    if (setup) setup(g);
     const size_t nd = iter_shape.size();
     Shape rs = row_major_strides(iter_shape);
     Aff lin;
@@ -703,6 +750,114 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     return k;
 }
 
+// Element-wise kernel over 64x64 tiles of the two innermost iteration dims, for passes that read a large operand
+// against the grain: consecutive *rows* of the result are adjacent in the operand's memory, consecutive columns are
+// far apart (a permuted operand of a gather or an addition).  Read directly, every lane of a wavefront would touch its
+// own cache line.  Here the block first fetches the operand's tile with the rows as the fast index (256-byte runs per
+// wavefront), parks it in LDS, and every thread then takes its four values from there; everything else in the kernel,
+// including the 128-bit accesses of all other operands and of the results, is the ordinary generated body.  The
+// staging phase evaluates the very index expression the body would have used, at the coordinates of the element it
+// fetches, so whatever view or concat piece the operand sits behind is handled by construction.
+// Returns false (and leaves `k` alone) when the pass has no such operand or not the shape for it.
+static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members, const Shape& shape, bool wide,
+                                 GeneratedKernel& k) {
+    const size_t nd = shape.size();
+    if (nd < 2) return false;
+    const int64_t I = shape[nd - 1], Rws = shape[nd - 2];
+    if (I % 4 != 0 || I < 32 || Rws < 32) return false;   // tiles are 64x64: smaller extents leave most of a block idle
+    const int64_t N = numel(spec.outputs[0]->shape);
+    std::set<std::string> keys;
+    {
+        ElwBody probe = elw_body(spec, members, shape, 4, wide);
+        const int row_atom = probe.dim_atoms[nd - 2];
+        for (const LoadRec& l : probe.g.loads) {
+            if (numel(l.node->shape) < (int64_t(1) << 18)) continue;
+            // unit stride along the rows (directly, or through a quotient / remainder of the row index), none along
+            // the thread's own four columns
+            bool unit_rows = false;
+            for (auto& x : l.idx.t)
+                if (x.second == 1 && !probe.g.atoms[(size_t)x.first].lane && probe.g.atom_depends_on(x.first, row_atom)) unit_rows = true;
+            if (!unit_rows || !probe.g.aff_lane(l.idx) || probe.g.vectorizable(l.idx)) continue;
+            keys.insert(l.key);
+        }
+    }
+    if (keys.empty() || keys.size() > 2) return false;
+    const std::string sfx = wide ? "ull" : "u";
+    ElwBody b = elw_body(spec, members, shape, 4, wide, [&](Gen& g) {
+        g.stage_keys = keys;
+        g.row_atom = (int)nd - 2;
+        g.tile_row_origin = "row0";
+        g.tile_col_origin = "col0";
+    });
+    Gen& g = b.g;
+    if (g.staged.empty()) return false;
+    const char* it = g.idx_t();
+    k = GeneratedKernel();
+    k.kind = "elw_tiled";
+    k.entry = spec.name;
+    std::string sig = "const int* __restrict__ guard";
+    std::vector<Node*> order;
+    for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* o%zu", i); order.push_back(spec.outputs[i]); }
+    for (auto& gb : g.bufs) { sig += ", const float* " + gb.param; order.push_back(gb.node); }
+    const int64_t TI = (I + 63) / 64, TJ = (Rws + 63) / 64;
+    int64_t outer = 1;
+    for (size_t d = 0; d + 2 < nd; ++d) outer *= shape[d];
+    const int64_t blocks = TI * TJ * outer;
+    if (blocks > 0x7fffffff) return false;
+    const std::string rowv = "c" + std::to_string(nd - 2), colv = "c" + std::to_string(nd - 1);
+    std::string src = kernel_prelude();
+    src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+    src += "    if (guard && *guard == 0) return;\n";
+    for (auto& st : g.staged) src += strf("    __shared__ float tile%d[64][65];\n", st.slot);
+    src += "    const unsigned tid = threadIdx.x;\n";
+    src += strf("    %s bid = blockIdx.x;\n", it);
+    src += strf("    const %s col0 = (bid %% %lld%s) * 64u;\n    bid /= %lld%s;\n", it, (long long)TI, sfx.c_str(), (long long)TI, sfx.c_str());
+    src += strf("    const %s row0 = (bid %% %lld%s) * 64u;\n    bid /= %lld%s;\n", it, (long long)TJ, sfx.c_str(), (long long)TJ, sfx.c_str());
+    for (size_t d = nd - 2; d-- > 0;) {
+        if (d == 0) src += strf("    const %s c0 = bid;\n", it);
+        else src += strf("    const %s c%zu = bid %% %lld%s;\n    bid /= %lld%s;\n", it, d, (long long)shape[d], sfx.c_str(), (long long)shape[d], sfx.c_str());
+    }
+    // staging: lane = row within the tile, so that a wavefront reads one 256-byte run of the operand per column
+    src += "#pragma unroll 2\n    for (unsigned k = 0; k < 16u; ++k) {\n";
+    src += "        const unsigned lj = tid & 63u, li = (tid >> 6) + 4u * k;\n";
+    src += strf("        const %s %s = row0 + lj;\n        const %s ii = col0 + li;\n", it, rowv.c_str(), it);
+    src += strf("        const %s %s = ii >> 2;\n        const %s j = ii & 3u;\n", it, colv.c_str(), it);
+    src += strf("        const bool inside = %s < %lld%s && ii < %lld%s;\n", rowv.c_str(), (long long)Rws, sfx.c_str(), (long long)I, sfx.c_str());
+    src += join(g.index_code, "        ");
+    for (auto& st : g.staged) {
+        src += strf("        { float v = 0.0f; if (inside%s%s) v = %s[%s]; tile%d[li][lj] = v; }\n", st.pred.empty() ? "" : " && ",
+                    st.pred.c_str(), st.param.c_str(), st.index.c_str(), st.slot);
+    }
+    src += "    }\n    __syncthreads();\n";
+    // compute: a thread owns four adjacent columns of four rows of the tile
+    src += "    const unsigned lc = tid & 15u, lr = tid >> 4;\n";
+    src += "#pragma unroll 1\n    for (unsigned k = 0; k < 4u; ++k) {\n";
+    src += strf("        const %s %s = row0 + lr + 16u * k;\n        const %s %s = (col0 >> 2) + lc;\n", it, rowv.c_str(), it, colv.c_str());
+    src += strf("        if (%s >= %lld%s || %s >= %lld%s) continue;\n", rowv.c_str(), (long long)Rws, sfx.c_str(), colv.c_str(), (long long)(I / 4), sfx.c_str());
+    src += join(g.codeA, "        ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("        float w%zu[4];\n", i);
+    src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+    src += join(g.codeB, "            ");
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
+    src += "        }\n";
+    // linear float4 index of the thread's element: row-major over the iteration shape
+    std::string lin = "c0";
+    for (size_t d = 1; d < nd; ++d)
+        lin = strf("(%s * %lld%s + c%zu)", lin.c_str(), (long long)(d + 1 == nd ? I / 4 : shape[d]), sfx.c_str(), d);
+    src += strf("        const %s t4 = %s;\n", it, lin.c_str());
+    for (size_t i = 0; i < spec.outputs.size(); ++i)
+        src += "        " + store4_stmt(strf("w%zu", i), strf("o%zu + t4 * 4u", i), N >= nontemporal_min_elems()) + "\n";
+    src += "    }\n}\n";
+    k.source = src;
+    k.buffer_args = order;
+    k.block[0] = 256;
+    k.grid[0] = (unsigned)blocks;
+    k.bytes = 4.0 * (double)N * (double)spec.outputs.size();
+    for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), N);
+    k.flops = g.flops * (double)N;
+    return true;
+}
+
 GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members) {
     if (!spec.colsums.empty()) return gen_elw_colsum_kernel(spec, members);
     ADHIP_CHECK(!spec.outputs.empty(), "internal: element-wise kernel without outputs");
@@ -719,6 +874,10 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
         shape = merge_dims(shape, dry.g.recorded, dry.dim_atoms);
     }
     int vec = (shape.back() % 4 == 0 && N >= 1024) ? 4 : 1;
+    if (vec == 4) {
+        GeneratedKernel tiled;
+        if (gen_elw_tiled_kernel(spec, members, shape, wide, tiled)) return tiled;
+    }
     ElwBody b = elw_body(spec, members, shape, vec, wide);
     Gen& g = b.g;
 

@@ -1304,6 +1304,62 @@ struct Lowerer {
                 group_of[E] = (int)gs;
             }
         }
+        // ---- 5c'. a dense transposed copy that a single element-wise kernel reads is not made at all when that kernel
+        // can fetch the operand's tiles through LDS itself (gen_elw_kernel then answers with its tiled form): the
+        // copy's round trip through memory -- twice the operand's size -- goes away
+        if (opt.fuse) {
+            for (size_t tg = 0; tg < groups.size(); ++tg) {
+                Group& TG = groups[tg];
+                if (TG.dead || TG.kind != Group::TRANSPOSE) continue;
+                Node* T = TG.members[0];
+                if (wanted_nodes.count(T) || T->force_root) continue;  // has to be in memory for its own sake
+                int consumer = -1;
+                bool fusable = true;
+                for (size_t g = 0; g < groups.size() && fusable; ++g) {
+                    if (groups[g].dead || g == tg) continue;
+                    bool rd = false;
+                    for (Node* m : groups[g].members) rd = rd || reads[m].count(T);
+                    for (Node* sd : groups[g].side) rd = rd || reads[sd].count(T);
+                    for (auto& cs : groups[g].colsums) {
+                        std::map<Node*, bool> er;
+                        if (in_mem(cs.first)) er[cs.first] = true;
+                        else collect_reads(cs.first, er);
+                        if (er.count(T)) fusable = false;
+                    }
+                    if (!rd) continue;
+                    if (consumer >= 0 || groups[g].kind != Group::ELW || !groups[g].colsums.empty() || !groups[g].side.empty() || g < tg) fusable = false;
+                    consumer = (int)g;
+                }
+                if (!fusable || consumer < 0) continue;
+                Group& G = groups[consumer];
+                T->root = false;
+                std::map<Node*, std::map<Node*, bool>> saved_reads;
+                std::map<Node*, std::set<Node*>> saved_folded;
+                for (Node* m : G.members) {
+                    saved_reads[m] = reads[m];
+                    saved_folded[m] = folded_in[m];
+                    reads[m].clear();
+                    folded_in[m].clear();
+                    collect_reads(m, reads[m], &folded_in[m]);
+                }
+                ElwKernelSpec probe_spec;
+                probe_spec.outputs = G.members;
+                probe_spec.name = "probe";
+                bool tiled = false;
+                try {
+                    tiled = gen_elw_kernel(probe_spec, std::set<const Node*>(G.members.begin(), G.members.end())).kind == "elw_tiled";
+                } catch (const Error&) {
+                    tiled = false;
+                }
+                if (tiled) {
+                    TG.dead = true;
+                    group_of.erase(T);  // T is no kernel's product any more: its consumer computes it in place
+                } else {
+                    T->root = true;
+                    for (Node* m : G.members) { reads[m] = saved_reads[m]; folded_in[m] = saved_folded[m]; }
+                }
+            }
+        }
         std::map<Node*, std::string> home_of_early;
         for (auto& w : wanted) home_of_early[w.second] = w.first;
         auto reads_node = [&](const Group& H, Node* what) {
