@@ -310,6 +310,38 @@ def encoder_layer(dev, seq: int = 64, d_model: int = 32, heads: int = 4, ff_dim:
     return Workload("encoder_layer", outs, inputs, flops=fl * (3.0 if backward else 1.0))
 
 
+def attention_forward(dev, seq: int = 64, d_model: int = 64, heads: int = 4, seed: int = 0, scale_x: float = 1.0) -> Workload:
+    """y = MultiHeadAttention(d_model, heads)(x), forward only (inference): per-head projections, attention, the
+    heads concatenated, the output projection (reference src/nn/transformer.rs:34-99).  Weights N(0, 1/fan_in), passed
+    in explicitly."""
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    inputs: Dict[str, np.ndarray] = {}
+    mha = nn.MultiHeadAttention(d_model, heads)
+    d_v = d_model // heads
+
+    def mat(name, fan_in, fan_out):
+        w = (rng.standard_normal((fan_in, fan_out)) / np.sqrt(fan_in)).astype(np.float32)
+        inputs[name] = w
+        return autodiff.tensor(w, [fan_in, fan_out])
+
+    for h in range(heads):
+        mha.wq[h].w = mat(f"wq{h}", d_model, d_v)
+        mha.wk[h].w = mat(f"wk{h}", d_model, d_v)
+        mha.wv[h].w = mat(f"wv{h}", d_model, d_v)
+    mha.wo.w = mat("wo", d_model, d_model)
+    xn = (scale_x * rng.standard_normal((seq, d_model))).astype(np.float32)
+    inputs["x"] = xn
+    x = autodiff.tensor(xn, [seq, d_model])
+    y = mha.f(x)
+    y.forward()
+    y.val().keep()
+    fl = heads * 3 * 2.0 * seq * d_model * d_v + heads * 2 * 2.0 * seq * seq * d_v + 2.0 * seq * d_model * d_model
+    wl = Workload("attention_forward", {"y": y.val()}, inputs, flops=fl)
+    wl.attention_flops = heads * 2 * 2.0 * seq * seq * d_v
+    return wl
+
+
 def encoder_train(dev, seq: int = 64, d_model: int = 32, heads: int = 4, ff_dim: int = 64, iters: int = 3,
                   lr: float = 0.05, seed: int = 0) -> Workload:
     """`iters` SGD steps on one TransformerEncoderLayer inside an IR for-loop: y = layer(x); loss = mean((y - t)^2);

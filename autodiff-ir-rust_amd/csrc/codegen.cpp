@@ -28,6 +28,7 @@ const char* op_name(Op o) {
     case Op::SUM: return "sum";
     case Op::MAX: return "max";
     case Op::DOT: return "dot";
+    case Op::ATTN: return "attention";
     }
     return "?";
 }

@@ -25,6 +25,10 @@ enum class Op : uint8_t {
     SUM,  // [V,R] -> [V]
     MAX,  // [V,R] -> [V], the largest element of every row (NaN only where a whole row is NaN)
     DOT,  // [M,K] x [K,N] -> [M,N]
+    // softmax over the rows of (cval * Q K^T), times V: operands Q [Sq,D], K^T [D,Sk] (a transposed view of K), V [Sk,DV].
+    // Never built from a command: the lowering puts it in the place of a DOT whose first operand it recognises as
+    // that softmax (the attention of reference src/nn/transformer.rs:10-18).
+    ATTN,
 };
 
 inline bool op_is_leaf(Op o) { return o == Op::LIVEIN || o == Op::UPLOAD; }

@@ -9,6 +9,7 @@
 #include <map>
 #include <unordered_map>
 
+#include "attention.hpp"
 #include "codegen.hpp"
 #include "gemm.hpp"
 #include "graph.hpp"
@@ -242,7 +243,7 @@ using RegionKey = std::pair<const Proc*, size_t>;
 struct Group {
     std::vector<Node*> members;
     int64_t n = 0;
-    enum Kind { ELW, SUM, DOT, TRANSPOSE } kind = ELW;
+    enum Kind { ELW, SUM, DOT, TRANSPOSE, ATTN } kind = ELW;
     // column sums computed by this element-wise kernel: (value node, SUM node that wanted it)
     std::vector<std::pair<Node*, Node*>> colsums;
     int64_t cs_rows = 0, cs_cols = 0;
@@ -984,6 +985,142 @@ struct Lowerer {
         push_launch(out, l, "copy");
     }
 
+    // -----------------------------------------------------------------------------------
+    // attention: dot(softmax(scale * dot(Q, K^T)), V) as one kernel
+    //
+    // The caller writes attention with ordinary commands (reference src/nn/transformer.rs:10-18): a product, a scaling, a
+    // row maximum, exp2((x - max) * log2 e), a row sum, a reciprocal, a multiplication, a product.  When a product's
+    // first operand is exactly that chain, and nothing else looks at the chain's intermediate values, the product node
+    // is turned into an ATTN node over (Q, K^T, V): the fused kernel computes the same arithmetic without the [Sq, Sk]
+    // matrices ever reaching memory.  Anything that does not match to the letter stays what it was.
+    // -----------------------------------------------------------------------------------
+    static Node* whole_value(const TRef& t) {
+        if (!t.single_full() || t.pieces[0].src.kind != Src::NODE || !identity_piece(t.pieces[0], t)) return nullptr;
+        Node* n = t.pieces[0].src.node;
+        return numel(n->shape) == numel(t.shape) ? n : nullptr;
+    }
+    // `t` of shape [V,R] is a [V] vector repeated along the columns
+    static Node* column_broadcast(const TRef& t, int64_t V, int64_t R) {
+        if (!t.single_full() || t.shape != Shape{V, R} || t.pieces[0].src.kind != Src::NODE) return nullptr;
+        const View& v = t.pieces[0].view;
+        if (v.st.empty()) return nullptr;
+        for (size_t i = 0; i + 1 < v.st.size(); ++i)
+            if (!stage_is_identity(v.st[i])) return nullptr;
+        const Stage& s = v.st.back();
+        if (s.shape != Shape{V, R} || s.stride != Shape{1, 0} || s.offset != 0) return nullptr;
+        Node* n = t.pieces[0].src.node;
+        return numel(n->shape) == V ? n : nullptr;
+    }
+    static bool constant_operand(const TRef& t, float& c) {
+        if (t.pieces.size() != 1 || t.pieces[0].src.kind != Src::CONST) return false;
+        c = t.pieces[0].src.c;
+        return true;
+    }
+    // n = MUL(x, constant) in either order
+    static Node* times_constant(Node* n, float& c) {
+        if (n->op != Op::MUL || n->in.size() != 2) return nullptr;
+        for (int k = 0; k < 2; ++k)
+            if (constant_operand(n->in[(size_t)(1 - k)], c)) return whole_value(n->in[(size_t)k]);
+        return nullptr;
+    }
+
+    struct AttentionKey {
+        int64_t sq = 0, sk = 0, d = 0, dv = 0, q_ld = 0, k_ld = 0, v_ld = 0;
+        float scale = 0.f;
+        bool operator==(const AttentionKey& o) const {
+            return sq == o.sq && sk == o.sk && d == o.d && dv == o.dv && q_ld == o.q_ld && k_ld == o.k_ld && v_ld == o.v_ld && scale == o.scale;
+        }
+    };
+    // shape and strides of an ATTN node's operands, if they are what the kernel reads: unit stride inside a row of Q,
+    // K and V, rows of K and V 16-byte aligned
+    static bool attention_key(const Node* n, AttentionKey& k, Affine2D& q, Affine2D& kt, Affine2D& v) {
+        if (n->in.size() != 3 || !tref_affine2d(n->in[0], q) || !tref_affine2d(n->in[1], kt) || !tref_affine2d(n->in[2], v)) return false;
+        k.sq = n->in[0].shape[0];
+        k.d = n->in[0].shape[1];
+        k.sk = n->in[1].shape[1];
+        k.dv = n->in[2].shape[1];
+        if (n->in[1].shape[0] != k.d || n->in[2].shape[0] != k.sk) return false;
+        if (k.d % 4 != 0 || k.d < 4 || k.d > 256 || k.dv % 16 != 0 || k.dv < 16 || k.dv > 256 || k.sq < 1 || k.sk < 1) return false;
+        if ((q.s1 != 1 && k.d > 1) || kt.s0 != 1 || v.s1 != 1) return false;
+        if (kt.offset % 4 || kt.s1 % 4 || v.offset % 4 || v.s0 % 4) return false;
+        k.q_ld = q.s0;
+        k.k_ld = kt.s1;
+        k.v_ld = v.s0;
+        k.scale = n->cval;
+        return true;
+    }
+
+    void fuse_attention(std::vector<Node*>& topo, const std::set<Node*>& wanted_nodes) {
+        std::map<Node*, std::set<Node*>> consumers;
+        for (Node* n : topo) for_each_src(n, [&](Node* s, const Piece&, const TRef&) { consumers[s].insert(n); });
+        auto only_for = [&](Node* n, std::initializer_list<Node*> users) {
+            if (wanted_nodes.count(n) || n->force_root) return false;
+            std::set<Node*> u(users.begin(), users.end());
+            return consumers[n] == u;
+        };
+        const float kLog2e = 1.44269502162933349609375f;
+        for (Node* O : topo) {
+            if (O->op != Op::DOT) continue;
+            Node* P = whole_value(O->in[0]);
+            if (!P || P->op != Op::MUL || P->shape.size() != 2) continue;
+            const int64_t Sq = P->shape[0], Sk = P->shape[1];
+            // P = E * (1 / sum(E)) broadcast along the row
+            Node *E = nullptr, *R = nullptr;
+            for (int k = 0; k < 2 && !R; ++k) {
+                Node* e = whole_value(P->in[(size_t)k]);
+                Node* r = column_broadcast(P->in[(size_t)(1 - k)], Sq, Sk);
+                if (e && r && e->op == Op::EXP2 && r->op == Op::RECIP) { E = e; R = r; }
+            }
+            if (!E || !R) continue;
+            Node* S = whole_value(R->in[0]);
+            if (!S || S->op != Op::SUM || whole_value(S->in[0]) != E) continue;
+            // E = exp2((X - max(X)) * log2 e)
+            float c = 0.f;
+            Node* E1 = whole_value(E->in[0]);
+            Node* Dn = E1 ? times_constant(E1, c) : nullptr;
+            if (!Dn || c != kLog2e || Dn->op != Op::ADD) continue;
+            Node *X = nullptr, *N1 = nullptr, *M = nullptr;
+            // the maximum is negated either as a vector (and repeated along the row afterwards) or after the repetition
+            for (int k = 0; k < 2 && !M; ++k) {
+                Node* x = whole_value(Dn->in[(size_t)k]);
+                if (!x) continue;
+                const TRef& other = Dn->in[(size_t)(1 - k)];
+                Node* n1 = column_broadcast(other, Sq, Sk);
+                const bool negated_vector = n1 != nullptr;
+                if (!n1) n1 = whole_value(other);
+                if (!n1 || n1->op != Op::MUL || n1->in.size() != 2) continue;
+                float minus = 0.f;
+                for (int q = 0; q < 2 && !M; ++q) {
+                    Node* m = negated_vector ? whole_value(n1->in[(size_t)q]) : column_broadcast(n1->in[(size_t)q], Sq, Sk);
+                    if (m && m->op == Op::MAX && constant_operand(n1->in[(size_t)(1 - q)], minus) && minus == -1.0f && whole_value(m->in[0]) == x) {
+                        X = x; N1 = n1; M = m;
+                    }
+                }
+            }
+            if (!M) continue;
+            // X = scale * (Q K^T)
+            float scale = 0.f;
+            Node* D1 = times_constant(X, scale);
+            if (!D1 || D1->op != Op::DOT) continue;
+            if (!only_for(P, {O}) || !only_for(E, {P, S}) || !only_for(R, {P}) || !only_for(S, {R}) || !only_for(E1, {E}) ||
+                !only_for(Dn, {E1}) || !only_for(N1, {Dn}) || !only_for(M, {N1}) || !only_for(X, {Dn, M}) || !only_for(D1, {X}))
+                continue;
+            // would the kernel accept the operands as they are?
+            Node probe;
+            probe.in = {D1->in[0], D1->in[1], O->in[1]};
+            probe.cval = scale;
+            AttentionKey key;
+            Affine2D q, kt, v;
+            if (!attention_key(&probe, key, q, kt, v)) continue;
+            auto in_memory_able = [](const Affine2D& a) { return op_is_leaf(a.base->op) || op_is_elw(a.base->op) || a.base->root || op_is_reduce(a.base->op) || a.base->op == Op::DOT || a.base->op == Op::ATTN; };
+            if (!in_memory_able(q) || !in_memory_able(kt) || !in_memory_able(v)) continue;
+            O->op = Op::ATTN;
+            O->in = probe.in;
+            O->cval = scale;
+            O->key.clear();
+        }
+    }
+
     void flush_region(const IdSet& live, bool final_region, std::vector<Step>& out) {
         // ---- 1. what has to be in a home buffer when the region ends
         std::vector<std::pair<std::string, Node*>> wanted;
@@ -1043,18 +1180,30 @@ struct Lowerer {
             for (auto& w : wanted) dfs(w.second);
         }
         if (topo.empty()) { end_region(wanted); return; }
+        // ---- 2b. attention chains become one node
+        if (opt.fuse && opt.fuse_attention) {
+            fuse_attention(topo, wanted_nodes);
+            topo.clear();
+            std::set<Node*> seen;
+            std::function<void(Node*)> dfs = [&](Node* n) {
+                if (!seen.insert(n).second) return;
+                for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
+                topo.push_back(n);
+            };
+            for (auto& w : wanted) dfs(w.second);
+        }
         // ---- 3. forced roots
         for (auto& w : wanted) w.second->root = true;
         for (size_t i = 0; i < topo.size(); ++i) {
             Node* n = topo[i];
-            if (op_is_reduce(n->op) || n->op == Op::DOT || n->force_root) n->root = true;
+            if (op_is_reduce(n->op) || n->op == Op::DOT || n->op == Op::ATTN || n->force_root) n->root = true;
             if (!opt.fuse && op_is_elw(n->op)) n->root = true;
             if (numel(n->shape) == 0) n->root = false;
         }
         // matmul operands must be strided 2-D views of memory
         for (size_t i = 0; i < topo.size(); ++i) {
             Node* n = topo[i];
-            if (n->op != Op::DOT) continue;
+            if (n->op != Op::DOT && n->op != Op::ATTN) continue;
             for (TRef& t : n->in) {
                 Affine2D a2;
                 if (tref_affine2d(t, a2) && (op_is_leaf(a2.base->op) || op_is_elw(a2.base->op) || a2.base->root)) {
@@ -1218,7 +1367,7 @@ struct Lowerer {
             if (chosen < 0) {
                 Group g;
                 g.n = numel(r->shape);
-                g.kind = op_is_reduce(r->op) ? Group::SUM : (r->op == Op::DOT ? Group::DOT : (r->transpose ? Group::TRANSPOSE : Group::ELW));
+                g.kind = op_is_reduce(r->op) ? Group::SUM : (r->op == Op::DOT ? Group::DOT : (r->op == Op::ATTN ? Group::ATTN : (r->transpose ? Group::TRANSPOSE : Group::ELW)));
                 groups.push_back(g);
                 chosen = (int)groups.size() - 1;
             }
@@ -1823,6 +1972,10 @@ struct Lowerer {
                 emit_transpose(G.members[0], out);
                 continue;
             }
+            if (G.kind == Group::ATTN) {
+                emit_attention(G.members, out);
+                continue;
+            }
             GeneratedKernel& k = gks[g].k;
             if (G.kind == Group::ELW && !G.colsums.empty()) {
                 launch_generated(k);
@@ -1948,11 +2101,24 @@ struct Lowerer {
         std::vector<std::array<int64_t, 8>> key(G);
         std::vector<char> cand(G, 0);
         int ncand = 0;
-        for (int g = 0; g < G; ++g)
-            if (!groups[g].dead && groups[g].kind == Group::DOT && dot_group_key(groups[g].members[0], key[g]) && !keeps_epilogue(g)) {
+        for (int g = 0; g < G; ++g) {
+            if (groups[g].dead) continue;
+            if (groups[g].kind == Group::DOT && dot_group_key(groups[g].members[0], key[g]) && !keeps_epilogue(g)) {
+                cand[g] = 1;
+                ++ncand;
+            } else if (groups[g].kind == Group::ATTN) {
+                // the heads of multi-head attention: same shapes and strides, one launch (bit 40 keeps these keys
+                // apart from those of plain products)
+                AttentionKey ak;
+                Affine2D q, kt, v;
+                if (!attention_key(groups[g].members[0], ak, q, kt, v)) continue;
+                uint32_t sb;
+                memcpy(&sb, &ak.scale, 4);
+                key[g] = {ak.sq, ak.sk, ak.d, ak.dv, ak.q_ld, ak.k_ld, ak.v_ld, (int64_t)sb | (int64_t(1) << 40)};
                 cand[g] = 1;
                 ++ncand;
             }
+        }
         if (ncand < 2) return;
         // depth of every kernel
         std::vector<int> level(G, 0);
@@ -1989,7 +2155,7 @@ struct Lowerer {
                 for (int r = 0; r < g; ++r)
                     if (!groups[r].dead && reads_node(groups[r], li->second)) preds.insert(r);
             }
-            for (int p : preds) level[g] = std::max(level[g], level[p] + (groups[p].kind == Group::DOT ? 1 : 0));
+            for (int p : preds) level[g] = std::max(level[g], level[p] + (groups[p].kind == Group::DOT || groups[p].kind == Group::ATTN ? 1 : 0));
         }
         // sets of at least two
         std::map<std::pair<int, std::array<int64_t, 8>>, std::vector<int>> sets;
@@ -2004,7 +2170,8 @@ struct Lowerer {
             if (!groups[g].dead) order.push_back(g);
         std::stable_sort(order.begin(), order.end(), [&](int x, int y) {
             if (level[x] != level[y]) return level[x] < level[y];
-            return (groups[x].kind == Group::DOT) < (groups[y].kind == Group::DOT);
+            auto product = [&](int g) { return groups[g].kind == Group::DOT || groups[g].kind == Group::ATTN; };
+            return product(x) < product(y);
         });
         std::vector<int> new_index(G, -1);
         std::vector<Group> sorted;
@@ -2139,6 +2306,57 @@ struct Lowerer {
             lf.flops = (double)cnt * (double)M * (double)N * (double)pl.splits;
             push_launch(out, lf, "sum_slices");
         }
+    }
+
+    // One launch of the fused attention kernel for up to 16 problems of one shape (block row y works on problem y).
+    void emit_attention(const std::vector<Node*>& atts, std::vector<Step>& out) {
+        const int cnt = (int)atts.size();
+        ADHIP_CHECK(cnt >= 1 && cnt <= kAttentionSlots, "internal: attention launch of %d problems", cnt);
+        AttentionKey key0;
+        Affine2D q0, k0, v0;
+        ADHIP_CHECK(attention_key(atts[0], key0, q0, k0, v0), "internal: attention node whose operands the kernel cannot read");
+        AttentionConfig cfg;
+        cfg.d = (int)key0.d;
+        cfg.dv = (int)key0.dv;
+        const int64_t row_blocks = (key0.sq + 63) / 64;
+        // 64 keys per step while that leaves room in LDS and the launch is too small for several blocks per CU anyway;
+        // 32 keys per step otherwise (half the LDS, two to three blocks per CU)
+        cfg.bn = (cfg.d <= 128 && cfg.dv <= 128 && row_blocks * cnt < 512) ? 64 : 32;
+        const std::string entry = strf("adhip_attention_d%d_v%d_k%d", cfg.d, cfg.dv, cfg.bn);
+        Launch l;
+        l.kernel = add_kernel(entry, attention_kernel_source(cfg, entry), "attention");
+        l.block[0] = 256;
+        l.grid[0] = (unsigned)row_blocks;
+        l.grid[1] = (unsigned)cnt;
+        auto B = [&](Node* x, int64_t off) {
+            Arg a;
+            a.kind = Arg::BUF;
+            ADHIP_CHECK(x->buffer >= 0, "internal: attention operand without buffer");
+            a.buf = x->buffer;
+            a.off = off;
+            return a;
+        };
+        auto I = [&](int64_t v) { Arg a; a.kind = Arg::I64; a.iv = v; return a; };
+        for (int i = 0; i < kAttentionSlots; ++i) {
+            Node* n = atts[(size_t)std::min(i, cnt - 1)];  // unused slots repeat the last problem; no block reads them
+            AttentionKey key;
+            Affine2D q, kt, v;
+            ADHIP_CHECK(attention_key(n, key, q, kt, v) && key == key0, "internal: attention problems of one launch differ");
+            l.args.push_back(B(n, 0));
+            l.args.push_back(B(q.base, q.offset));
+            l.args.push_back(B(kt.base, kt.offset));
+            l.args.push_back(B(v.base, v.offset));
+        }
+        for (int64_t v : {key0.sq, key0.sk, key0.q_ld, key0.k_ld, key0.v_ld}) l.args.push_back(I(v));
+        Arg sc;
+        sc.kind = Arg::F32;
+        sc.fv = key0.scale;
+        l.args.push_back(sc);
+        l.label = strf("attention_%s_%dx_%lldx%lldx%lldx%lld", atts[0]->name.c_str(), cnt, (long long)key0.sq, (long long)key0.sk,
+                       (long long)key0.d, (long long)key0.dv);
+        l.bytes = 4.0 * cnt * ((double)key0.sq * key0.d + (double)key0.sk * key0.d + (double)key0.sk * key0.dv + (double)key0.sq * key0.dv);
+        l.flops = 2.0 * cnt * (double)key0.sq * (double)key0.sk * (double)(key0.d + key0.dv);
+        push_launch(out, l, "attention");
     }
 
     // whether a product goes to the matrix-core kernel (else the one-thread-per-output kernel)
@@ -2589,6 +2807,7 @@ std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::str
     LowerOptions opt = opt_in;
     if (const char* e = getenv("ADHIP_GROUP_DOTS")) opt.group_dots = opt.group_dots && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_LAYER_KERNELS")) opt.layer_kernels = opt.layer_kernels && atoi(e) != 0;
+    if (const char* e = getenv("ADHIP_FUSE_ATTENTION")) opt.fuse_attention = opt.fuse_attention && atoi(e) != 0;
     Lowerer l(prog, dep_ids, opt);
     return l.run();
 }

@@ -16,6 +16,7 @@ struct LowerOptions {
     bool fuse = true;  // false: one kernel per compute command (diagnostic mode)
     bool group_dots = true;  // same-shape independent matrix products share a launch
     bool layer_kernels = true;  // groups that run the same generated kernels on other buffers share their launches
+    bool fuse_attention = true;  // dot(softmax(scale * dot(Q, K^T)), V) runs as one kernel
 };
 
 std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids,

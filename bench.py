@@ -151,6 +151,41 @@ def measure_mlp(dev, iters):
     return out
 
 
+MFMA_FP32_PEAK_TFLOPS = 157.3
+
+
+def measure_attention(dev, seq=2048, d_model=1024, heads=8):
+    """Multi-head attention forward (inference), [seq, d_model] activations: the fused attention kernel's rate against
+    the FP32 matrix-core peak, and the same program lowered without the fusion beside it."""
+    out = {}
+    for mode in ("fused", "unfused"):
+        if mode == "unfused":
+            os.environ["ADHIP_FUSE_ATTENTION"] = "0"
+        try:
+            wl = W.attention_forward(dev, seq, d_model, heads, seed=0)
+            prog = compile_resident(dev, wl)
+        finally:
+            os.environ.pop("ADHIP_FUSE_ATTENTION", None)
+        ms = timed_runs(prog, 10, 3)
+        ks = profile(prog, 3)
+        entry = {"ms_per_step": ms, "launches_per_step": sum(k["launches_per_run"] for k in ks),
+                 "matmul_TFLOPs_whole_step": wl.flops / (ms * 1e-3) / 1e12}
+        if mode == "fused":
+            for k in ks:
+                if k["kernel"].startswith("attention"):
+                    tf = wl.attention_flops / (k["avg_ms"] * 1e-3) / 1e12
+                    entry["roofline"] = {"kernel": k["kernel"], "bound": "mfma", "achieved": tf, "peak": MFMA_FP32_PEAK_TFLOPS,
+                                         "unit": "TFLOP/s", "frac": tf / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+                                         "avg_ms": k["avg_ms"],
+                                         "flops_per_launch": wl.attention_flops,
+                                         "note": "2 * 2 * seq^2 * head_width flops per head (the two products; the "
+                                                 "softmax arithmetic is not counted), all heads in one launch"}
+        out[mode] = entry
+        prog.close()
+    out["config"] = {"seq": seq, "d_model": d_model, "heads": heads}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,7 +194,7 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "attention"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by; "
                          "'streammix': only a bare 3-reads + 4-writes kernel over 8192x8192 f32 (the stream mix of the "
@@ -215,6 +250,9 @@ def main():
         ms3 = timed_runs(p3, args.steps, args.warmup)
         print(json.dumps({"metric": "reductions forward + backward, f32 [16384,4096]", "value": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
                           "unit": "GB/s", "ms_per_step": ms3, "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}))
+        return
+    if args.workload == "attention":
+        print(json.dumps(dict(measure_attention(dev), metric="multi-head attention forward, fp32")))
         return
     if args.workload == "mlp":
         print(json.dumps(dict(measure_mlp(dev, args.mlp_iters), metric="fp32 MLP train steps/s")))
@@ -301,6 +339,7 @@ def main():
                                   "matmul_TFLOPs_whole_step": wl6.flops / (ms6 * 1e-3) / 1e12,
                                   "matmul_kernels_ms": dot6, "launches_per_step": sum(k["launches_per_run"] for k in k6)}
         p6.close()
+        extra["attention_forward"] = measure_attention(dev)
 
     cpu = None
     if not args.skip_cpu:

@@ -137,3 +137,200 @@ def test_encoder_training_loop_matches_oracle(seq, d_model, heads, ff, hip_devic
         assert np.abs(moved_ref).max() > 1e-4, f"{k} did not train"
         err = np.abs(moved_got - moved_ref).max()
         assert err <= 2e-3 * np.abs(moved_ref).max() + 4e-7 * np.abs(w0).max(), (k, err, np.abs(moved_ref).max())
+
+
+# ---- fused attention --------------------------------------------------------------------------------------------
+
+def _attention_float64(q, k, v, d_model, mask=None):
+    s = q.astype(np.float64) @ k.astype(np.float64).T / math.sqrt(float(d_model))
+    if mask is not None:
+        s = s * mask
+    e = np.exp(s - s.max(-1, keepdims=True))
+    return (e / e.sum(-1, keepdims=True)) @ v.astype(np.float64)
+
+
+def _attention_program(dev, sq, sk, d, dv, d_model, seed, spread=1.0, mask=False, keep_scores=False):
+    """O = Attention(Q, K, V) on tensors handed in as they are: Q [sq, d], K [sk, d], V [sk, dv]."""
+    from adhip import nn
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(seed)
+    qn = (spread * rng.standard_normal((sq, d))).astype(np.float32)
+    kn = (spread * rng.standard_normal((sk, d))).astype(np.float32)
+    vn = rng.standard_normal((sk, dv)).astype(np.float32)
+    mn = (rng.random((sq, sk)) < 0.7).astype(np.float32) if mask else None
+    Q, K, V = autodiff.tensor(qn, [sq, d]), autodiff.tensor(kn, [sk, d]), autodiff.tensor(vn, [sk, dv])
+    if mask:
+        o = nn.AttentionMasked(Q, K, V, d_model, autodiff.tensor(mn, [sq, sk]))
+    else:
+        o = nn.Attention(Q, K, V, d_model)
+    o.forward()
+    o.val().keep()
+    return o, (qn, kn, vn, mn)
+
+
+_FUSED_SHAPES = [
+    # sq, sk, d, dv: one query block and many, ragged in both directions, narrow and wide heads, sq != sk, d != dv
+    (64, 64, 16, 16), (100, 100, 48, 48), (1, 7, 4, 16), (65, 129, 8, 32), (300, 77, 64, 64), (257, 640, 128, 128),
+    (130, 1000, 36, 80), (96, 200, 256, 256), (200, 96, 20, 240),
+]
+
+
+@pytest.mark.parametrize("sq,sk,d,dv", _FUSED_SHAPES)
+def test_attention_lowers_to_one_kernel(sq, sk, d, dv):
+    from adhip.core import ValueData
+    from adhip.device import Device, lower_describe
+
+    class Capture(Device):
+        def execute(self, proc, deps):
+            self.proc, self.deps = proc, list(deps)
+
+        def get_tensor(self, id):
+            return ValueData.none()
+
+    dev = Capture()
+    _attention_program(dev, sq, sk, d, dv, 64, 0)
+    autodiff.execute()
+    launches = [l for l in lower_describe(dev.proc, dev.deps).splitlines() if l.lstrip().startswith("launch")]
+    assert len(launches) == 1 and "[attention]" in launches[0], launches
+    assert f"adhip_attention_d{d}_v{dv}_k" in launches[0]
+
+
+@pytest.mark.parametrize("what", ["mask", "scores_kept", "head_of_6", "plain_exp"])
+def test_attention_that_does_not_match_stays_unfused(what, monkeypatch):
+    """A mask between the scaling and the softmax, a softmax somebody else reads, a head width the kernel has no tile
+    for, or the reference's own max-less softmax: none of them is the fused kernel's arithmetic."""
+    from adhip.core import ValueData
+    from adhip.device import Device, lower_describe
+
+    class Capture(Device):
+        def execute(self, proc, deps):
+            self.proc, self.deps = proc, list(deps)
+
+        def get_tensor(self, id):
+            return ValueData.none()
+
+    dev = Capture()
+    autodiff.set_device(dev)
+    if what == "mask":
+        _attention_program(dev, 64, 64, 16, 16, 64, 0, mask=True)
+    elif what == "head_of_6":
+        _attention_program(dev, 64, 64, 6, 16, 64, 0)
+    else:
+        rng = np.random.default_rng(0)
+        Q, K, V = (autodiff.tensor(rng.standard_normal((64, 16)).astype(np.float32), [64, 16]) for _ in range(3))
+        s = dot(Q, K.t()) / 8.0
+        if what == "scores_kept":
+            p = s.softmax(-1)
+        else:
+            e = s.exp()
+            p = e / e.sum(-1).unsqueeze(-1)
+        o = dot(p, V)
+        o.forward()
+        o.val().keep()
+        if what == "scores_kept":
+            p.val().keep()
+    autodiff.execute()
+    text = lower_describe(dev.proc, dev.deps)
+    assert "[attention]" not in text, text
+
+
+def test_attention_fusion_can_be_switched_off(monkeypatch):
+    from adhip.core import ValueData
+    from adhip.device import Device, lower_describe
+
+    class Capture(Device):
+        def execute(self, proc, deps):
+            self.proc, self.deps = proc, list(deps)
+
+        def get_tensor(self, id):
+            return ValueData.none()
+
+    dev = Capture()
+    _attention_program(dev, 64, 64, 16, 16, 64, 0)
+    autodiff.execute()
+    assert "[attention]" in lower_describe(dev.proc, dev.deps)
+    monkeypatch.setenv("ADHIP_FUSE_ATTENTION", "0")
+    assert "[attention]" not in lower_describe(dev.proc, dev.deps)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sq,sk,d,dv", _FUSED_SHAPES)
+def test_fused_attention_matches_oracle_and_float64(sq, sk, d, dv, hip_device):
+    """The fused kernel against the oracle running the unfused commands, and both against float64.  Scores reach a few
+    tens: without the running maximum exp2 would lose the small terms or overflow."""
+    print(f"[case] fused attention {sq}x{sk} d {d} dv {dv}", flush=True)
+    o, (qn, kn, vn, _) = _attention_program(hip_device, sq, sk, d, dv, 16, sq + sk, spread=2.0)
+    autodiff.execute()
+    got = o.val().get()
+    ro, _ = _attention_program(OracleDevice(), sq, sk, d, dv, 16, sq + sk, spread=2.0)
+    autodiff.execute()
+    ref = ro.val().get()
+    assert got.dim == ref.dim == [sq, dv]
+    tol = RED_RTOL * math.sqrt(max(sk, d))
+    assert_close(got.data, ref.data, 4 * tol, "o vs oracle")
+    assert_close(got.data, _attention_float64(qn, kn, vn, 16).reshape(-1), 4 * tol, "o vs float64")
+
+
+@pytest.mark.gpu
+def test_fused_attention_survives_extreme_scores(hip_device):
+    """Rows whose scores differ by hundreds (one key wins outright), a row of identical scores, and a key block in which
+    every score is far below the running maximum."""
+    print("[case] fused attention extreme scores", flush=True)
+    autodiff.set_device(hip_device)
+    sq, sk, d, dv = 70, 200, 16, 32
+    rng = np.random.default_rng(11)
+    qn = rng.standard_normal((sq, d)).astype(np.float32) * 30.0
+    kn = rng.standard_normal((sk, d)).astype(np.float32) * 30.0
+    qn[3, :] = 0.0                      # all scores equal: the mean of V
+    kn[64:128, :] *= 1e-3               # a whole block of keys that hardly counts
+    vn = rng.standard_normal((sk, dv)).astype(np.float32)
+    Q, K, V = autodiff.tensor(qn, [sq, d]), autodiff.tensor(kn, [sk, d]), autodiff.tensor(vn, [sk, dv])
+    from adhip import nn
+    o = nn.Attention(Q, K, V, 4)
+    o.forward()
+    o.val().keep()
+    autodiff.execute()
+    got = np.asarray(o.val().get().data, dtype=np.float64).reshape(sq, dv)
+    ref = _attention_float64(qn, kn, vn, 4)
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got[3], vn.astype(np.float64).mean(0), rtol=0, atol=2e-6)
+    # a product of 16 terms of size 900 carries an absolute error of 1e-4 into the exponent
+    np.testing.assert_allclose(got, ref, rtol=0, atol=2e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seq,d_model,heads", [(100, 96, 2), (128, 64, 4), (320, 512, 2)])
+def test_attention_forward_workload_fused_equals_unfused(seq, d_model, heads, hip_device, monkeypatch):
+    """Multi-head attention end to end (projections, fused attention of all heads in one launch, concatenation, output
+    projection) against the same program lowered without the fusion, and against the oracle."""
+    print(f"[case] attention forward {seq}x{d_model} heads {heads}", flush=True)
+    fused = W.attention_forward(hip_device, seq, d_model, heads, seed=seq).run()["y"]
+    monkeypatch.setenv("ADHIP_FUSE_ATTENTION", "0")
+    plain = W.attention_forward(hip_device, seq, d_model, heads, seed=seq).run()["y"]
+    monkeypatch.delenv("ADHIP_FUSE_ATTENTION")
+    ref = W.attention_forward(OracleDevice(), seq, d_model, heads, seed=seq).run()["y"]
+    tol = 4 * RED_RTOL * math.sqrt(max(seq, d_model))
+    assert_close(fused.data, plain.data, tol, "fused vs unfused")
+    assert_close(fused.data, ref.data, tol, "fused vs oracle")
+
+
+@pytest.mark.gpu
+def test_attention_forward_full_size_matches_float64(hip_device):
+    """2048 tokens, d_model 1024, 8 heads of 128: the size the throughput is quoted on, against float64 on sampled
+    rows of every head's share of the output."""
+    print("[case] attention forward 2048x1024 heads 8", flush=True)
+    seq, d_model, heads = 2048, 1024, 8
+    wl = W.attention_forward(hip_device, seq, d_model, heads, seed=1, scale_x=3.0)
+    got = np.asarray(wl.run()["y"].data, dtype=np.float64).reshape(seq, d_model)
+    x = wl.inputs["x"].astype(np.float64)
+    d_v = d_model // heads
+    rows = [0, 1, 63, 64, 1000, 1027, 2047]
+    cat = np.zeros((len(rows), d_model))
+    for h in range(heads):
+        q = x[rows] @ wl.inputs[f"wq{h}"].astype(np.float64)
+        k = x @ wl.inputs[f"wk{h}"].astype(np.float64)
+        v = x @ wl.inputs[f"wv{h}"].astype(np.float64)
+        cat[:, h * d_v:(h + 1) * d_v] = _attention_float64(q, k, v, d_model)
+    ref = cat @ wl.inputs["wo"].astype(np.float64)
+    err = np.abs(got[rows] - ref).max()
+    assert err <= RED_RTOL * math.sqrt(seq) * np.abs(ref).max() * 4, err
