@@ -157,6 +157,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 def measure_attention(dev, seq=2048, d_model=1024, heads=8):
     """Multi-head attention forward (inference), [seq, d_model] activations: the fused attention kernel's rate against
     the FP32 matrix-core peak, and the same program lowered without the fusion beside it."""
+    from adhip import workloads as W
     out = {}
     for mode in ("fused", "unfused"):
         if mode == "unfused":
