@@ -1121,10 +1121,74 @@ struct Lowerer {
         }
     }
 
-    void flush_region(const IdSet& live, bool final_region, std::vector<Step>& out) {
-        // ---- 1. what has to be in a home buffer when the region ends
-        std::vector<std::pair<std::string, Node*>> wanted;
+    // ---------------------------------------------------------------------------------------------------------
+    // A straight-line region is lowered by a sequence of passes over one RegionPlan.  Each pass names, in the
+    // references at its top, the parts of the plan it reads or changes.
+    // ---------------------------------------------------------------------------------------------------------
+    struct GroupKernels {
+        GeneratedKernel k;
+        std::vector<GeneratedKernel> extra;
+        std::vector<Node*> extra_nodes;
+        DotEpilogueCode dot_epi;   // DOT groups with an epilogue
+        bool dot_store = true;     // ... and whether the product itself is still written
+    };
+    struct Commit { int dst, src; int64_t n; std::string id; };
+    struct RegionPlan {
+        std::vector<std::pair<std::string, Node*>> wanted;  // (id, node) that must be in the id's home buffer at the end
         std::set<Node*> wanted_nodes;
+        std::vector<Node*> topo;                             // every needed node, producers first
+        std::map<Node*, std::map<Node*, bool>> reads;        // per root: in-memory values it reads (true: element for element only)
+        std::map<Node*, std::set<Node*>> folded_in;          // per root: folded nodes it evaluates at its own index
+        std::vector<Group> groups;                           // kernels, in launch order
+        std::map<Node*, int> group_of;
+        std::map<Node*, std::string> home_of;                // wanted node -> id
+        std::vector<GroupKernels> gks;                       // per group: generated code
+        std::vector<std::map<Node*, bool>> greads;           // per group: reads, for hazard analysis
+        std::vector<int> set_end;                            // per group: last group of the shared launches it runs in
+        std::vector<Commit> commits;                         // results computed beside their home buffer, copied in at the end
+    };
+
+    void order_nodes(RegionPlan& rp) {
+        rp.topo.clear();
+        std::set<Node*> seen;
+        std::function<void(Node*)> dfs = [&](Node* n) {
+            if (!seen.insert(n).second) return;
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
+            rp.topo.push_back(n);
+        };
+        for (auto& w : rp.wanted) dfs(w.second);
+    }
+
+    void flush_region(const IdSet& live, bool final_region, std::vector<Step>& out) {
+        RegionPlan rp;
+        collect_wanted(rp, live, final_region);
+        order_nodes(rp);
+        if (rp.topo.empty()) { end_region(rp.wanted); return; }
+        if (opt.fuse && opt.fuse_attention) {
+            fuse_attention(rp.topo, rp.wanted_nodes);
+            order_nodes(rp);
+        }
+        force_roots(rp);
+        if (opt.fuse) plan_transposed_copies(rp);
+        keep_shared_values(rp);
+        form_groups(rp);
+        if (opt.fuse) {
+            attach_column_sums(rp);
+            attach_row_sum_operands(rp);
+            fold_transposed_copies(rp);
+            if (opt.group_dots) group_independent_products(rp);
+        }
+        generate_kernels(rp);
+        if (opt.fuse && opt.layer_kernels) share_launches(rp);
+        assign_buffers(rp);
+        emit_launches(rp, out);
+        end_region(rp.wanted);
+    }
+
+    // ---- 1. what has to be in a home buffer when the region ends
+    void collect_wanted(RegionPlan& rp, const IdSet& live, bool final_region) {
+        auto& wanted = rp.wanted;
+        auto& wanted_nodes = rp.wanted_nodes;
         auto want = [&](const std::string& id, Node* n) {
             if (numel(n->shape) == 0) return;
             if (op_is_leaf(n->op) || wanted_nodes.count(n)) n = new_node(Op::COPY, n->shape, {tr_node(n, n->shape)}, id, 0.f, false);
@@ -1168,31 +1232,13 @@ struct Lowerer {
                 wanted.push_back({id, n});
             }
         }
-        // ---- 2. needed nodes in topological order
-        std::vector<Node*> topo;
-        {
-            std::set<Node*> seen;
-            std::function<void(Node*)> dfs = [&](Node* n) {
-                if (!seen.insert(n).second) return;
-                for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
-                topo.push_back(n);
-            };
-            for (auto& w : wanted) dfs(w.second);
-        }
-        if (topo.empty()) { end_region(wanted); return; }
-        // ---- 2b. attention chains become one node
-        if (opt.fuse && opt.fuse_attention) {
-            fuse_attention(topo, wanted_nodes);
-            topo.clear();
-            std::set<Node*> seen;
-            std::function<void(Node*)> dfs = [&](Node* n) {
-                if (!seen.insert(n).second) return;
-                for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
-                topo.push_back(n);
-            };
-            for (auto& w : wanted) dfs(w.second);
-        }
-        // ---- 3. forced roots
+    }
+
+    // ---- 3. values that get a kernel and a buffer of their own whatever happens; product operands that are not
+    // strided 2-D views of memory are copied first
+    void force_roots(RegionPlan& rp) {
+        auto& wanted = rp.wanted;
+        auto& topo = rp.topo;
         for (auto& w : wanted) w.second->root = true;
         for (size_t i = 0; i < topo.size(); ++i) {
             Node* n = topo[i];
@@ -1216,139 +1262,128 @@ struct Lowerer {
                 t = tr_node(c, t.shape);
             }
         }
-        // recompute topo (copies were added)
-        topo.clear();
-        {
-            std::set<Node*> seen;
-            std::function<void(Node*)> dfs = [&](Node* n) {
-                if (!seen.insert(n).second) return;
-                for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
-                topo.push_back(n);
-            };
-            for (auto& w : wanted) dfs(w.second);
-        }
-        // ---- 3b. large operands read against the grain (unit stride on a dim that is not the innermost one
-        // of the consumer) are first copied densely by the tiled transposing kernel
-        if (opt.fuse) {
-            std::vector<Node*> work = topo;
-            std::stable_sort(work.begin(), work.end(), [](Node* a, Node* b) { return a->order < b->order; });
-            std::map<std::string, Node*> transposed;  // region of a source node -> its dense copy
-            bool added = false;
-            for (Node* n : work) {
-                if (!op_is_elw(n->op) || n->transpose) continue;
-                for (TRef& t : n->in) {
-                    for (Piece& pc : t.pieces) {
-                        if (pc.src.kind != Src::NODE || !in_mem(pc.src.node) || pc.view.st.empty()) continue;
-                        // the last stage is the one that addresses the buffer; earlier stages only
-                        // produce a row-major index into its shape, which a dense copy keeps valid
-                        const Stage st = pc.view.st.back();
-                        int last = -1, u = -1, nbatch = 0;
-                        for (int d = (int)st.shape.size() - 1; d >= 0; --d)
-                            if (st.shape[d] > 1) { last = d; break; }
-                        if (last < 0 || st.stride[last] <= 1) continue;
+        order_nodes(rp);  // copies were added
+    }
+
+    // ---- 3b. large operands read against the grain (unit stride on a dim that is not the innermost one
+    // of the consumer) are first copied densely by the tiled transposing kernel
+    void plan_transposed_copies(RegionPlan& rp) {
+        auto& topo = rp.topo;
+        std::vector<Node*> work = topo;
+        std::stable_sort(work.begin(), work.end(), [](Node* a, Node* b) { return a->order < b->order; });
+        std::map<std::string, Node*> transposed;  // region of a source node -> its dense copy
+        bool added = false;
+        for (Node* n : work) {
+            if (!op_is_elw(n->op) || n->transpose) continue;
+            for (TRef& t : n->in) {
+                for (Piece& pc : t.pieces) {
+                    if (pc.src.kind != Src::NODE || !in_mem(pc.src.node) || pc.view.st.empty()) continue;
+                    // the last stage is the one that addresses the buffer; earlier stages only
+                    // produce a row-major index into its shape, which a dense copy keeps valid
+                    const Stage st = pc.view.st.back();
+                    int last = -1, u = -1, nbatch = 0;
+                    for (int d = (int)st.shape.size() - 1; d >= 0; --d)
+                        if (st.shape[d] > 1) { last = d; break; }
+                    if (last < 0 || st.stride[last] <= 1) continue;
+                    for (int d = 0; d < last; ++d)
+                        if (st.shape[d] > 1 && st.stride[d] == 1) u = d;
+                    if (u < 0 || st.shape[u] < 16 || st.shape[last] < 16 || numel(st.shape) < (int64_t(1) << 18)) continue;
+                    for (int d = 0; d < last; ++d)
+                        if (d != u && st.shape[d] > 1) ++nbatch;
+                    if (nbatch > 3) continue;
+                    {
+                        // every 64x64 tile of every batch is one block along grid dimension x
+                        int64_t blocks = ((st.shape[u] + 63) / 64) * ((st.shape[last] + 63) / 64);
                         for (int d = 0; d < last; ++d)
-                            if (st.shape[d] > 1 && st.stride[d] == 1) u = d;
-                        if (u < 0 || st.shape[u] < 16 || st.shape[last] < 16 || numel(st.shape) < (int64_t(1) << 18)) continue;
-                        for (int d = 0; d < last; ++d)
-                            if (d != u && st.shape[d] > 1) ++nbatch;
-                        if (nbatch > 3) continue;
-                        {
-                            // every 64x64 tile of every batch is one block along grid dimension x
-                            int64_t blocks = ((st.shape[u] + 63) / 64) * ((st.shape[last] + 63) / 64);
-                            for (int d = 0; d < last; ++d)
-                                if (d != u && st.shape[d] > 1) blocks *= st.shape[d];
-                            if (blocks > 0x7fffffff) continue;
-                        }
-                        // a dense copy of exactly this region that must be in memory anyway (Contigious, a kept view)
-                        // is written by the transposing kernel itself; later readers of the region read that copy
-                        const std::string region_key = std::to_string(pc.src.node->id) + "@" + stage_str(st);
-                        Node* T = nullptr;
-                        auto known = transposed.find(region_key);
-                        if (known != transposed.end() && known->second->order < n->order) T = known->second;
-                        if (!T && n->root && n->op == Op::COPY && t.single_full() && pc.view.st.size() == 1 && t.shape == st.shape &&
-                            n->shape == st.shape) {
-                            n->transpose = true;
-                            n->transpose_u = u;
-                            transposed[region_key] = n;
-                            added = true;
-                            continue;
-                        }
-                        if (!T) {
-                            TRef region;
-                            region.shape = st.shape;
-                            Piece whole;
-                            whole.lo.assign(st.shape.size(), 0);
-                            whole.hi = st.shape;
-                            whole.view.st = {st};
-                            whole.src = pc.src;
-                            region.pieces.push_back(whole);
-                            T = new_node(Op::COPY, st.shape, {region}, pc.src.node->name + ".t", 0.f, true);
-                            T->root = true;
-                            T->transpose = true;
-                            T->transpose_u = u;
-                            T->order = std::min(T->order, n->order - 0.25);
-                            transposed[region_key] = T;
-                        }
-                        pc.view.st.back() = contiguous_stage(st.shape);
-                        pc.src = Src();
-                        pc.src.kind = Src::NODE;
-                        pc.src.node = T;
-                        added = true;
+                            if (d != u && st.shape[d] > 1) blocks *= st.shape[d];
+                        if (blocks > 0x7fffffff) continue;
                     }
+                    // a dense copy of exactly this region that must be in memory anyway (Contigious, a kept view)
+                    // is written by the transposing kernel itself; later readers of the region read that copy
+                    const std::string region_key = std::to_string(pc.src.node->id) + "@" + stage_str(st);
+                    Node* T = nullptr;
+                    auto known = transposed.find(region_key);
+                    if (known != transposed.end() && known->second->order < n->order) T = known->second;
+                    if (!T && n->root && n->op == Op::COPY && t.single_full() && pc.view.st.size() == 1 && t.shape == st.shape &&
+                        n->shape == st.shape) {
+                        n->transpose = true;
+                        n->transpose_u = u;
+                        transposed[region_key] = n;
+                        added = true;
+                        continue;
+                    }
+                    if (!T) {
+                        TRef region;
+                        region.shape = st.shape;
+                        Piece whole;
+                        whole.lo.assign(st.shape.size(), 0);
+                        whole.hi = st.shape;
+                        whole.view.st = {st};
+                        whole.src = pc.src;
+                        region.pieces.push_back(whole);
+                        T = new_node(Op::COPY, st.shape, {region}, pc.src.node->name + ".t", 0.f, true);
+                        T->root = true;
+                        T->transpose = true;
+                        T->transpose_u = u;
+                        T->order = std::min(T->order, n->order - 0.25);
+                        transposed[region_key] = T;
+                    }
+                    pc.view.st.back() = contiguous_stage(st.shape);
+                    pc.src = Src();
+                    pc.src.kind = Src::NODE;
+                    pc.src.node = T;
+                    added = true;
                 }
             }
-            if (added) {
-                topo.clear();
-                std::set<Node*> seen;
-                std::function<void(Node*)> dfs = [&](Node* n) {
-                    if (!seen.insert(n).second) return;
-                    for_each_src(n, [&](Node* s, const Piece&, const TRef&) { dfs(s); });
-                    topo.push_back(n);
-                };
-                for (auto& w : wanted) dfs(w.second);
-            }
         }
-        // ---- 4. folded nodes used by several kernels: keep in memory when recomputing costs more
-        {
-            std::map<Node*, std::set<std::string>> users;
-            std::map<Node*, std::set<Node*>> bigleaves;
-            for (Node* n : topo) {  // producers first
-                if (in_mem(n)) continue;
-                std::set<Node*>& bl = bigleaves[n];
-                for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
-                    if (in_mem(s)) { if (numel(s->shape) * 2 >= numel(n->shape)) bl.insert(s); }
-                    else bl.insert(bigleaves[s].begin(), bigleaves[s].end());
-                });
-            }
-            for (size_t i = topo.size(); i-- > 0;) {  // consumers first
-                Node* n = topo[i];
-                std::set<std::string> mine;
-                int64_t csr = 0, csc = 0;
-                if (n->root && opt.fuse && colsum_source(n, csr, csc)) mine.insert("E" + std::to_string(csr * csc));
-                else if (n->root) mine.insert(op_is_elw(n->op) ? "E" + std::to_string(numel(n->shape)) : "K" + std::to_string(n->id));
-                else mine = users[n];
-                if (!n->root && op_is_elw(n->op) && users[n].size() >= 2 && bigleaves[n].size() >= 3) {
-                    n->root = true;
-                    mine.clear();
-                    mine.insert("E" + std::to_string(numel(n->shape)));
-                }
-                for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
-                    if (!in_mem(s)) users[s].insert(mine.begin(), mine.end());
-                });
-            }
+        if (added) order_nodes(rp);
+    }
+
+    // ---- 4. folded nodes used by several kernels: keep in memory when recomputing costs more
+    void keep_shared_values(RegionPlan& rp) {
+        auto& topo = rp.topo;
+        std::map<Node*, std::set<std::string>> users;
+        std::map<Node*, std::set<Node*>> bigleaves;
+        for (Node* n : topo) {  // producers first
+            if (in_mem(n)) continue;
+            std::set<Node*>& bl = bigleaves[n];
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                if (in_mem(s)) { if (numel(s->shape) * 2 >= numel(n->shape)) bl.insert(s); }
+                else bl.insert(bigleaves[s].begin(), bigleaves[s].end());
+            });
         }
-        // ---- 5. group roots into kernels
+        for (size_t i = topo.size(); i-- > 0;) {  // consumers first
+            Node* n = topo[i];
+            std::set<std::string> mine;
+            int64_t csr = 0, csc = 0;
+            if (n->root && opt.fuse && colsum_source(n, csr, csc)) mine.insert("E" + std::to_string(csr * csc));
+            else if (n->root) mine.insert(op_is_elw(n->op) ? "E" + std::to_string(numel(n->shape)) : "K" + std::to_string(n->id));
+            else mine = users[n];
+            if (!n->root && op_is_elw(n->op) && users[n].size() >= 2 && bigleaves[n].size() >= 3) {
+                n->root = true;
+                mine.clear();
+                mine.insert("E" + std::to_string(numel(n->shape)));
+            }
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                if (!in_mem(s)) users[s].insert(mine.begin(), mine.end());
+            });
+        }
+    }
+
+    // ---- 5. group roots into kernels
+    void form_groups(RegionPlan& rp) {
+        auto& topo = rp.topo;
+        auto& reads = rp.reads;
+        auto& folded_in = rp.folded_in;
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
         // kernels run in program order: it is a valid topological order, and it keeps in-place updates
         // after the reads of the old value that precede them in the program
         std::vector<Node*> roots;
         for (Node* n : topo)
             if (n->root && !op_is_leaf(n->op)) roots.push_back(n);
         std::stable_sort(roots.begin(), roots.end(), [](Node* a, Node* b) { return a->order < b->order; });
-        std::map<Node*, std::map<Node*, bool>> reads;
-        std::map<Node*, std::set<Node*>> folded_in;  // per root: folded nodes it evaluates at its own index
         for (Node* r : roots) collect_reads(r, reads[r], &folded_in[r]);
-        std::vector<Group> groups;
-        std::map<Node*, int> group_of;
         for (Node* r : roots) {
             int chosen = -1;
             if (op_is_elw(r->op) && opt.fuse && !r->transpose) {
@@ -1374,217 +1409,241 @@ struct Lowerer {
             groups[chosen].members.push_back(r);
             group_of[r] = chosen;
         }
-        // ---- 5b. column sums ride along with the element-wise pass that computes their operand
-        if (opt.fuse) {
-            for (size_t gs = 0; gs < groups.size(); ++gs) {
-                if (groups[gs].kind != Group::SUM) continue;
-                Node* S = groups[gs].members[0];
-                int64_t R = 0, C = 0;
-                Node* E = colsum_source(S, R, C);
-                if (!E) continue;
-                int target = -1;
-                for (size_t g = 0; g < groups.size() && target < 0; ++g) {
+        for (auto& w : rp.wanted) rp.home_of[w.second] = w.first;
+    }
+
+    // does kernel group H read `what` from memory?
+    bool group_reads(RegionPlan& rp, const Group& H, Node* what) {
+        auto& reads = rp.reads;
+        std::vector<Node*> rs = H.members;
+        for (Node* sd : H.side) rs.push_back(sd);
+        for (Node* ep : H.epi) rs.push_back(ep);
+        for (Node* m : rs)
+            if (reads[m].count(what)) return true;
+        for (auto& cs : H.colsums) {
+            std::map<Node*, bool> er;
+            if (in_mem(cs.first)) er[cs.first] = true;
+            else collect_reads(cs.first, er);
+            if (er.count(what)) return true;
+        }
+        return false;
+    }
+
+    // The element-wise group that can run as the epilogue of group g, whose result P has n_elems elements: the
+    // first later group that reads P, provided it is element-wise over n_elems, reads P element for element only,
+    // and may be moved up to g's position: everything else it reads exists before g runs, and no group in between
+    // reads the old contents of a buffer it overwrites in place.  -1 if there is none.
+    int find_epilogue(RegionPlan& rp, size_t g, Node* P, int64_t n_elems) {
+        auto& reads = rp.reads;
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        const auto& home_of = rp.home_of;
+        auto reads_node = [&](const Group& H, Node* what) { return group_reads(rp, H, what); };
+        for (size_t ge = g + 1; ge < groups.size(); ++ge) {
+            Group& E = groups[ge];
+            if (E.dead) continue;
+            if (!reads_node(E, P)) continue;
+            if (E.kind != Group::ELW || !E.colsums.empty() || E.n != n_elems) return -1;
+            for (Node* m : E.members) {
+                auto it = reads[m].find(P);
+                if (it != reads[m].end() && !it->second) return -1;
+                for (auto& rd : reads[m]) {
+                    if (rd.first == P) continue;
+                    auto gi = group_of.find(rd.first);
+                    if (gi != group_of.end() && gi->second >= (int)g && gi->second != (int)ge) return -1;
+                }
+                auto ho = home_of.find(m);
+                if (ho == home_of.end()) continue;
+                auto li = livein.find(ho->second);
+                if (li == livein.end()) continue;
+                for (size_t h = g + 1; h < ge; ++h)
+                    if (!groups[h].dead && reads_node(groups[h], li->second)) return -1;
+            }
+            return (int)ge;
+        }
+        return -1;
+    }
+
+    // ---- 5b. column sums ride along with the element-wise pass that computes their operand
+    void attach_column_sums(RegionPlan& rp) {
+        auto& reads = rp.reads;
+        auto& folded_in = rp.folded_in;
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        for (size_t gs = 0; gs < groups.size(); ++gs) {
+            if (groups[gs].kind != Group::SUM) continue;
+            Node* S = groups[gs].members[0];
+            int64_t R = 0, C = 0;
+            Node* E = colsum_source(S, R, C);
+            if (!E) continue;
+            int target = -1;
+            for (size_t g = 0; g < groups.size() && target < 0; ++g) {
+                Group& G = groups[g];
+                if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
+                if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
+                for (Node* m : G.members)
+                    if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
+            }
+            if (target < 0) {
+                // no pass computes E itself; one that already loads, element for element, everything E is made
+                // of can still produce the sum without reading anything more (x.sum(0) next to dx = f(x))
+                std::map<Node*, bool> er;
+                if (in_mem(E)) er[E] = true;
+                else collect_reads(E, er);
+                bool ident = !er.empty();
+                for (auto& kv : er) ident = ident && kv.second;
+                for (size_t g = 0; ident && g < groups.size() && target < 0; ++g) {
                     Group& G = groups[g];
                     if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
                     if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
-                    for (Node* m : G.members)
-                        if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
-                }
-                if (target < 0) {
-                    // no pass computes E itself; one that already loads, element for element, everything E is made
-                    // of can still produce the sum without reading anything more (x.sum(0) next to dx = f(x))
-                    std::map<Node*, bool> er;
-                    if (in_mem(E)) er[E] = true;
-                    else collect_reads(E, er);
-                    bool ident = !er.empty();
-                    for (auto& kv : er) ident = ident && kv.second;
-                    for (size_t g = 0; ident && g < groups.size() && target < 0; ++g) {
-                        Group& G = groups[g];
-                        if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
-                        if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
-                        bool all = true;
-                        for (auto& kv : er) {
-                            bool found = false;
-                            for (Node* m : G.members) {
-                                auto it = reads[m].find(kv.first);
-                                if (it != reads[m].end() && it->second) { found = true; break; }
-                            }
-                            all = all && found;
+                    bool all = true;
+                    for (auto& kv : er) {
+                        bool found = false;
+                        for (Node* m : G.members) {
+                            auto it = reads[m].find(kv.first);
+                            if (it != reads[m].end() && it->second) { found = true; break; }
                         }
-                        if (all) target = (int)g;
+                        all = all && found;
                     }
+                    if (all) target = (int)g;
                 }
-                if (target < 0) continue;
-                // everything that reads S must run after the pass that now produces it
-                bool ok = true;
-                for (size_t g = 0; g < groups.size(); ++g) {
-                    if (groups[g].dead) continue;
-                    for (Node* m : groups[g].members)
-                        if (reads[m].count(S) && (int)g <= target) ok = false;
+            }
+            if (target < 0) continue;
+            // everything that reads S must run after the pass that now produces it
+            bool ok = true;
+            for (size_t g = 0; g < groups.size(); ++g) {
+                if (groups[g].dead) continue;
+                for (Node* m : groups[g].members)
+                    if (reads[m].count(S) && (int)g <= target) ok = false;
+            }
+            if (!ok) continue;
+            groups[target].colsums.push_back({E, S});
+            groups[target].cs_rows = R;
+            groups[target].cs_cols = C;
+            groups[gs].dead = true;
+            group_of[S] = target;
+        }
+    }
+
+    // ---- 5c. a row sum over an element-wise value produced by the kernel just before it: the
+    // reduction computes, stores and sums that value in one pass
+    void attach_row_sum_operands(RegionPlan& rp) {
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        for (size_t gs = 1; gs < groups.size(); ++gs) {
+            Group& GS = groups[gs];
+            if (GS.dead || GS.kind != Group::SUM) continue;
+            Node* S = GS.members[0];
+            const TRef& t = S->in[0];
+            if (!t.single_full() || t.pieces[0].src.kind != Src::NODE) continue;
+            Node* E = t.pieces[0].src.node;
+            if (!E->root || !op_is_elw(E->op) || E->transpose || !identity_piece(t.pieces[0], t)) continue;
+            if (numel(E->shape) != numel(t.shape) || t.shape[1] % 4 != 0 || t.shape[1] < 256) continue;
+            int ge = group_of[E];
+            int prev = (int)gs - 1;
+            while (prev >= 0 && groups[prev].dead) --prev;
+            if (ge != prev) continue;
+            Group& GE = groups[ge];
+            if (GE.kind != Group::ELW || GE.members.size() != 1 || !GE.colsums.empty()) continue;
+            GS.side.push_back(E);
+            GE.dead = true;
+            group_of[E] = (int)gs;
+        }
+    }
+
+    // ---- 5c'. a dense transposed copy that a single element-wise kernel reads is not made at all when that kernel
+    // can fetch the operand's tiles through LDS itself (gen_elw_kernel then answers with its tiled form): the
+    // copy's round trip through memory -- twice the operand's size -- goes away
+    void fold_transposed_copies(RegionPlan& rp) {
+        auto& wanted_nodes = rp.wanted_nodes;
+        auto& reads = rp.reads;
+        auto& folded_in = rp.folded_in;
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        for (size_t tg = 0; tg < groups.size(); ++tg) {
+            Group& TG = groups[tg];
+            if (TG.dead || TG.kind != Group::TRANSPOSE) continue;
+            Node* T = TG.members[0];
+            if (wanted_nodes.count(T) || T->force_root) continue;  // has to be in memory for its own sake
+            int consumer = -1;
+            bool fusable = true;
+            for (size_t g = 0; g < groups.size() && fusable; ++g) {
+                if (groups[g].dead || g == tg) continue;
+                bool rd = false;
+                for (Node* m : groups[g].members) rd = rd || reads[m].count(T);
+                for (Node* sd : groups[g].side) rd = rd || reads[sd].count(T);
+                for (auto& cs : groups[g].colsums) {
+                    std::map<Node*, bool> er;
+                    if (in_mem(cs.first)) er[cs.first] = true;
+                    else collect_reads(cs.first, er);
+                    if (er.count(T)) fusable = false;
                 }
-                if (!ok) continue;
-                groups[target].colsums.push_back({E, S});
-                groups[target].cs_rows = R;
-                groups[target].cs_cols = C;
-                groups[gs].dead = true;
-                group_of[S] = target;
+                if (!rd) continue;
+                if (consumer >= 0 || groups[g].kind != Group::ELW || !groups[g].colsums.empty() || !groups[g].side.empty() || g < tg) fusable = false;
+                consumer = (int)g;
+            }
+            if (!fusable || consumer < 0) continue;
+            Group& G = groups[consumer];
+            T->root = false;
+            std::map<Node*, std::map<Node*, bool>> saved_reads;
+            std::map<Node*, std::set<Node*>> saved_folded;
+            for (Node* m : G.members) {
+                saved_reads[m] = reads[m];
+                saved_folded[m] = folded_in[m];
+                reads[m].clear();
+                folded_in[m].clear();
+                collect_reads(m, reads[m], &folded_in[m]);
+            }
+            ElwKernelSpec probe_spec;
+            probe_spec.outputs = G.members;
+            probe_spec.name = "probe";
+            bool tiled = false;
+            try {
+                tiled = gen_elw_kernel(probe_spec, std::set<const Node*>(G.members.begin(), G.members.end())).kind == "elw_tiled";
+            } catch (const Error&) {
+                tiled = false;
+            }
+            if (tiled) {
+                TG.dead = true;
+                group_of.erase(T);  // T is no kernel's product any more: its consumer computes it in place
+            } else {
+                T->root = true;
+                for (Node* m : G.members) { reads[m] = saved_reads[m]; folded_in[m] = saved_folded[m]; }
             }
         }
-        // ---- 5c. a row sum over an element-wise value produced by the kernel just before it: the
-        // reduction computes, stores and sums that value in one pass
-        if (opt.fuse) {
-            for (size_t gs = 1; gs < groups.size(); ++gs) {
-                Group& GS = groups[gs];
-                if (GS.dead || GS.kind != Group::SUM) continue;
-                Node* S = GS.members[0];
-                const TRef& t = S->in[0];
-                if (!t.single_full() || t.pieces[0].src.kind != Src::NODE) continue;
-                Node* E = t.pieces[0].src.node;
-                if (!E->root || !op_is_elw(E->op) || E->transpose || !identity_piece(t.pieces[0], t)) continue;
-                if (numel(E->shape) != numel(t.shape) || t.shape[1] % 4 != 0 || t.shape[1] < 256) continue;
-                int ge = group_of[E];
-                int prev = (int)gs - 1;
-                while (prev >= 0 && groups[prev].dead) --prev;
-                if (ge != prev) continue;
-                Group& GE = groups[ge];
-                if (GE.kind != Group::ELW || GE.members.size() != 1 || !GE.colsums.empty()) continue;
-                GS.side.push_back(E);
-                GE.dead = true;
-                group_of[E] = (int)gs;
-            }
-        }
-        // ---- 5c'. a dense transposed copy that a single element-wise kernel reads is not made at all when that kernel
-        // can fetch the operand's tiles through LDS itself (gen_elw_kernel then answers with its tiled form): the
-        // copy's round trip through memory -- twice the operand's size -- goes away
-        if (opt.fuse) {
-            for (size_t tg = 0; tg < groups.size(); ++tg) {
-                Group& TG = groups[tg];
-                if (TG.dead || TG.kind != Group::TRANSPOSE) continue;
-                Node* T = TG.members[0];
-                if (wanted_nodes.count(T) || T->force_root) continue;  // has to be in memory for its own sake
-                int consumer = -1;
-                bool fusable = true;
-                for (size_t g = 0; g < groups.size() && fusable; ++g) {
-                    if (groups[g].dead || g == tg) continue;
-                    bool rd = false;
-                    for (Node* m : groups[g].members) rd = rd || reads[m].count(T);
-                    for (Node* sd : groups[g].side) rd = rd || reads[sd].count(T);
-                    for (auto& cs : groups[g].colsums) {
-                        std::map<Node*, bool> er;
-                        if (in_mem(cs.first)) er[cs.first] = true;
-                        else collect_reads(cs.first, er);
-                        if (er.count(T)) fusable = false;
-                    }
-                    if (!rd) continue;
-                    if (consumer >= 0 || groups[g].kind != Group::ELW || !groups[g].colsums.empty() || !groups[g].side.empty() || g < tg) fusable = false;
-                    consumer = (int)g;
-                }
-                if (!fusable || consumer < 0) continue;
-                Group& G = groups[consumer];
-                T->root = false;
-                std::map<Node*, std::map<Node*, bool>> saved_reads;
-                std::map<Node*, std::set<Node*>> saved_folded;
-                for (Node* m : G.members) {
-                    saved_reads[m] = reads[m];
-                    saved_folded[m] = folded_in[m];
-                    reads[m].clear();
-                    folded_in[m].clear();
-                    collect_reads(m, reads[m], &folded_in[m]);
-                }
-                ElwKernelSpec probe_spec;
-                probe_spec.outputs = G.members;
-                probe_spec.name = "probe";
-                bool tiled = false;
-                try {
-                    tiled = gen_elw_kernel(probe_spec, std::set<const Node*>(G.members.begin(), G.members.end())).kind == "elw_tiled";
-                } catch (const Error&) {
-                    tiled = false;
-                }
-                if (tiled) {
-                    TG.dead = true;
-                    group_of.erase(T);  // T is no kernel's product any more: its consumer computes it in place
-                } else {
-                    T->root = true;
-                    for (Node* m : G.members) { reads[m] = saved_reads[m]; folded_in[m] = saved_folded[m]; }
-                }
-            }
-        }
-        std::map<Node*, std::string> home_of_early;
-        for (auto& w : wanted) home_of_early[w.second] = w.first;
-        auto reads_node = [&](const Group& H, Node* what) {
-            std::vector<Node*> rs = H.members;
-            for (Node* sd : H.side) rs.push_back(sd);
-            for (Node* ep : H.epi) rs.push_back(ep);
-            for (Node* m : rs)
-                if (reads[m].count(what)) return true;
-            for (auto& cs : H.colsums) {
-                std::map<Node*, bool> er;
-                if (in_mem(cs.first)) er[cs.first] = true;
-                else collect_reads(cs.first, er);
-                if (er.count(what)) return true;
-            }
-            return false;
+    }
+
+    // ---- 5d. matrix-core products of one shape that each fill only part of the chip and do not depend on one
+    // another (the per-head projections, scores and weighted values of multi-head attention, and their
+    // gradients) become one grouped launch.  Products are independent when they sit at the same depth, counted
+    // in products along the longest chain of dependencies; ordering the kernels by that depth, products last
+    // within a depth, puts everything such a set reads before all of it and everything that reads it after.
+    // Dependencies are the values a kernel reads plus, for a kernel that overwrites an id's buffer, the earlier
+    // kernels that still read the id's old contents.  Regions without such a set keep program order.
+    void group_independent_products(RegionPlan& rp) {
+        auto& groups = rp.groups;
+        // a product that fills the chip by itself gives up an epilogue only for nothing: it stays out of grouped
+        // launches when an element-wise consumer could run on its accumulators
+        auto keeps_epilogue = [&](int g) {
+            Node* D = groups[g].members[0];
+            const int64_t M = D->shape[0], N = D->shape[1];
+            if (((M + 127) / 128) * ((N + 127) / 128) < 256) return false;
+            return find_epilogue(rp, (size_t)g, D, numel(D->shape)) >= 0;
         };
-        // ---- 5d. matrix-core products of one shape that each fill only part of the chip and do not depend on one
-        // another (the per-head projections, scores and weighted values of multi-head attention, and their
-        // gradients) become one grouped launch.  Products are independent when they sit at the same depth, counted
-        // in products along the longest chain of dependencies; ordering the kernels by that depth, products last
-        // within a depth, puts everything such a set reads before all of it and everything that reads it after.
-        // Dependencies are the values a kernel reads plus, for a kernel that overwrites an id's buffer, the earlier
-        // kernels that still read the id's old contents.  Regions without such a set keep program order.
-        // ---- 6. generate code per group (no buffers needed yet)
-        struct GK {
-            GeneratedKernel k;
-            std::vector<GeneratedKernel> extra;
-            std::vector<Node*> extra_nodes;
-            DotEpilogueCode dot_epi;   // DOT groups with an epilogue
-            bool dot_store = true;     // ... and whether the product itself is still written
-        };
-        std::vector<GK> gks(groups.size());
-        // reads per group, with "identity only" flags, for hazard analysis
-        std::vector<std::map<Node*, bool>> greads(groups.size());
-        // The element-wise group that can run as the epilogue of group g, whose result P has n_elems elements: the
-        // first later group that reads P, provided it is element-wise over n_elems, reads P element for element only,
-        // and may be moved up to g's position: everything else it reads exists before g runs, and no group in between
-        // reads the old contents of a buffer it overwrites in place.  -1 if there is none.
-        auto find_epilogue = [&](size_t g, Node* P, int64_t n_elems) -> int {
-            for (size_t ge = g + 1; ge < groups.size(); ++ge) {
-                Group& E = groups[ge];
-                if (E.dead) continue;
-                if (!reads_node(E, P)) continue;
-                if (E.kind != Group::ELW || !E.colsums.empty() || E.n != n_elems) return -1;
-                for (Node* m : E.members) {
-                    auto it = reads[m].find(P);
-                    if (it != reads[m].end() && !it->second) return -1;
-                    for (auto& rd : reads[m]) {
-                        if (rd.first == P) continue;
-                        auto gi = group_of.find(rd.first);
-                        if (gi != group_of.end() && gi->second >= (int)g && gi->second != (int)ge) return -1;
-                    }
-                    auto ho = home_of_early.find(m);
-                    if (ho == home_of_early.end()) continue;
-                    auto li = livein.find(ho->second);
-                    if (li == livein.end()) continue;
-                    for (size_t h = g + 1; h < ge; ++h)
-                        if (!groups[h].dead && reads_node(groups[h], li->second)) return -1;
-                }
-                return (int)ge;
-            }
-            return -1;
-        };
-        if (opt.fuse && opt.group_dots) {
-            // a product that fills the chip by itself gives up an epilogue only for nothing: it stays out of grouped
-            // launches when an element-wise consumer could run on its accumulators
-            auto keeps_epilogue = [&](int g) {
-                Node* D = groups[g].members[0];
-                const int64_t M = D->shape[0], N = D->shape[1];
-                if (((M + 127) / 128) * ((N + 127) / 128) < 256) return false;
-                return find_epilogue((size_t)g, D, numel(D->shape)) >= 0;
-            };
-            group_products(groups, group_of, reads, home_of_early, reads_node, keeps_epilogue);
-            gks.resize(groups.size());  // dead groups were dropped if the region was reordered
-            greads.resize(groups.size());
-        }
+        group_products(groups, rp.group_of, rp.reads, rp.home_of, [&](const Group& H, Node* what) { return group_reads(rp, H, what); }, keeps_epilogue);
+
+    }
+
+    // ---- 6. generate code per group (no buffers needed yet)
+    void generate_kernels(RegionPlan& rp) {
+        auto& reads = rp.reads;
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        auto& gks = rp.gks;
+        auto& greads = rp.greads;
+        const auto& home_of = rp.home_of;
+        gks.assign(groups.size(), GroupKernels());
+        greads.assign(groups.size(), {});
         for (size_t g = 0; g < groups.size(); ++g) {
             Group& G = groups[g];
             if (G.dead) continue;
@@ -1625,7 +1684,7 @@ struct Lowerer {
                 DotLaunchPlan dpl;
                 const bool grouped = G.members.size() > 1;  // one launch for all of them: whole k, no epilogue
                 if (dot_uses_mfma(D) && !grouped) dpl = plan_dot(D);
-                int nx = (grouped || dpl.splits > 1 || !opt.fuse || !dot_uses_mfma(D)) ? -1 : find_epilogue(g, D, numel(D->shape));
+                int nx = (grouped || dpl.splits > 1 || !opt.fuse || !dot_uses_mfma(D)) ? -1 : find_epilogue(rp, g, D, numel(D->shape));
                 if (nx >= 0) {
                     // an epilogue streams its other operands in the accumulator layout (32 floats of a row per half
                     // wave); with many of them (a sum over all heads' gradients) a separate element-wise pass, with
@@ -1665,7 +1724,7 @@ struct Lowerer {
                             }
                         }
                         // is the product itself still needed in memory?
-                        bool needed = home_of_early.count(D) != 0;
+                        bool needed = home_of.count(D) != 0;
                         for (size_t g2 = 0; g2 < groups.size() && !needed; ++g2) {
                             if (groups[g2].dead || g2 == g) continue;
                             std::vector<Node*> rs = groups[g2].members;
@@ -1691,7 +1750,7 @@ struct Lowerer {
                 // the element-wise group scheduled right after this reduction, if all it needs from it is the result
                 // element for element, becomes the reduction's epilogue (the reference's Reduce + ELW fusion,
                 // src/kernel/fusion/reduce_elw.rs:12-143)
-                const int ge = opt.fuse ? find_epilogue(g, G.members[0], numel(G.members[0]->shape)) : -1;
+                const int ge = opt.fuse ? find_epilogue(rp, g, G.members[0], numel(G.members[0]->shape)) : -1;
                 if (ge >= 0) spec.epilogue_outputs = groups[ge].members;
                 gks[g].k = gen_reduce_kernel(spec);
                 ADHIP_CHECK(G.side.empty() || gks[g].k.side_done, "internal: row reduction did not take over its operand's store");
@@ -1726,119 +1785,130 @@ struct Lowerer {
                 }
             }
         }
-        // ---- 6b. groups that run the same kernels on other buffers (every attention head's softmax passes) share
-        // their launches: block layer blockIdx.z works on member z.  A follower is moved up behind its lead, which
-        // needs everything it reads to exist before the lead runs; groups that update a live id's buffer in place
-        // stay where they are.
-        if (opt.fuse && opt.layer_kernels) {
-            const size_t n_groups = groups.size();
-            auto updates_in_place = [&](const Group& H) {
-                std::vector<Node*> produced = H.members;
-                for (Node* sd : H.side) produced.push_back(sd);
-                for (Node* ep : H.epi) produced.push_back(ep);
-                for (Node* m : produced) {
-                    auto ho = home_of_early.find(m);
-                    if (ho != home_of_early.end() && livein.count(ho->second)) return true;
-                }
-                return false;
+    }
+
+    // ---- 6b. groups that run the same kernels on other buffers (every attention head's softmax passes) share
+    // their launches: block layer blockIdx.z works on member z.  A follower is moved up behind its lead, which
+    // needs everything it reads to exist before the lead runs; groups that update a live id's buffer in place
+    // stay where they are.
+    void share_launches(RegionPlan& rp) {
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        auto& gks = rp.gks;
+        auto& greads = rp.greads;
+        const auto& home_of = rp.home_of;
+        const size_t n_groups = groups.size();
+        auto updates_in_place = [&](const Group& H) {
+            std::vector<Node*> produced = H.members;
+            for (Node* sd : H.side) produced.push_back(sd);
+            for (Node* ep : H.epi) produced.push_back(ep);
+            for (Node* m : produced) {
+                auto ho = home_of.find(m);
+                if (ho != home_of.end() && livein.count(ho->second)) return true;
+            }
+            return false;
+        };
+        std::map<std::vector<int64_t>, std::vector<size_t>> by_signature;
+        for (size_t g = 0; g < n_groups; ++g) {
+            Group& H = groups[g];
+            if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM) || !H.colsums.empty() || updates_in_place(H)) continue;
+            std::vector<int64_t> sig;
+            bool ok = true;
+            auto add = [&](const GeneratedKernel& k) {
+                if (k.source.find("blockIdx.z") != std::string::npos || !k.int_args.empty()) ok = false;
+                sig.push_back(add_kernel(k.entry, k.source, k.kind));
+                for (int d = 0; d < 3; ++d) { sig.push_back(k.grid[d]); sig.push_back(k.block[d]); }
+                sig.push_back(k.lds_bytes);
+                sig.push_back((int64_t)k.buffer_args.size());
+                sig.push_back(k.chunks);
             };
-            std::map<std::vector<int64_t>, std::vector<size_t>> by_signature;
-            for (size_t g = 0; g < n_groups; ++g) {
-                Group& H = groups[g];
-                if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM) || !H.colsums.empty() || updates_in_place(H)) continue;
-                std::vector<int64_t> sig;
-                bool ok = true;
-                auto add = [&](const GeneratedKernel& k) {
-                    if (k.source.find("blockIdx.z") != std::string::npos || !k.int_args.empty()) ok = false;
-                    sig.push_back(add_kernel(k.entry, k.source, k.kind));
-                    for (int d = 0; d < 3; ++d) { sig.push_back(k.grid[d]); sig.push_back(k.block[d]); }
-                    sig.push_back(k.lds_bytes);
-                    sig.push_back((int64_t)k.buffer_args.size());
-                    sig.push_back(k.chunks);
-                };
-                add(gks[g].k);
-                for (const GeneratedKernel& e : gks[g].extra) add(e);
-                if (ok && gks[g].k.grid[2] == 1) by_signature[sig].push_back(g);
-            }
-            std::vector<std::vector<size_t>> followers(n_groups);
-            bool any = false;
-            // sets in the order of their first member, so that a set whose members read the results of another
-            // (the pass after each head's reduction) sees where those have moved to
-            std::vector<const std::pair<const std::vector<int64_t>, std::vector<size_t>>*> sets;
-            for (auto& kv : by_signature) sets.push_back(&kv);
-            std::sort(sets.begin(), sets.end(), [](auto* x, auto* y) { return x->second[0] < y->second[0]; });
-            std::vector<size_t> position(n_groups);  // the old index of the group a group will run behind (its own if it stays)
-            for (size_t g = 0; g < n_groups; ++g) position[g] = g;
-            for (auto* set : sets) {
-                auto& kv = *set;
-                if (kv.second.size() < 2) continue;
-                const size_t n_buf = (size_t)kv.first[8];
-                const size_t cap = std::max<size_t>(1, std::min<size_t>(16, 96 / std::max<size_t>(1, n_buf)));
-                std::vector<size_t> leads;
-                for (size_t f : kv.second) {
-                    bool placed = false;
-                    for (size_t h : leads) {
-                        if (followers[h].size() + 1 >= cap) continue;
-                        bool ready = true;
-                        for (auto& rd : greads[f]) {
-                            if (op_is_leaf(rd.first->op)) continue;
-                            auto it = group_of.find(rd.first);
-                            if (it != group_of.end() && position[it->second] >= h) { ready = false; break; }
-                        }
-                        if (!ready) continue;
-                        followers[h].push_back(f);
-                        position[f] = h;
-                        placed = any = true;
-                        break;
+            add(gks[g].k);
+            for (const GeneratedKernel& e : gks[g].extra) add(e);
+            if (ok && gks[g].k.grid[2] == 1) by_signature[sig].push_back(g);
+        }
+        std::vector<std::vector<size_t>> followers(n_groups);
+        bool any = false;
+        // sets in the order of their first member, so that a set whose members read the results of another
+        // (the pass after each head's reduction) sees where those have moved to
+        std::vector<const std::pair<const std::vector<int64_t>, std::vector<size_t>>*> sets;
+        for (auto& kv : by_signature) sets.push_back(&kv);
+        std::sort(sets.begin(), sets.end(), [](auto* x, auto* y) { return x->second[0] < y->second[0]; });
+        std::vector<size_t> position(n_groups);  // the old index of the group a group will run behind (its own if it stays)
+        for (size_t g = 0; g < n_groups; ++g) position[g] = g;
+        for (auto* set : sets) {
+            auto& kv = *set;
+            if (kv.second.size() < 2) continue;
+            const size_t n_buf = (size_t)kv.first[8];
+            const size_t cap = std::max<size_t>(1, std::min<size_t>(16, 96 / std::max<size_t>(1, n_buf)));
+            std::vector<size_t> leads;
+            for (size_t f : kv.second) {
+                bool placed = false;
+                for (size_t h : leads) {
+                    if (followers[h].size() + 1 >= cap) continue;
+                    bool ready = true;
+                    for (auto& rd : greads[f]) {
+                        if (op_is_leaf(rd.first->op)) continue;
+                        auto it = group_of.find(rd.first);
+                        if (it != group_of.end() && position[it->second] >= h) { ready = false; break; }
                     }
-                    if (!placed) leads.push_back(f);
+                    if (!ready) continue;
+                    followers[h].push_back(f);
+                    position[f] = h;
+                    placed = any = true;
+                    break;
                 }
-            }
-            if (any) {
-                std::vector<char> is_follower(n_groups, 0);
-                for (auto& fs : followers)
-                    for (size_t f : fs) is_follower[f] = 1;
-                std::vector<int> new_index(n_groups, -1);
-                std::vector<Group> sorted;
-                std::vector<GK> sorted_gks;
-                std::vector<std::map<Node*, bool>> sorted_reads;
-                auto take = [&](size_t g, int lead) {
-                    new_index[g] = (int)sorted.size();
-                    sorted.push_back(std::move(groups[g]));
-                    sorted.back().lead = lead;
-                    sorted_gks.push_back(std::move(gks[g]));
-                    sorted_reads.push_back(std::move(greads[g]));
-                };
-                for (size_t g = 0; g < n_groups; ++g) {
-                    if (is_follower[g]) continue;
-                    take(g, -1);
-                    const int lead = new_index[g];
-                    for (size_t f : followers[g]) take(f, lead);
-                }
-                for (auto& kv : group_of) kv.second = new_index[kv.second];
-                groups.swap(sorted);
-                gks.swap(sorted_gks);
-                greads.swap(sorted_reads);
+                if (!placed) leads.push_back(f);
             }
         }
+        if (any) {
+            std::vector<char> is_follower(n_groups, 0);
+            for (auto& fs : followers)
+                for (size_t f : fs) is_follower[f] = 1;
+            std::vector<int> new_index(n_groups, -1);
+            std::vector<Group> sorted;
+            std::vector<GroupKernels> sorted_gks;
+            std::vector<std::map<Node*, bool>> sorted_reads;
+            auto take = [&](size_t g, int lead) {
+                new_index[g] = (int)sorted.size();
+                sorted.push_back(std::move(groups[g]));
+                sorted.back().lead = lead;
+                sorted_gks.push_back(std::move(gks[g]));
+                sorted_reads.push_back(std::move(greads[g]));
+            };
+            for (size_t g = 0; g < n_groups; ++g) {
+                if (is_follower[g]) continue;
+                take(g, -1);
+                const int lead = new_index[g];
+                for (size_t f : followers[g]) take(f, lead);
+            }
+            for (auto& kv : group_of) kv.second = new_index[kv.second];
+            groups.swap(sorted);
+            gks.swap(sorted_gks);
+            greads.swap(sorted_reads);
+        }
+    }
+
+    // ---- 7. buffers: homes, temporaries, in-place hazards
+    void assign_buffers(RegionPlan& rp) {
+        auto& groups = rp.groups;
+        auto& gks = rp.gks;
+        auto& greads = rp.greads;
+        auto& set_end = rp.set_end;
+        auto& commits = rp.commits;
+        const auto& home_of = rp.home_of;
         // the last group of the shared launches a group runs in (itself if it runs alone)
-        std::vector<int> set_end(groups.size());
+        set_end.assign(groups.size(), 0);
         for (size_t g = 0; g < groups.size(); ++g) {
             set_end[g] = (int)g;
             const int lead = groups[g].lead;
             if (lead >= 0)
                 for (int q = lead; q <= (int)g; ++q) set_end[q] = (int)g;
         }
-        // ---- 7. buffers: homes, temporaries, in-place hazards
-        std::map<Node*, std::string> home_of;
-        for (auto& w : wanted) home_of[w.second] = w.first;
         std::vector<int> last_use(arena.size() + 16, -1);
         std::map<Node*, int> last_reader;
         for (size_t g = 0; g < groups.size(); ++g)
             if (!groups[g].dead)
                 for (auto& rd : greads[g]) last_reader[rd.first] = (int)g;
-        struct Commit { int dst, src; int64_t n; std::string id; };
-        std::vector<Commit> commits;
         std::vector<std::vector<Node*>> free_after(groups.size());
         std::vector<int> scratch_to_free;
         for (size_t g = 0; g < groups.size(); ++g) {
@@ -1903,7 +1973,13 @@ struct Lowerer {
             scratch_to_free.clear();
             for (Node* f : free_after[g]) free_temp(f->buffer);
         }
-        // ---- 8. launches
+    }
+
+    // ---- 8. launches
+    void emit_launches(RegionPlan& rp, std::vector<Step>& out) {
+        auto& groups = rp.groups;
+        auto& gks = rp.gks;
+        auto& commits = rp.commits;
         auto buf_arg = [&](Node* n) {
             ADHIP_CHECK(n->buffer >= 0, "internal: node %d (%s, %s) has no buffer", n->id, n->name.c_str(), op_name(n->op));
             Arg a;
@@ -2032,7 +2108,6 @@ struct Lowerer {
         }
         for (auto& c : commits) emit_copy(out, c.dst, c.src, c.n, "commit_" + c.id);
         for (auto& c : commits) free_temp(c.src);
-        end_region(wanted);
     }
 
     void emit_transpose(Node* n, std::vector<Step>& out) {
@@ -2096,7 +2171,7 @@ struct Lowerer {
 
     template <class ReadsNode, class KeepsEpilogue>
     void group_products(std::vector<Group>& groups, std::map<Node*, int>& group_of, std::map<Node*, std::map<Node*, bool>>& reads,
-                        const std::map<Node*, std::string>& home_of_early, ReadsNode&& reads_node, KeepsEpilogue&& keeps_epilogue) {
+                        const std::map<Node*, std::string>& home_of, ReadsNode&& reads_node, KeepsEpilogue&& keeps_epilogue) {
         const int G = (int)groups.size();
         std::vector<std::array<int64_t, 8>> key(G);
         std::vector<char> cand(G, 0);
@@ -2148,8 +2223,8 @@ struct Lowerer {
             }
             if (!ok) return;  // not in dependency order as it stands: leave the region alone
             for (Node* m : produced) {
-                auto ho = home_of_early.find(m);
-                if (ho == home_of_early.end()) continue;
+                auto ho = home_of.find(m);
+                if (ho == home_of.end()) continue;
                 auto li = livein.find(ho->second);
                 if (li == livein.end()) continue;
                 for (int r = 0; r < g; ++r)
