@@ -26,8 +26,13 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 # copy kernel of known size (the summaries under profiles/ give the runs).  These counters sit in front of the 256 MiB
 # last-level cache, so they bound HBM traffic from above.  Valid for the full-size workloads only.
 TRAFFIC_BYTES = {
-    "fused_elw": {"elw_colsum": None},
-    "reductions": {"reduce_row": None, "elw_colsum": None},
+    # 2 x 393277.1 KiB fetched + 1081886.5 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
+    "fused_elw": {"elw_colsum": int((2 * 393277.1 + 1081886.5) * 1024)},
+    # row sums: 2 x 131086.5 KiB fetched + 512 KiB written; backward pass with x.sum(0) riding along: 2 x 131352.5 KiB
+    # fetched + 278528.3 KiB written (dx and the [1024][4096] partial column sums)
+    "reductions": {"reduce_row": int((2 * 131086.5 + 512.0) * 1024), "elw_colsum": int((2 * 131352.5 + 278528.3) * 1024)},
+    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73756.4 KiB fetched + 294912.0 KiB written
+    "manip_loop": {"gather_stage": int((2 * 73756.4 + 294912.0) * 1024)},
 }
 
 
@@ -195,12 +200,13 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "attention"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "manip", "attention"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by; "
                          "'streammix': only a bare 3-reads + 4-writes kernel over 8192x8192 f32 (the stream mix of the "
                          "headline pass with trivial arithmetic and no column sums: what the memory system gives that mix); "
-                         "'reductions': only configs[2]; 'mlp': only configs[3]")
+                         "'reductions': only configs[2]; 'mlp': only configs[3]; 'manip': only configs[4] (one run: its "
+                         "loop consumes its counter); 'attention': only multi-head attention forward")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the device path is single-device (run with --gpus 1)", file=sys.stderr)
@@ -251,6 +257,15 @@ def main():
         ms3 = timed_runs(p3, args.steps, args.warmup)
         print(json.dumps({"metric": "reductions forward + backward, f32 [16384,4096]", "value": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
                           "unit": "GB/s", "ms_per_step": ms3, "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}))
+        return
+    if args.workload == "manip":
+        wl5 = W.manip_loop(dev)
+        p5 = compile_resident(dev, wl5)
+        t0 = time.perf_counter()
+        p5.run()
+        ms5 = (time.perf_counter() - t0) * 1e3
+        print(json.dumps({"metric": "tensor manipulation + data-dependent loop, one run", "value": ms5, "unit": "ms",
+                          "kernels": profile_once(p5)}))
         return
     if args.workload == "attention":
         print(json.dumps(dict(measure_attention(dev), metric="multi-head attention forward, fp32")))
@@ -322,8 +337,9 @@ def main():
             k["GBps"] = k["bytes"] / (k["avg_ms"] * 1e-3) / 1e9
             k["memory"] = "LLC-resident" if k["launches"] > 1 else "HBM"
         extra["manip_loop"] = {"ms_total": ms5, "kernels": k5,
-                               "gather_stage": {"algorithmic_bytes": 301989888 + 150994944, "note": "p and q regions read, r and the kept "
-                                                "copy of the gathered tensor written",
+                               "gather_stage": {"algorithmic_bytes": 150994944 + 301989888, "note": "the gathered regions of p and q read "
+                                                "once (151 MB), r and the kept copy of the gathered tensor written (151 MB each)",
+                                                "traffic": TRAFFIC_BYTES["manip_loop"]["gather_stage"],
                                                 "moved_bytes": sum(k["bytes"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce")),
                                                 "ms": sum(k["avg_ms"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce"))}}
         p5.close()
