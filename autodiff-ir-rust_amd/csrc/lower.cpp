@@ -1042,7 +1042,9 @@ struct Lowerer {
         if (n->in[1].shape[0] != k.d || n->in[2].shape[0] != k.sk) return false;
         if (k.d % 4 != 0 || k.d < 4 || k.d > 256 || k.dv % 16 != 0 || k.dv < 16 || k.dv > 256 || k.sq < 1 || k.sk < 1) return false;
         if ((q.s1 != 1 && k.d > 1) || kt.s0 != 1 || v.s1 != 1) return false;
-        if (kt.offset % 4 || kt.s1 % 4 || v.offset % 4 || v.s0 % 4) return false;
+        if (q.offset % 4 || q.s0 % 4 || kt.offset % 4 || kt.s1 % 4 || v.offset % 4 || v.s0 % 4) return false;
+        // a thread's position inside a tile of 64 rows is a 32-bit offset
+        if (q.s0 >= (int64_t(1) << 24) || kt.s1 >= (int64_t(1) << 24) || v.s0 >= (int64_t(1) << 24)) return false;
         k.q_ld = q.s0;
         k.k_ld = kt.s1;
         k.v_ld = v.s0;
@@ -2394,15 +2396,20 @@ struct Lowerer {
         cfg.d = (int)key0.d;
         cfg.dv = (int)key0.dv;
         const int64_t row_blocks = (key0.sq + 63) / 64;
-        // 64 keys per step while that leaves room in LDS and the launch is too small for several blocks per CU anyway;
-        // 32 keys per step otherwise (half the LDS, two to three blocks per CU)
-        cfg.bn = (cfg.d <= 128 && cfg.dv <= 128 && row_blocks * cnt < 512) ? 64 : 32;
-        const std::string entry = strf("adhip_attention_d%d_v%d_k%d", cfg.d, cfg.dv, cfg.bn);
+        // A launch with two or more blocks per CU runs blocks of four wavefronts on tiles of 32 keys, two of which fit
+        // a CU's LDS while the heads are not too wide; a smaller launch splits every tile between two groups of four
+        // wavefronts instead, so that a SIMD still has two wavefronts to switch between.  Tiles of 64 keys where two
+        // stages of them fit in LDS.
+        const bool narrow = cfg.d + cfg.dv <= 256;
+        if (row_blocks * cnt >= 512 && narrow) { cfg.bn = 32; cfg.wg = 1; }
+        else { cfg.bn = narrow ? 64 : 32; cfg.wg = 2; }
+        ADHIP_CHECK(attention_lds_bytes(cfg) <= 160 * 1024, "internal: attention tiles of %d keys do not fit in LDS", cfg.bn);
+        const std::string entry = strf("adhip_attention_d%d_v%d_k%d_w%d", cfg.d, cfg.dv, cfg.bn, cfg.wg);
         Launch l;
         l.kernel = add_kernel(entry, attention_kernel_source(cfg, entry), "attention");
-        l.block[0] = 256;
-        l.grid[0] = (unsigned)row_blocks;
-        l.grid[1] = (unsigned)cnt;
+        l.block[0] = 256u * (unsigned)cfg.wg;
+        ADHIP_CHECK(row_blocks * cnt <= 0x7fffffff, "internal: attention grid too large");
+        l.grid[0] = (unsigned)(row_blocks * cnt);
         auto B = [&](Node* x, int64_t off) {
             Arg a;
             a.kind = Arg::BUF;
@@ -2427,6 +2434,7 @@ struct Lowerer {
         sc.kind = Arg::F32;
         sc.fv = key0.scale;
         l.args.push_back(sc);
+        for (int64_t v : {row_blocks, (int64_t)cnt}) { Arg a; a.kind = Arg::I32; a.iv = v; l.args.push_back(a); }
         l.label = strf("attention_%s_%dx_%lldx%lldx%lldx%lld", atts[0]->name.c_str(), cnt, (long long)key0.sq, (long long)key0.sk,
                        (long long)key0.d, (long long)key0.dv);
         l.bytes = 4.0 * cnt * ((double)key0.sq * key0.d + (double)key0.sk * key0.d + (double)key0.sk * key0.dv + (double)key0.sq * key0.dv);

@@ -171,7 +171,9 @@ def _attention_program(dev, sq, sk, d, dv, d_model, seed, spread=1.0, mask=False
 _FUSED_SHAPES = [
     # sq, sk, d, dv: one query block and many, ragged in both directions, narrow and wide heads, sq != sk, d != dv
     (64, 64, 16, 16), (100, 100, 48, 48), (1, 7, 4, 16), (65, 129, 8, 32), (300, 77, 64, 64), (257, 640, 128, 128),
-    (130, 1000, 36, 80), (96, 200, 256, 256), (200, 96, 20, 240),
+    (130, 1000, 36, 80), (96, 200, 256, 256), (200, 96, 20, 240), (33, 31, 16, 16), (64, 33, 64, 48), (2100, 40, 32, 32),
+    # 512 row blocks and more: the variant with blocks of four wavefronts
+    (33000, 40, 16, 16), (32768, 70, 20, 32),
 ]
 
 
@@ -193,6 +195,10 @@ def test_attention_lowers_to_one_kernel(sq, sk, d, dv):
     launches = [l for l in lower_describe(dev.proc, dev.deps).splitlines() if l.lstrip().startswith("launch")]
     assert len(launches) == 1 and "[attention]" in launches[0], launches
     assert f"adhip_attention_d{d}_v{dv}_k" in launches[0]
+    # the kernel of this head width compiles for gfx950 (both score layouts: d % 16 == 0 and not; narrow and wide tiles)
+    from test_library_cpu import _compile_check
+    rc, msg = _compile_check(dev.proc, dev.deps)
+    assert rc == 0, msg
 
 
 @pytest.mark.parametrize("what", ["mask", "scores_kept", "head_of_6", "plain_exp"])
@@ -299,7 +305,7 @@ def test_fused_attention_survives_extreme_scores(hip_device):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("seq,d_model,heads", [(100, 96, 2), (128, 64, 4), (320, 512, 2)])
+@pytest.mark.parametrize("seq,d_model,heads", [(100, 96, 2), (128, 64, 4), (320, 512, 2), (2112, 512, 16)])
 def test_attention_forward_workload_fused_equals_unfused(seq, d_model, heads, hip_device, monkeypatch):
     """Multi-head attention end to end (projections, fused attention of all heads in one launch, concatenation, output
     projection) against the same program lowered without the fusion, and against the oracle."""
@@ -308,10 +314,11 @@ def test_attention_forward_workload_fused_equals_unfused(seq, d_model, heads, hi
     monkeypatch.setenv("ADHIP_FUSE_ATTENTION", "0")
     plain = W.attention_forward(hip_device, seq, d_model, heads, seed=seq).run()["y"]
     monkeypatch.delenv("ADHIP_FUSE_ATTENTION")
-    ref = W.attention_forward(OracleDevice(), seq, d_model, heads, seed=seq).run()["y"]
     tol = 4 * RED_RTOL * math.sqrt(max(seq, d_model))
     assert_close(fused.data, plain.data, tol, "fused vs unfused")
-    assert_close(fused.data, ref.data, tol, "fused vs oracle")
+    if seq <= 512:  # the oracle's one-thread-per-output products take too long beyond
+        ref = W.attention_forward(OracleDevice(), seq, d_model, heads, seed=seq).run()["y"]
+        assert_close(fused.data, ref.data, tol, "fused vs oracle")
 
 
 @pytest.mark.gpu
