@@ -749,3 +749,46 @@ def test_tiled_kernels_with_operands_read_against_the_grain(case, hip_device):
     got = _run_ir(hip_device, cmds, ["y"])
     assert got["y"].dim == list(want.shape)
     assert_exact(got["y"].data, want.reshape(-1), "y")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["flat_ragged", "broadcast_3d", "two_outputs_in_place", "whole_bands"])
+def test_large_flat_kernels_in_banded_order(case, hip_device):
+    """Element-wise kernels of a million float4 and more hand their blocks out band by band instead of front to
+    back (16 wavefronts of a block on 16 rows of 32 KiB).  Every element must still be computed exactly once: sizes
+    that are no multiple of a band, an index that is decomposed into three coordinates after the reordering, an
+    in-place update next to a second output.  Bit-exact against numpy (one exactly rounded operation per element)."""
+    print(f"[case] banded element-wise kernel: {case}", flush=True)
+    from adhip import ir as IR
+    rng = np.random.default_rng(len(case))
+    f = lambda *sh: rng.standard_normal(sh, dtype=np.float32)  # noqa: E731
+    if case == "flat_ragged":
+        a, b = f(1025, 4100), f(1025, 4100)
+        cmds = [IR.CreateMat(a.reshape(-1), [1025, 4100], "a"), IR.CreateMat(b.reshape(-1), [1025, 4100], "b"),
+                IR.ElwAdd(a="a", b="b", res="y")]
+        want = {"y": a + b}
+    elif case == "broadcast_3d":
+        a, r, c = f(37, 300, 512), f(37, 1, 512), f(300, 1)
+        cmds = [IR.CreateMat(a.reshape(-1), [37, 300, 512], "a"), IR.CreateMat(r.reshape(-1), [37, 1, 512], "r"),
+                IR.CreateMat(c.reshape(-1), [300, 1], "c"),
+                IR.Broadcast(a="r", dim=1, r=300, res="rb"), IR.Broadcast(a="c", dim=1, r=512, res="cb1"),
+                IR.View(a="cb1", target_dim=[1, 300, 512], res="cb2"), IR.Broadcast(a="cb2", dim=0, r=37, res="cb"),
+                IR.ElwMultiply(a="a", b="rb", res="m"), IR.ElwAdd(a="m", b="cb", res="y")]
+        want = {"y": a * r + c.reshape(1, 300, 1)}
+    elif case == "two_outputs_in_place":
+        a, b = f(3000, 1400), f(3000, 1400)
+        cmds = [IR.CreateMat(a.reshape(-1), [3000, 1400], "a"), IR.CreateMat(b.reshape(-1), [3000, 1400], "b"),
+                IR.ElwMultiply(a="a", b="b", res="p"), IR.ElwAddEq(s="a", o="b")]
+        want = {"p": a * b, "a": a + b}
+    else:
+        a = f(2048, 2048)
+        cmds = [IR.CreateMat(a.reshape(-1), [2048, 2048], "a"), IR.ElwMultiply(a="a", b="a", res="y")]
+        want = {"y": a * a}
+    proc = IR.IRProcedure("main", cmds + [IR.EX()])
+    from adhip.device import lower_describe
+    plan = lower_describe(proc, set(want))
+    assert "block=1024" in plan, plan
+    got = _run_ir(hip_device, cmds, sorted(want))
+    for k, w in want.items():
+        assert got[k].dim == list(w.shape), k
+        assert_exact(got[k].data, w.reshape(-1), k)
