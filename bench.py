@@ -26,13 +26,13 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 # copy kernel of known size (the summaries under profiles/ give the runs).  These counters sit in front of the 256 MiB
 # last-level cache, so they bound HBM traffic from above.  Valid for the full-size workloads only.
 TRAFFIC_BYTES = {
-    # 2 x 393277.1 KiB fetched + 1081886.5 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
-    "fused_elw": {"elw_colsum": int((2 * 393277.1 + 1081886.5) * 1024)},
+    # 2 x 393277.1 KiB fetched + 1081909.2 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
+    "fused_elw": {"elw_colsum": int((2 * 393277.1 + 1081909.2) * 1024)},
     # row sums: 2 x 131086.5 KiB fetched + 512 KiB written; backward pass with x.sum(0) riding along: 2 x 131352.5 KiB
     # fetched + 278528.3 KiB written (dx and the [1024][4096] partial column sums)
     "reductions": {"reduce_row": int((2 * 131086.5 + 512.0) * 1024), "elw_colsum": int((2 * 131352.5 + 278528.3) * 1024)},
-    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73756.4 KiB fetched + 294912.0 KiB written
-    "manip_loop": {"gather_stage": int((2 * 73756.4 + 294912.0) * 1024)},
+    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73756.9 KiB fetched + 294912.0 KiB written
+    "manip_loop": {"gather_stage": int((2 * 73756.9 + 294912.0) * 1024)},
 }
 
 
