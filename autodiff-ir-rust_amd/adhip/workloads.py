@@ -135,14 +135,14 @@ def reductions(dev, rows: int = 16384, cols: int = 4096, seed: int = 0, backward
     n = rows * cols
     small = 4.0 * (rows + cols + 1)
     unfused = 3 * 4.0 * n + small           # three reductions, x read once by each
-    fused = 4.0 * n + small                 # forward alone: one pass over x yields all three (s2 is the sum of s0)
+    fused = 4.0 * n + small                 # one pass over x yields all three sums (s2 is the sum of s0)
     if backward:
         s0.backward()
         s1.backward()
         s2.backward()
         outs["dx"] = x.grad()
         unfused += 2 * 4.0 * n              # read x, write dx
-        fused += 2 * 4.0 * n                # as lowered: a second pass reads x and writes dx (x.sum(0) rides along with it)
+        fused += 4.0 * n                    # as lowered: the one pass over x also writes dx (row and column sums ride along)
     return Workload("reductions", outs, {"x": xn}, algorithmic_bytes=fused, unfused_bytes=unfused)
 
 

@@ -632,6 +632,7 @@ struct ElwBody {
     Gen g;
     std::vector<std::string> out_exprs;
     std::vector<std::string> cs_exprs;
+    std::vector<std::string> rs_exprs;
     std::vector<int> dim_atoms;
     Shape iter_shape;
 };
@@ -669,6 +670,10 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
         Val v = g.gen_node(cs.value, lin, "");
         b.cs_exprs.push_back(v.expr);
     }
+    for (auto& rs : spec.rowsums) {
+        Val v = g.gen_node(rs.value, lin, "");
+        b.rs_exprs.push_back(v.expr);
+    }
     return b;
 }
 
@@ -677,6 +682,8 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
 // Rows one block of the column-sum layout covers: 16 (one per wavefront), times the number of rows each wavefront
 // walks, which is 1 until the partial sums would exceed 1024 rows.
 static int64_t elw_colsum_rows_per_wave(int64_t rows) { return std::max<int64_t>(1, (rows + 16 * 1024 - 1) / (16 * 1024)); }
+
+int64_t elw_rowsum_runs(int64_t cols) { return (cols / 4 + 63) / 64; }
 
 int64_t elw_colsum_tiles(int64_t rows, int64_t cols) {
     (void)cols;
@@ -698,7 +705,9 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     for (Node* o : spec.outputs) ADHIP_CHECK(numel(o->shape) == N, "internal: fused outputs differ in size");
     std::vector<Node*> all = spec.outputs;
     for (auto& cs : spec.colsums) all.push_back(cs.value);
+    for (auto& rs : spec.rowsums) all.push_back(rs.value);
     const bool wide = needs_wide(all);
+    const int64_t runs = elw_rowsum_runs(C);
     ElwBody b = elw_body(spec, members, Shape{R, C}, 4, wide);
     Gen& g = b.g;
     const int64_t K = elw_colsum_rows_per_wave(R);
@@ -711,6 +720,7 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     // no __restrict__: an output may share its buffer with an input it replaces in place
     for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* o%zu", i); order.push_back(spec.outputs[i]); }
     for (size_t i = 0; i < spec.colsums.size(); ++i) { sig += strf(", float* q%zu", i); order.push_back(spec.colsums[i].partial); }
+    for (size_t i = 0; i < spec.rowsums.size(); ++i) { sig += strf(", float* r%zu", i); order.push_back(spec.rowsums[i].partial); }
     for (auto& gb : g.bufs) { sig += strf(", const float* %s", gb.param.c_str()); order.push_back(gb.node); }
     const char* it = g.idx_t();
     const char* sfx = wide ? "ull" : "u";
@@ -718,7 +728,7 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     std::string src = kernel_prelude();
     src += strf("extern \"C\" __global__ __launch_bounds__(1024) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
     src += "    if (guard && *guard == 0) return;\n";
-    src += "    __shared__ float4_t part[2][16][64];\n";
+    if (!spec.colsums.empty()) src += "    __shared__ float4_t part[2][16][64];\n";
     src += "    const unsigned lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;\n";
     src += strf("    const %s c1 = (%s)blockIdx.x * 64u + lane;\n", it, it);
     src += strf("    const bool col_ok = c1 < %lld%s;\n", (long long)(C / 4), sfx);
@@ -726,6 +736,7 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     if (K == 1) src += strf("    {\n        const %s c0 = (%s)blockIdx.y * 16u + wv;\n", it, it);
     else src += strf("#pragma unroll 1\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n",
                      (long long)K, it, it, (long long)(16 * K), sfx);
+    for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("        float rs%zu = 0.f;\n", i);
     src += strf("        if (col_ok && c0 < %lld%s) {\n", (long long)R, sfx);
     src += join(g.codeA, "            ");
     for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            float w%zu[4];\n", i);
@@ -733,10 +744,17 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     src += join(g.codeB, "                ");
     for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("                w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
     for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("                cs%zu[j] += %s;\n", i, b.cs_exprs[i].c_str());
+    for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("                rs%zu += %s;\n", i, b.rs_exprs[i].c_str());
     src += "            }\n";
     for (size_t i = 0; i < spec.outputs.size(); ++i)
         src += "            " + store4_stmt(strf("w%zu", i), strf("o%zu + (c0 * %lld%s + c1 * 4u)", i, (long long)C, sfx), nt_out) + "\n";
-    src += "        }\n    }\n";
+    src += "        }\n";
+    // a wavefront's run of a row: lanes outside the columns hold 0; one value per (row, run)
+    for (size_t i = 0; i < spec.rowsums.size(); ++i) {
+        src += strf("        rs%zu = wave_sum(rs%zu);\n", i, i);
+        src += strf("        if (lane == 0u && c0 < %lld%s) r%zu[c0 * %lld%s + blockIdx.x] = rs%zu;\n", (long long)R, sfx, i, (long long)runs, sfx, i);
+    }
+    src += "    }\n";
     // the 16 wavefronts' sums, added in wavefront order; two sums per round through LDS (wavefronts 0 and 1 add them)
     for (size_t i0 = 0; i0 < spec.colsums.size(); i0 += 2) {
         const size_t cnt = std::min<size_t>(2, spec.colsums.size() - i0);
@@ -756,9 +774,10 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     k.grid[0] = (unsigned)((C / 4 + 63) / 64);
     k.grid[1] = (unsigned)tiles;
     k.chunks = tiles;
-    k.bytes = 4.0 * (double)N * (double)spec.outputs.size() + 4.0 * (double)tiles * C * spec.colsums.size();
+    k.bytes = 4.0 * (double)N * (double)spec.outputs.size() + 4.0 * (double)tiles * C * spec.colsums.size() +
+              4.0 * (double)R * (double)runs * spec.rowsums.size();
     for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), N);
-    k.flops = (g.flops + spec.colsums.size()) * (double)N;
+    k.flops = (g.flops + spec.colsums.size() + spec.rowsums.size()) * (double)N;
     return k;
 }
 
@@ -871,7 +890,7 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
 }
 
 GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members) {
-    if (!spec.colsums.empty()) return gen_elw_colsum_kernel(spec, members);
+    if (!spec.colsums.empty() || !spec.rowsums.empty()) return gen_elw_colsum_kernel(spec, members);
     ADHIP_CHECK(!spec.outputs.empty(), "internal: element-wise kernel without outputs");
     const int64_t N = numel(spec.outputs[0]->shape);
     for (Node* o : spec.outputs) ADHIP_CHECK(numel(o->shape) == N, "internal: fused outputs differ in size");

@@ -32,8 +32,15 @@ struct ElwKernelSpec {
     // with rows*cols elements) to a [tiles][cols] buffer (`partial`).  The caller adds the partials.
     struct ColSum { Node* value; Node* partial; };
     std::vector<ColSum> colsums;
+    // Row sums produced by the same pass: a wavefront adds up `value` over its run of a row (256 columns) and writes the
+    // result to `partial`, a [rows][ceil(cols / 256)] buffer.  The caller adds the runs of a row.
+    struct RowSum { Node* value; Node* partial; };
+    std::vector<RowSum> rowsums;
     int64_t rows = 0, cols = 0;
 };
+
+// number of 256-column runs a row of the column-/row-sum layout is cut into
+int64_t elw_rowsum_runs(int64_t cols);
 
 struct ReduceKernelSpec {
     Node* node = nullptr;  // Op::SUM, operand [V,R]

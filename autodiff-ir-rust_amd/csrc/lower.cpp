@@ -246,12 +246,22 @@ struct Group {
     enum Kind { ELW, SUM, DOT, TRANSPOSE, ATTN } kind = ELW;
     // column sums computed by this element-wise kernel: (value node, SUM node that wanted it)
     std::vector<std::pair<Node*, Node*>> colsums;
-    int64_t cs_rows = 0, cs_cols = 0;
+    // row sums computed by this element-wise kernel, likewise: every wavefront adds up its run of a row, the runs of a
+    // row are added by a second pass
+    std::vector<std::pair<Node*, Node*>> rowsums;
+    int64_t cs_rows = 0, cs_cols = 0;  // the [rows, cols] view of the iteration space both kinds of sums refer to
+    bool rides() const { return !colsums.empty() || !rowsums.empty(); }
+    std::vector<std::pair<Node*, Node*>> riders() const {
+        std::vector<std::pair<Node*, Node*>> r = colsums;
+        r.insert(r.end(), rowsums.begin(), rowsums.end());
+        return r;
+    }
     // element-wise values a row reduction stores while it sums them
     std::vector<Node*> side;
     // element-wise values of the result's size that the reduction evaluates and stores right after summing
     std::vector<Node*> epi;
     bool dead = false;  // its only member was absorbed by another group
+    bool tiled = false; // fetches an operand read against the grain through LDS tiles (takes no sums along)
     int lead = -1;      // >= 0: runs inside the launches of that group (same kernels on other buffers), which it follows directly
 };
 
@@ -817,6 +827,20 @@ struct Lowerer {
         return a.base;
     }
 
+    // The element-wise (or in-memory) value E with rows*cols elements whose rows the reduction `s` adds up, if `s` is
+    // such a plain row sum over a space large enough for the 2-D element-wise layout.
+    static Node* rowsum_source(const Node* s, int64_t& rows, int64_t& cols) {
+        if (s->op != Op::SUM) return nullptr;
+        Affine2D a;
+        if (!tref_affine2d(s->in[0], a)) return nullptr;
+        const int64_t V = s->in[0].shape[0], R = s->in[0].shape[1];
+        if (!(op_is_elw(a.base->op) || in_mem(a.base)) || a.offset != 0 || a.s0 != R || a.s1 != 1) return nullptr;
+        if (numel(a.base->shape) != V * R || R % 4 != 0 || R < 256 || V < 16 || V * R < (int64_t(1) << 16)) return nullptr;
+        rows = V;
+        cols = R;
+        return a.base;
+    }
+
     // True when, below the reduction `sum` over a [V,R] space, every read of `old` (V values) is the broadcast
     // (v, r) -> old[v] reached through element-for-element references only.
     static bool reads_at_kept_coordinate_only(Node* sum, Node* old, int64_t V, int64_t R) {
@@ -1133,6 +1157,10 @@ struct Lowerer {
         std::vector<Node*> extra_nodes;
         DotEpilogueCode dot_epi;   // DOT groups with an epilogue
         bool dot_store = true;     // ... and whether the product itself is still written
+        // row sums riding along with an element-wise group: per sum the [rows][runs] partial buffer, the node that
+        // stands for the second pass over it, and that pass's kernel
+        std::vector<Node*> row_partials, row_fins;
+        std::vector<GeneratedKernel> row_kernels;
     };
     struct Commit { int dst, src; int64_t n; std::string id; };
     struct RegionPlan {
@@ -1178,6 +1206,7 @@ struct Lowerer {
             attach_column_sums(rp);
             attach_row_sum_operands(rp);
             fold_transposed_copies(rp);
+            attach_row_sums(rp);
             if (opt.group_dots) group_independent_products(rp);
         }
         generate_kernels(rp);
@@ -1422,7 +1451,7 @@ struct Lowerer {
         for (Node* ep : H.epi) rs.push_back(ep);
         for (Node* m : rs)
             if (reads[m].count(what)) return true;
-        for (auto& cs : H.colsums) {
+        for (auto& cs : H.riders()) {
             std::map<Node*, bool> er;
             if (in_mem(cs.first)) er[cs.first] = true;
             else collect_reads(cs.first, er);
@@ -1445,7 +1474,7 @@ struct Lowerer {
             Group& E = groups[ge];
             if (E.dead) continue;
             if (!reads_node(E, P)) continue;
-            if (E.kind != Group::ELW || !E.colsums.empty() || E.n != n_elems) return -1;
+            if (E.kind != Group::ELW || E.rides() || E.n != n_elems) return -1;
             for (Node* m : E.members) {
                 auto it = reads[m].find(P);
                 if (it != reads[m].end() && !it->second) return -1;
@@ -1482,7 +1511,7 @@ struct Lowerer {
             for (size_t g = 0; g < groups.size() && target < 0; ++g) {
                 Group& G = groups[g];
                 if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
-                if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
+                if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                 for (Node* m : G.members)
                     if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
             }
@@ -1497,7 +1526,7 @@ struct Lowerer {
                 for (size_t g = 0; ident && g < groups.size() && target < 0; ++g) {
                     Group& G = groups[g];
                     if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
-                    if (!G.colsums.empty() && (G.cs_rows != R || G.cs_cols != C)) continue;
+                    if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                     bool all = true;
                     for (auto& kv : er) {
                         bool found = false;
@@ -1527,6 +1556,112 @@ struct Lowerer {
         }
     }
 
+    // ---- 5b'. row sums ride along too: a plain row sum over an element-wise value E of [rows, cols] is produced by an
+    // element-wise pass over the same space that computes E anyway or already loads, element for element, everything
+    // E is made of (s = (x*x).sum(1) next to dx = f(x): x is read once for both).  Every wavefront of the 2-D layout
+    // adds up its run of a row; a second pass adds a row's runs.  When the pass comes later in the program than the
+    // sum did, it is moved up to the sum's place, which needs everything it reads to exist there already and nobody in
+    // between to read the old contents of a buffer it overwrites.
+    void attach_row_sums(RegionPlan& rp) {
+        auto& reads = rp.reads;
+        auto& folded_in = rp.folded_in;
+        auto& groups = rp.groups;
+        auto& group_of = rp.group_of;
+        for (size_t gs = 0; gs < groups.size(); ++gs) {
+            if (groups[gs].dead || groups[gs].kind != Group::SUM || groups[gs].members.size() != 1 || !groups[gs].side.empty()) continue;
+            Node* S = groups[gs].members[0];
+            int64_t R = 0, C = 0;
+            Node* E = rowsum_source(S, R, C);
+            if (!E) continue;
+            std::map<Node*, bool> er;
+            if (in_mem(E)) er[E] = true;
+            else collect_reads(E, er);
+            bool ident = !er.empty();
+            for (auto& kv : er) ident = ident && kv.second;
+            int target = -1;
+            for (size_t g = 0; g < groups.size() && target < 0; ++g) {
+                Group& G = groups[g];
+                if (g == gs || G.dead || G.tiled || G.kind != Group::ELW || G.n != R * C || !G.side.empty()) continue;
+                if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
+                bool computes = false;
+                for (Node* m : G.members) computes = computes || m == E || folded_in[m].count(E);
+                bool loads_all = ident;
+                for (auto& kv : er) {
+                    if (!loads_all) break;
+                    bool found = false;
+                    for (Node* m : G.members) {
+                        auto it = reads[m].find(kv.first);
+                        if (it != reads[m].end() && it->second) { found = true; break; }
+                    }
+                    loads_all = found;
+                }
+                if (!computes && !loads_all) continue;
+                // the pass must not need the sum itself, directly or through what it reads
+                bool independent = true;
+                for (Node* m : G.members) independent = independent && !reads[m].count(S);
+                for (auto& cs : G.riders()) {
+                    std::map<Node*, bool> cr;
+                    if (in_mem(cs.first)) cr[cs.first] = true;
+                    else collect_reads(cs.first, cr);
+                    independent = independent && !cr.count(S);
+                }
+                if (!independent) continue;
+                if (g > gs) {
+                    // moving the pass up to the sum's place
+                    bool movable = true;
+                    auto early_enough = [&](const std::map<Node*, bool>& rd) {
+                        for (auto& kv : rd) {
+                            if (op_is_leaf(kv.first->op)) continue;
+                            auto it = group_of.find(kv.first);
+                            if (it != group_of.end() && it->second >= (int)gs && it->second != (int)g) movable = false;
+                        }
+                    };
+                    std::vector<Node*> produced = G.members;
+                    for (Node* m : G.members) early_enough(reads[m]);
+                    for (auto& cs : G.riders()) {
+                        std::map<Node*, bool> cr;
+                        if (in_mem(cs.first)) cr[cs.first] = true;
+                        else collect_reads(cs.first, cr);
+                        early_enough(cr);
+                        produced.push_back(cs.second);
+                    }
+                    for (Node* m : produced) {
+                        auto ho = rp.home_of.find(m);
+                        if (ho == rp.home_of.end()) continue;
+                        auto li = livein.find(ho->second);
+                        if (li == livein.end()) continue;
+                        for (size_t h = gs; h < g; ++h)
+                            if (!groups[h].dead && group_reads(rp, groups[h], li->second)) movable = false;
+                    }
+                    // whatever reads a result of the pass keeps coming after it; whatever the pass overwrites in place
+                    // was checked above
+                    if (!movable) continue;
+                }
+                target = (int)g;
+            }
+            if (target < 0) continue;
+            if (target > (int)gs) {
+                // everything that reads S runs after gs already; the pass takes the place right after the (now dead) sum
+                Group moved = std::move(groups[(size_t)target]);
+                groups.erase(groups.begin() + target);
+                groups.insert(groups.begin() + (std::ptrdiff_t)gs + 1, std::move(moved));
+                for (auto& kv : group_of) {
+                    if (kv.second == target) kv.second = (int)gs + 1;
+                    else if (kv.second > (int)gs && kv.second < target) kv.second += 1;
+                }
+                target = (int)gs + 1;
+            } else {
+                // the sum is produced earlier than it was: its readers all come after gs, hence after the pass
+            }
+            Group& G = groups[(size_t)target];
+            G.rowsums.push_back({E, S});
+            G.cs_rows = R;
+            G.cs_cols = C;
+            groups[gs].dead = true;
+            group_of[S] = target;
+        }
+    }
+
     // ---- 5c. a row sum over an element-wise value produced by the kernel just before it: the
     // reduction computes, stores and sums that value in one pass
     void attach_row_sum_operands(RegionPlan& rp) {
@@ -1546,7 +1681,7 @@ struct Lowerer {
             while (prev >= 0 && groups[prev].dead) --prev;
             if (ge != prev) continue;
             Group& GE = groups[ge];
-            if (GE.kind != Group::ELW || GE.members.size() != 1 || !GE.colsums.empty()) continue;
+            if (GE.kind != Group::ELW || GE.members.size() != 1 || GE.rides()) continue;
             GS.side.push_back(E);
             GE.dead = true;
             group_of[E] = (int)gs;
@@ -1574,14 +1709,14 @@ struct Lowerer {
                 bool rd = false;
                 for (Node* m : groups[g].members) rd = rd || reads[m].count(T);
                 for (Node* sd : groups[g].side) rd = rd || reads[sd].count(T);
-                for (auto& cs : groups[g].colsums) {
+                for (auto& cs : groups[g].riders()) {
                     std::map<Node*, bool> er;
                     if (in_mem(cs.first)) er[cs.first] = true;
                     else collect_reads(cs.first, er);
                     if (er.count(T)) fusable = false;
                 }
                 if (!rd) continue;
-                if (consumer >= 0 || groups[g].kind != Group::ELW || !groups[g].colsums.empty() || !groups[g].side.empty() || g < tg) fusable = false;
+                if (consumer >= 0 || groups[g].kind != Group::ELW || groups[g].rides() || !groups[g].side.empty() || g < tg) fusable = false;
                 consumer = (int)g;
             }
             if (!fusable || consumer < 0) continue;
@@ -1606,6 +1741,7 @@ struct Lowerer {
                 tiled = false;
             }
             if (tiled) {
+                G.tiled = true;
                 TG.dead = true;
                 group_of.erase(T);  // T is no kernel's product any more: its consumer computes it in place
             } else {
@@ -1676,6 +1812,22 @@ struct Lowerer {
                     spec.colsums.push_back({cs.first, partial});
                     gks[g].extra_nodes.push_back(partial);
                 }
+                for (auto& rs : G.rowsums) {
+                    // one partial sum per (row, run of 256 columns), added by a generated row reduction over [rows][runs]
+                    const int64_t runs = elw_rowsum_runs(G.cs_cols);
+                    Node* S = rs.second;
+                    Node* partial = new_node(Op::COPY, Shape{G.cs_rows, runs}, {}, S->name + ".runs", 0.f, false);
+                    partial->root = true;
+                    Node* fin = new_node(Op::SUM, Shape{G.cs_rows}, {tr_node(partial, Shape{G.cs_rows, runs})}, S->name, 0.f, false);
+                    fin->root = true;
+                    spec.rowsums.push_back({rs.first, partial});
+                    ReduceKernelSpec s2;
+                    s2.node = fin;
+                    s2.name = name + strf("_rs%zu", gks[g].row_fins.size());
+                    gks[g].row_kernels.push_back(gen_reduce_kernel(s2, 1));
+                    gks[g].row_partials.push_back(partial);
+                    gks[g].row_fins.push_back(fin);
+                }
                 gks[g].k = gen_elw_kernel(spec, members);
             } else if (G.kind == Group::DOT) {
                 // the element-wise group scheduled right after a matrix-core product, if all it needs from the
@@ -1734,7 +1886,7 @@ struct Lowerer {
                             for (Node* ep : groups[g2].epi) rs.push_back(ep);
                             for (Node* m : rs)
                                 if (reads[m].count(D)) needed = true;
-                            for (auto& cs : groups[g2].colsums) {
+                            for (auto& cs : groups[g2].riders()) {
                                 std::map<Node*, bool> er;
                                 if (in_mem(cs.first)) er[cs.first] = true;
                                 else collect_reads(cs.first, er);
@@ -1813,7 +1965,7 @@ struct Lowerer {
         std::map<std::vector<int64_t>, std::vector<size_t>> by_signature;
         for (size_t g = 0; g < n_groups; ++g) {
             Group& H = groups[g];
-            if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM) || !H.colsums.empty() || updates_in_place(H)) continue;
+            if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM) || H.rides() || updates_in_place(H)) continue;
             std::vector<int64_t> sig;
             bool ok = true;
             auto add = [&](const GeneratedKernel& k) {
@@ -1916,7 +2068,7 @@ struct Lowerer {
         for (size_t g = 0; g < groups.size(); ++g) {
             if (groups[g].dead) continue;
             std::vector<Node*> produced = groups[g].members;
-            for (auto& cs : groups[g].colsums) produced.push_back(cs.second);
+            for (auto& cs : groups[g].riders()) produced.push_back(cs.second);
             for (Node* sd : groups[g].side) produced.push_back(sd);
             for (Node* ep : groups[g].epi) produced.push_back(ep);
             if (groups[g].kind == Group::DOT && !gks[g].dot_store) produced.erase(produced.begin());  // lives in registers only
@@ -1970,6 +2122,10 @@ struct Lowerer {
             }
             for (Node* e : gks[g].extra_nodes)
                 if (e->op == Op::COPY) scratch_to_free.push_back(e->buffer);
+            for (Node* e : gks[g].row_partials) {
+                e->buffer = alloc_temp(numel(e->shape), e->name);
+                scratch_to_free.push_back(e->buffer);
+            }
             if (set_end[g] != (int)g) continue;
             for (int b : scratch_to_free) free_temp(b);
             scratch_to_free.clear();
@@ -2055,8 +2211,12 @@ struct Lowerer {
                 continue;
             }
             GeneratedKernel& k = gks[g].k;
-            if (G.kind == Group::ELW && !G.colsums.empty()) {
+            if (G.kind == Group::ELW && G.rides()) {
                 launch_generated(k);
+                for (size_t i = 0; i < G.rowsums.size(); ++i) {
+                    gks[g].row_fins[i]->buffer = G.rowsums[i].second->buffer;
+                    launch_generated(gks[g].row_kernels[i]);
+                }
                 // one launch of the fixed second-pass kernel per four sums
                 if (fixed_finalize < 0) fixed_finalize = add_kernel("adhip_colsum_finalize", fixed_kernels_source(), "colsum_finalize");
                 const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
@@ -2216,7 +2376,7 @@ struct Lowerer {
             std::vector<Node*> produced = H.members;
             for (Node* sd : H.side) produced.push_back(sd);
             for (Node* m : produced) add_reads(reads[m]);
-            for (auto& cs : H.colsums) {
+            for (auto& cs : H.riders()) {
                 std::map<Node*, bool> er;
                 if (in_mem(cs.first)) er[cs.first] = true;
                 else collect_reads(cs.first, er);

@@ -51,7 +51,7 @@ def test_fused_elw_small(rows, cols, hip_device):
     compare_outputs(got, ref, rules, ("close", 4 * ELW_RTOL))
 
 
-@pytest.mark.parametrize("rows,cols", [(128, 64), (100, 36), (1024, 512), (5, 3), (3, 2048), (2048, 3)])
+@pytest.mark.parametrize("rows,cols", [(128, 64), (100, 36), (1024, 512), (5, 3), (3, 2048), (2048, 3), (300, 260), (77, 1028)])
 def test_reductions_small(rows, cols, hip_device):
     print(f"[case] reductions {rows}x{cols}", flush=True)
     got, ref = _both(lambda d: W.reductions(d, rows, cols, seed=2), hip_device)
@@ -792,3 +792,64 @@ def test_large_flat_kernels_in_banded_order(case, hip_device):
     for k, w in want.items():
         assert got[k].dim == list(w.shape), k
         assert_exact(got[k].data, w.reshape(-1), k)
+
+
+def _row_rider_program(case, rng):
+    from adhip import ir as IR
+    f = lambda *sh: rng.standard_normal(sh, dtype=np.float32)  # noqa: E731
+    R, C = (520, 384) if case != "ragged" else (77, 1028)
+    x = f(R, C)
+    cmds = [IR.CreateMat(x.reshape(-1), [R, C], "x"), IR.CreateConstant(2.0, "two", [R, C]), IR.CreateConstant(1.0, "one", [R, C])]
+    x64 = x.astype(np.float64)
+    if case in ("independent_later", "ragged"):
+        # the sum comes first in the program, the pass that can carry it later
+        cmds += [IR.ElwMultiply(a="x", b="x", res="xx"), IR.Sum(a="xx", res="s"),
+                 IR.ElwMultiply(a="x", b="two", res="t"), IR.ElwAdd(a="t", b="one", res="y")]
+        want = {"s": (x64 * x64).sum(1), "y": 2 * x64 + 1}
+        fused = True
+    elif case == "independent_earlier":
+        cmds += [IR.ElwMultiply(a="x", b="two", res="t"), IR.ElwAdd(a="t", b="one", res="y"),
+                 IR.ElwMultiply(a="x", b="x", res="xx"), IR.Sum(a="xx", res="s")]
+        want = {"s": (x64 * x64).sum(1), "y": 2 * x64 + 1}
+        fused = True
+    elif case == "sums_of_the_pass_itself":
+        # the summed value is what the pass stores; a second row sum and a column sum ride along as well
+        cmds += [IR.ElwMultiply(a="x", b="two", res="t"), IR.ElwAdd(a="t", b="one", res="y"), IR.Sum(a="y", res="s"),
+                 IR.ElwMultiply(a="x", b="x", res="xx"), IR.Sum(a="xx", res="s2"),
+                 IR.Permute(a="x", p=[1, 0], res="xt"), IR.Sum(a="xt", res="c")]
+        want = {"s": (2 * x64 + 1).sum(1), "s2": (x64 * x64).sum(1), "c": x64.sum(0), "y": 2 * x64 + 1}
+        fused = True
+    elif case == "dependent":
+        # the pass needs the sum: y = x * s[:, None]
+        cmds += [IR.ElwMultiply(a="x", b="x", res="xx"), IR.Sum(a="xx", res="s"), IR.View(a="s", target_dim=[R, 1], res="sv"),
+                 IR.Broadcast(a="sv", dim=1, r=C, res="sb"), IR.ElwMultiply(a="x", b="sb", res="y")]
+        s_ = (x64 * x64).sum(1)
+        want = {"s": s_, "y": x64 * s_[:, None]}
+        fused = False
+    else:  # in_place_between: something between the sum and the pass reads the buffer the pass overwrites
+        cmds += [IR.ElwMultiply(a="x", b="x", res="xx"), IR.Sum(a="xx", res="s"),
+                 IR.ElwAdd(a="x", b="one", res="z"),           # reads the old x
+                 IR.ElwMultiplyEq(s="x", o="two")]             # x *= 2 in place: may not move in front of z
+        want = {"s": (x64 * x64).sum(1), "z": x64 + 1, "x": 2 * x64}
+        fused = None
+    return cmds, want, fused
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["independent_later", "independent_earlier", "sums_of_the_pass_itself", "dependent", "in_place_between", "ragged"])
+def test_row_sums_riding_with_elementwise_pass(case, hip_device):
+    """A plain row sum is produced by an element-wise pass over the same [rows, cols] space that loads its operand
+    anyway (one read of x for both), wherever the two stand in the program -- unless the pass needs the sum, or moving
+    it would overtake a reader of a buffer it overwrites.  Checked against float64."""
+    print(f"[case] row sums riding along: {case}", flush=True)
+    from adhip import ir as IR
+    from adhip.device import lower_describe
+    cmds, want, fused = _row_rider_program(case, np.random.default_rng(len(case)))
+    plan = lower_describe(IR.IRProcedure("main", cmds + [IR.EX()]), set(want))
+    if fused is not None:
+        assert ("_rs0 [reduce_row]" in plan) == fused, plan
+    got = _run_ir(hip_device, cmds, sorted(want))
+    for k, w in want.items():
+        assert got[k].dim == list(w.shape), k
+        tol = RED_RTOL * math.sqrt(1028) if k in ("s", "s2", "c") else 2 * ELW_RTOL  # sums of at most 1028 terms
+        assert_close(got[k].data, w.reshape(-1), tol, k)
