@@ -847,7 +847,7 @@ def test_row_sums_riding_with_elementwise_pass(case, hip_device):
     cmds, want, fused = _row_rider_program(case, np.random.default_rng(len(case)))
     plan = lower_describe(IR.IRProcedure("main", cmds + [IR.EX()]), set(want))
     if fused is not None:
-        assert ("_rs0 [reduce_row]" in plan) == fused, plan
+        assert ("_rs0 [" in plan) == fused, plan
     got = _run_ir(hip_device, cmds, sorted(want))
     for k, w in want.items():
         assert got[k].dim == list(w.shape), k
