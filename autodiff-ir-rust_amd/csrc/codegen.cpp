@@ -930,6 +930,11 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
         sig += ", const float* " + gb.param;
         order.push_back(gb.node);
     }
+    int latch_output = -1;
+    if (spec.latch && vec == 1 && N == 1)
+        for (size_t i = 0; i < spec.outputs.size(); ++i)
+            if (spec.outputs[i] == spec.latch) latch_output = (int)i;
+    if (latch_output >= 0) { sig += ", int* latch"; k.latch_done = true; }
     std::string src = kernel_prelude();
     // Large kernels do not walk through memory block after block.  A block is 16 wavefronts; wavefront w takes a 1 KiB
     // run (64 float4) in band row w, where a band is 16 rows of `band` bytes, and consecutive blocks take consecutive
@@ -976,6 +981,7 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
         if (vec == 4) src += "    " + store4_stmt(strf("w%zu", i), strf("o%zu + t * 4u", i), N >= nontemporal_min_elems()) + "\n";
         else src += strf("    o%zu[t] = w%zu[0];\n", i, i);
     }
+    if (latch_output >= 0) src += strf("    latch[0] = w%d[0] != 0.0f ? 1 : 0;\n", latch_output);
     src += "}\n";
     k.source = src;
     k.buffer_args = order;
@@ -1169,6 +1175,11 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         if (epi)
             for (size_t i = 0; i < spec.epilogue_outputs.size(); ++i) { sig += strf(", float* e%zu", i); order.push_back(spec.epilogue_outputs[i]); }
         for (auto& gb : g.bufs) { sig += std::string(", const float* ") + gb.param; order.push_back(gb.node); }
+        int latch_epi = -1;
+        if (epi && spec.latch && V == 1)
+            for (size_t i = 0; i < spec.epilogue_outputs.size(); ++i)
+                if (spec.epilogue_outputs[i] == spec.latch) latch_epi = (int)i;
+        if (latch_epi >= 0) { sig += ", int* latch"; k.latch_done = true; }
         src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
         src += strf("    const unsigned lane = threadIdx.x %% %du;\n", T);
@@ -1202,6 +1213,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         if (epi) {
             epilogue = join(epi_code, "        ");
             for (size_t i = 0; i < epi_exprs.size(); ++i) epilogue += strf("        e%zu[x] = %s;\n", i, epi_exprs[i].c_str());
+            if (latch_epi >= 0) epilogue += strf("        latch[0] = (%s) != 0.0f ? 1 : 0;\n", epi_exprs[(size_t)latch_epi].c_str());
         }
         if (T == 64) {
             src += strf("    s = %s(s);\n", wave_comb);

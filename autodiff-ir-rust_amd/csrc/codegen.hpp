@@ -37,6 +37,11 @@ struct ElwKernelSpec {
     struct RowSum { Node* value; Node* partial; };
     std::vector<RowSum> rowsums;
     int64_t rows = 0, cols = 0;
+    // A one-element output that is the predicate of the device-predicated loop the kernel runs in: the thread that
+    // stores it also latches `value != 0` into the loop's flag (a trailing `int* latch` parameter), which saves the
+    // one-thread kernel that would do so at the top of the next iteration.  Honoured by the plain kernel form only;
+    // `GeneratedKernel::latch_done` tells.
+    const Node* latch = nullptr;
 };
 
 // number of 256-column runs a row of the column-/row-sum layout is cut into
@@ -52,6 +57,8 @@ struct ReduceKernelSpec {
     // the lane that holds a finished sum also evaluates and stores them, so no further kernel is needed.  Done only
     // in the row layout when one pass finishes the sum; `GeneratedKernel::epilogue_done` tells.
     std::vector<Node*> epilogue_outputs;
+    // as ElwKernelSpec::latch, for a one-element epilogue output
+    const Node* latch = nullptr;
 };
 
 struct GeneratedKernel {
@@ -68,6 +75,7 @@ struct GeneratedKernel {
     int64_t chunks = 1;
     bool side_done = false;  // the reduction stored its side outputs
     bool epilogue_done = false;  // the reduction evaluated and stored its epilogue outputs
+    bool latch_done = false;     // the kernel takes a trailing `int* latch` and stores the loop flag
 };
 
 GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members);

@@ -282,6 +282,12 @@ struct Lowerer {
     int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sum_slices = -1, fixed_sum_slices_grouped = -1;
     int dot_epilogue_counter = 0;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
+    // The device-predicated loop whose body is being lowered: its block, predicate id and flag.  The last region of the
+    // block may hand the flag's upkeep to its last kernel (`latch_attached`).
+    const Proc* latch_block = nullptr;
+    std::string latch_id;
+    int latch_slot = -1;
+    bool latch_region = false, latch_attached = false;
 
     // per region
     std::vector<Node*> rnodes;
@@ -1161,6 +1167,11 @@ struct Lowerer {
         // stands for the second pass over it, and that pass's kernel
         std::vector<Node*> row_partials, row_fins;
         std::vector<GeneratedKernel> row_kernels;
+        // what the group's kernel was generated from, should it be generated again with a loop flag to latch
+        int spec_kind = 0;  // 1: elw_spec + spec_members, 2: red_spec
+        ElwKernelSpec elw_spec;
+        std::set<const Node*> spec_members;
+        ReduceKernelSpec red_spec;
     };
     struct Commit { int dst, src; int64_t n; std::string id; };
     struct RegionPlan {
@@ -1829,6 +1840,9 @@ struct Lowerer {
                     gks[g].row_fins.push_back(fin);
                 }
                 gks[g].k = gen_elw_kernel(spec, members);
+                gks[g].spec_kind = 1;
+                gks[g].elw_spec = spec;
+                gks[g].spec_members = members;
             } else if (G.kind == Group::DOT) {
                 // the element-wise group scheduled right after a matrix-core product, if all it needs from the
                 // product is the result element for element, runs on the accumulators before they are stored (the
@@ -1907,6 +1921,8 @@ struct Lowerer {
                 const int ge = opt.fuse ? find_epilogue(rp, g, G.members[0], numel(G.members[0]->shape)) : -1;
                 if (ge >= 0) spec.epilogue_outputs = groups[ge].members;
                 gks[g].k = gen_reduce_kernel(spec);
+                gks[g].spec_kind = 2;
+                gks[g].red_spec = spec;
                 ADHIP_CHECK(G.side.empty() || gks[g].k.side_done, "internal: row reduction did not take over its operand's store");
                 if (ge >= 0 && gks[g].k.epilogue_done) {
                     G.epi = groups[ge].members;
@@ -2268,8 +2284,55 @@ struct Lowerer {
             }
             g = last;
         }
+        if (latch_region && latch_slot >= 0 && commits.empty() && opt.fuse) attach_latch(rp, out);
         for (auto& c : commits) emit_copy(out, c.dst, c.src, c.n, "commit_" + c.id);
         for (auto& c : commits) free_temp(c.src);
+    }
+
+    // The region is the last one of a device-predicated loop's body.  When its last launch is the generated kernel
+    // that produces the loop's predicate (a one-element value), that kernel is generated once more with the loop flag
+    // as a trailing argument: the thread that stores the predicate also stores `predicate != 0` into the flag, for the
+    // next iteration's kernels to see.  Nothing may run after it in the iteration (it would see the new flag), which is
+    // why the region must end with it and have no commits.
+    void attach_latch(RegionPlan& rp, std::vector<Step>& out) {
+        if (out.empty() || out.back().kind != Step::LAUNCH) return;
+        Node* n = nullptr;
+        for (auto& w : rp.wanted)
+            if (w.first == latch_id) n = w.second;
+        if (!n || numel(n->shape) != 1) return;
+        auto it = rp.group_of.find(n);
+        if (it == rp.group_of.end()) return;
+        const size_t g = (size_t)it->second;
+        Group& G = rp.groups[g];
+        if (G.dead || G.lead >= 0) return;
+        for (size_t h = g + 1; h < rp.groups.size(); ++h)
+            if (!rp.groups[h].dead) return;
+        GroupKernels& gk = rp.gks[g];
+        GeneratedKernel nk;
+        if (G.kind == Group::ELW && gk.spec_kind == 1 && !G.rides() && !G.tiled) {
+            ElwKernelSpec spec = gk.elw_spec;
+            spec.latch = n;
+            spec.name += "_latch";
+            nk = gen_elw_kernel(spec, gk.spec_members);
+        } else if (G.kind == Group::SUM && gk.spec_kind == 2 && gk.k.epilogue_done && gk.k.chunks == 1) {
+            ReduceKernelSpec spec = gk.red_spec;
+            spec.latch = n;
+            spec.name += "_latch";
+            nk = gen_reduce_kernel(spec);
+        } else {
+            return;
+        }
+        Launch& l = out.back().launch;
+        if (!nk.latch_done || l.label != gk.k.entry || nk.buffer_args.size() != gk.k.buffer_args.size()) return;
+        l.kernel = add_kernel(nk.entry, nk.source, nk.kind);
+        l.label = nk.entry;
+        plan->stats[(size_t)l.stat].label = nk.entry;
+        plan->stats[(size_t)l.stat].kernel = l.kernel;
+        Arg a;
+        a.kind = Arg::FLAG;
+        a.iv = latch_slot;
+        l.args.push_back(a);
+        latch_attached = true;
     }
 
     void emit_transpose(Node* n, std::vector<Step>& out) {
@@ -2886,7 +2949,9 @@ struct Lowerer {
             const bool final_region = (j == n && &p == &prog) || (j < n && p.cmds[j].tag == T_EX);
             if (final_region)
                 for (auto& d : deps) live.insert(d);
+            latch_region = j == n && &p == latch_block;
             flush_region(live, final_region, out);
+            latch_region = false;
             if (j == n) break;
             const Cmd& c = p.cmds[j];
             if (c.tag == T_EX) {
@@ -2905,8 +2970,17 @@ struct Lowerer {
                 if (!counted && cur_guard < 0 && !has_loop_or_exit(*c.block)) {
                     s.flag_slot = plan->n_flags++;
                     cur_guard = s.flag_slot;
+                    latch_block = c.block.get();
+                    latch_id = c.a;
+                    latch_slot = s.flag_slot;
+                    latch_attached = false;
                 }
                 lower_block(*c.block, s.body, false);
+                if (s.flag_slot >= 0) {
+                    s.latch_in_body = latch_attached;
+                    latch_block = nullptr;
+                    latch_attached = false;
+                }
                 cur_guard = saved;
                 out.push_back(std::move(s));
             } else {
@@ -3002,6 +3076,7 @@ void describe_steps(const std::vector<Step>& steps, const Plan& p, int indent, s
             for (const Arg& a : l.args) {
                 if (a.kind == Arg::BUF) o += " " + p.buffers[a.buf].name + "#" + std::to_string(a.buf) + (a.off ? strf("+%lld", (long long)a.off) : std::string());
                 else if (a.kind == Arg::F32) o += strf(" %g", a.fv);
+                else if (a.kind == Arg::FLAG) o += strf(" flag%lld", (long long)a.iv);
                 else o += strf(" %lld", (long long)a.iv);
             }
             o += "\n";
@@ -3009,7 +3084,7 @@ void describe_steps(const std::vector<Step>& steps, const Plan& p, int indent, s
         }
         case Step::LOOP:
             o += pad + strf("while %s#%d != 0", p.buffers[s.cond_buf].name.c_str(), s.cond_buf);
-            if (s.flag_slot >= 0) o += strf("   [device-predicated, flag %d]", s.flag_slot);
+            if (s.flag_slot >= 0) o += strf("   [device-predicated, flag %d%s]", s.flag_slot, s.latch_in_body ? ", latched by the body's last kernel" : "");
             if (s.counter_buf >= 0) o += strf("   [counted: %s += %g; cond = (%s + %g) < 0]", p.buffers[s.counter_buf].name.c_str(), s.counter_inc, p.buffers[s.counter_buf].name.c_str(), s.counter_add);
             o += " {\n";
             describe_steps(s.body, p, indent + 1, o);

@@ -25,10 +25,10 @@ struct KernelDef {
 };
 
 struct Arg {
-    enum Kind { BUF, I32, I64, F32 } kind = I32;
+    enum Kind { BUF, I32, I64, F32, FLAG } kind = I32;
     int buf = -1;
     int64_t off = 0;  // BUF: element offset
-    int64_t iv = 0;
+    int64_t iv = 0;   // FLAG: the flag slot whose address is passed
     float fv = 0.f;
 };
 
@@ -66,6 +66,9 @@ struct Step {
     // that an earlier arm ran).  parent_guard is the flag of the enclosing predicated block or -1.
     int flag_slot = -1, parent_guard = -1, taken_slot = -1, else_slot = -1;
     std::vector<int> arm_slots;
+    // LOOP with flag_slot >= 0: the last kernel of the body, which produces the predicate, latches the flag for the
+    // next iteration itself; the one-thread kernel runs only once, before the first iteration.
+    bool latch_in_body = false;
 };
 
 struct KernelStat {

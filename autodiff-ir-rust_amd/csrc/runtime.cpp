@@ -515,6 +515,7 @@ void launch(adhip_program* p, const Launch& l) {
         case Arg::I32: { int v = (int)a.iv; memcpy(&vals[i], &v, sizeof v); break; }
         case Arg::I64: { long long v = a.iv; memcpy(&vals[i], &v, sizeof v); break; }
         case Arg::F32: { memcpy(&vals[i], &a.fv, sizeof a.fv); break; }
+        case Arg::FLAG: { int* q = cur_flags(p) + a.iv; memcpy(&vals[i], &q, sizeof q); break; }
         }
         ptrs[i + 1] = &vals[i];
     }
@@ -621,10 +622,14 @@ void exec_steps(adhip_program* p, const std::vector<Step>& steps) {
                 for (int64_t i = 0; i < n && !p->exited; ++i) exec_steps(p, s.body);
             } else if (s.flag_slot >= 0) {
                 // device-predicated: enqueue a batch of iterations, then look at the predicate once
+                // (when the body's last kernel latches the flag for the next iteration itself, the one-thread kernel
+                // that does so runs before the first iteration only)
                 int batch = 4;
+                bool first = true;
                 while (true) {
                     for (int b = 0; b < batch; ++b) {
-                        launch_flag(p, s.flag_slot, s.parent_guard, s.cond_buf, 0, -1);
+                        if (first || !s.latch_in_body) launch_flag(p, s.flag_slot, s.parent_guard, s.cond_buf, 0, -1);
+                        first = false;
                         exec_steps(p, s.body);
                     }
                     read_scalar(p, s.cond_buf, 0);
