@@ -853,3 +853,64 @@ def test_row_sums_riding_with_elementwise_pass(case, hip_device):
         assert got[k].dim == list(w.shape), k
         tol = RED_RTOL * math.sqrt(1028) if k in ("s", "s2", "c") else 2 * ELW_RTOL  # sums of at most 1028 terms
         assert_close(got[k].data, w.reshape(-1), tol, k)
+
+
+def _latch_loop_program(case, rng):
+    """x [rows, cols] shrinks by a factor per iteration until a predicate computed from it turns 0.
+    Returns (commands, ids to keep, whether the body's last kernel is expected to latch the loop flag)."""
+    from adhip import ir as IR
+    rows, cols = 40, 64
+    x = (rng.random((rows, cols), dtype=np.float32) + 1.0)          # in [1, 2)
+    top = [IR.CreateMat(x.reshape(-1), [rows, cols], "x"), IR.CreateMat(np.zeros(1, np.float32), [1], "n"),
+           IR.CreateConstant(0.5, "half", [rows, cols]), IR.CreateConstant(1.0, "one1", [1]),
+           IR.CreateConstant(-40.0, "mthr", [1])]
+
+    def predicate(prefix):
+        # cond = (sum of all elements - 40 > 0)
+        return [IR.Sum(a="x", res=prefix + "s"), IR.View(a=prefix + "s", target_dim=[1, rows], res=prefix + "sv"),
+                IR.Sum(a=prefix + "sv", res=prefix + "t"), IR.ElwAdd(a=prefix + "t", b="mthr", res=prefix + "d"),
+                IR.MoreZero(a=prefix + "d", res="cond")]
+    body = [IR.ElwMultiplyEq(s="x", o="half"), IR.ElwAddEq(s="n", o="one1")]
+    if case == "predicate_last":
+        body += predicate("b")
+        latched = True
+    elif case == "kernel_after_predicate":
+        # the counter update comes after the predicate's kernel in the iteration
+        body = [IR.ElwMultiplyEq(s="x", o="half")] + predicate("b") + [IR.Contigious(a="x", res="copy"), IR.ElwAddEq(s="n", o="one1")]
+        latched = None
+    else:  # predicate_from_elementwise: cond = (n - 5 < 0) * (n - 100 < 0), a one-element kernel of its own (the product
+        # of two comparisons keeps it from being the counted-loop shape)
+        top += [IR.CreateConstant(-5.0, "m5", [1]), IR.CreateConstant(-100.0, "m100", [1])]
+
+        def small(prefix):
+            return [IR.ElwAdd(a="n", b="m5", res=prefix + "d"), IR.LessZero(a=prefix + "d", res=prefix + "l"),
+                    IR.ElwAdd(a="n", b="m100", res=prefix + "e"), IR.LessZero(a=prefix + "e", res=prefix + "m"),
+                    IR.ElwMultiply(a=prefix + "l", b=prefix + "m", res="cond")]
+        body += small("b")
+        latched = True
+    cmds = top + (predicate("a") if case != "predicate_from_elementwise" else small("a"))
+    cmds.append(IR.While(conditional_var="cond", block=IR.IRProcedure("body", body)))
+    return cmds, ["x", "n", "cond"], latched
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["predicate_last", "kernel_after_predicate", "predicate_from_elementwise"])
+def test_loop_flag_latched_by_the_body(case, hip_device):
+    """A device-predicated loop whose body ends with the kernel that produces the predicate lets that kernel keep the
+    loop flag; a body in which something still runs after the predicate's kernel keeps the separate flag kernel.
+    Either way the loop must stop after the same iteration as on the oracle."""
+    print(f"[case] loop flag: {case}", flush=True)
+    from adhip import ir as IR
+    from adhip.device import lower_describe
+    cmds, keep, latched = _latch_loop_program(case, np.random.default_rng(3))
+    plan = lower_describe(IR.IRProcedure("main", cmds + [IR.EX()]), set(keep))
+    assert "device-predicated" in plan, plan
+    if latched is not None:
+        assert ("latched by the body's last kernel" in plan) == latched, plan
+    got = _run_ir(hip_device, cmds, keep)
+    oracle = OracleDevice()
+    ref = _run_ir(oracle, cmds, keep)
+    assert float(ref["n"].data[0]) >= 3.0   # the loop really iterates
+    for k in keep:
+        assert got[k].dim == ref[k].dim, k
+        assert_close(got[k].data, ref[k].data, 4 * ELW_RTOL, k)
