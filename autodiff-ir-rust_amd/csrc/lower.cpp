@@ -1201,6 +1201,95 @@ struct Lowerer {
     }
 
     void flush_region(const IdSet& live, bool final_region, std::vector<Step>& out) {
+        const size_t first_step = out.size();
+        flush_region_launches(live, final_region, out);
+        if (opt.fuse && opt.merge_small) merge_single_block_runs(out, first_step);
+    }
+
+    // Consecutive launches of one region that are a single block each (the kernels of a program on tiny tensors: the
+    // reference's README example is eleven of them) run as the phases of one launch instead: every kernel's translation
+    // unit goes into a namespace of its own with its entry turned into a device function, and a new entry calls them
+    // in order with a block-wide barrier in between, which is also what makes one phase's global writes visible to the
+    // next.  Only kernel kinds in which no thread leaves before a barrier the others still reach.
+    void merge_single_block_runs(std::vector<Step>& out, size_t from) {
+        static const std::set<std::string> mergeable = {"elw", "reduce_row", "reduce_row_store", "reduce_col", "dot_naive", "copy"};
+        auto single_block = [&](const Step& st) {
+            if (st.kind != Step::LAUNCH) return false;
+            const Launch& l = st.launch;
+            if (l.grid[0] != 1 || l.grid[1] != 1 || l.grid[2] != 1 || l.block[0] != 256 || l.block[1] != 1 || l.block[2] != 1 || l.lds_bytes != 0) return false;
+            return mergeable.count(plan->kernels[(size_t)l.kernel].kind) > 0;
+        };
+        for (size_t i = from; i < out.size(); ++i) {
+            if (!single_block(out[i])) continue;
+            size_t j = i, nargs = 0;
+            while (j < out.size() && single_block(out[j]) && out[j].launch.guard == out[i].launch.guard &&
+                   nargs + out[j].launch.args.size() <= 160) {
+                nargs += out[j].launch.args.size();
+                ++j;
+            }
+            if (j - i < 2) continue;
+            std::string src, calls, params = "const int* __restrict__ guard";
+            Launch merged;
+            merged.block[0] = 256;
+            merged.guard = out[i].launch.guard;
+            bool ok = true;
+            for (size_t q = i; q < j && ok; ++q) {
+                const Launch& l = out[q].launch;
+                const KernelDef& kd = plan->kernels[(size_t)l.kernel];
+                std::string body = kd.source;
+                const std::string head = "extern \"C\" __global__", bounds = "__launch_bounds__(";
+                for (size_t at = body.find(head); at != std::string::npos; at = body.find(head)) body.replace(at, head.size(), "static __device__");
+                for (size_t at = body.find(bounds); at != std::string::npos; at = body.find(bounds)) body.erase(at, body.find(')', at) + 1 - at);
+                const size_t fn = body.find(" void " + kd.entry + "(");
+                const size_t open = fn == std::string::npos ? fn : body.find('(', fn);
+                const size_t close = open == std::string::npos ? open : body.find(") {", open);
+                if (close == std::string::npos) { ok = false; break; }
+                std::string list = body.substr(open + 1, close - open - 1), args;
+                size_t pos = 0, index = 0;
+                while (pos < list.size()) {
+                    size_t comma = list.find(',', pos);
+                    if (comma == std::string::npos) comma = list.size();
+                    std::string prm = list.substr(pos, comma - pos);
+                    pos = comma + 1;
+                    while (!prm.empty() && isspace((unsigned char)prm.front())) prm.erase(prm.begin());
+                    while (!prm.empty() && isspace((unsigned char)prm.back())) prm.pop_back();
+                    if (index++ == 0) continue;  // guard
+                    const size_t sp = prm.find_last_of(" *");
+                    if (sp == std::string::npos) { ok = false; break; }
+                    const std::string name = strf("s%zu_%s", q - i, prm.substr(sp + 1).c_str());
+                    params += ", " + prm.substr(0, sp + 1) + name;
+                    args += ", " + name;
+                }
+                if (index != l.args.size() + 1) ok = false;  // the launch must pass exactly the entry's parameters
+                src += strf("namespace seg%zu {\n", q - i) + body + "\n}\n";
+                calls += strf("    seg%zu::%s(guard%s);\n", q - i, kd.entry.c_str(), args.c_str());
+                if (q + 1 < j) calls += "    __syncthreads();\n";
+                merged.args.insert(merged.args.end(), l.args.begin(), l.args.end());
+                merged.bytes += l.bytes;
+                merged.flops += l.flops;
+            }
+            if (!ok) continue;
+            const std::string entry = strf("run%d_%s_x%zu", kernel_counter++, out[i].launch.label.c_str(), j - i);
+            src += "extern \"C\" __global__ __launch_bounds__(256) void " + entry + "(" + params + ") {\n" + calls + "}\n";
+            merged.kernel = add_kernel(entry, src, "merged");
+            merged.label = entry;
+            KernelStat st;
+            st.label = entry;
+            st.kind = "merged";
+            st.kernel = merged.kernel;
+            st.bytes = merged.bytes;
+            st.flops = merged.flops;
+            plan->stats.push_back(st);
+            merged.stat = (int)plan->stats.size() - 1;
+            Step ms;
+            ms.kind = Step::LAUNCH;
+            ms.launch = std::move(merged);
+            out.erase(out.begin() + (std::ptrdiff_t)i, out.begin() + (std::ptrdiff_t)j);
+            out.insert(out.begin() + (std::ptrdiff_t)i, std::move(ms));
+        }
+    }
+
+    void flush_region_launches(const IdSet& live, bool final_region, std::vector<Step>& out) {
         RegionPlan rp;
         collect_wanted(rp, live, final_region);
         order_nodes(rp);
@@ -3060,7 +3149,44 @@ struct Lowerer {
             plan->results[d] = r;
         }
         for (auto& s : slots) plan->slot_elems.push_back(s.first);
+        drop_unused_kernels();
         return std::move(plan);
+    }
+
+    // Kernels and statistics entries that no launch refers to any more (their launches became phases of a merged
+    // launch, or were generated again with a loop flag) are left out of the plan: they would only be compiled.
+    void drop_unused_kernels() {
+        std::vector<int> kernel_map(plan->kernels.size(), -1), stat_map(plan->stats.size(), -1);
+        std::function<void(std::vector<Step>&, bool)> walk = [&](std::vector<Step>& steps, bool assign) {
+            for (Step& st : steps) {
+                if (st.kind == Step::LAUNCH) {
+                    if (!assign) {
+                        kernel_map[(size_t)st.launch.kernel] = 0;
+                        if (st.launch.stat >= 0) stat_map[(size_t)st.launch.stat] = 0;
+                    } else {
+                        st.launch.kernel = kernel_map[(size_t)st.launch.kernel];
+                        if (st.launch.stat >= 0) st.launch.stat = stat_map[(size_t)st.launch.stat];
+                    }
+                }
+                walk(st.body, assign);
+                for (auto& arm : st.arms) walk(arm.second, assign);
+                walk(st.else_body, assign);
+            }
+        };
+        walk(plan->steps, false);
+        std::vector<KernelDef> kernels;
+        for (size_t i = 0; i < plan->kernels.size(); ++i)
+            if (kernel_map[i] == 0) { kernel_map[i] = (int)kernels.size(); kernels.push_back(std::move(plan->kernels[i])); }
+        std::vector<KernelStat> stats;
+        for (size_t i = 0; i < plan->stats.size(); ++i)
+            if (stat_map[i] == 0) {
+                stat_map[i] = (int)stats.size();
+                stats.push_back(std::move(plan->stats[i]));
+                stats.back().kernel = kernel_map[(size_t)stats.back().kernel];
+            }
+        plan->kernels.swap(kernels);
+        plan->stats.swap(stats);
+        walk(plan->steps, true);
     }
 };
 
@@ -3125,6 +3251,7 @@ std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::str
     LowerOptions opt = opt_in;
     if (const char* e = getenv("ADHIP_GROUP_DOTS")) opt.group_dots = opt.group_dots && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_LAYER_KERNELS")) opt.layer_kernels = opt.layer_kernels && atoi(e) != 0;
+    if (const char* e = getenv("ADHIP_MERGE_SMALL")) opt.merge_small = opt.merge_small && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_FUSE_ATTENTION")) opt.fuse_attention = opt.fuse_attention && atoi(e) != 0;
     Lowerer l(prog, dep_ids, opt);
     return l.run();

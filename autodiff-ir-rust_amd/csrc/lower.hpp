@@ -16,6 +16,7 @@ struct LowerOptions {
     bool fuse = true;  // false: one kernel per compute command (diagnostic mode)
     bool group_dots = true;  // same-shape independent matrix products share a launch
     bool layer_kernels = true;  // groups that run the same generated kernels on other buffers share their launches
+    bool merge_small = true;    // consecutive single-block launches of a region run as phases of one launch
     bool fuse_attention = true;  // dot(softmax(scale * dot(Q, K^T)), V) runs as one kernel
 };
 

@@ -64,7 +64,8 @@ def test_cxx_writer_matches_the_committed_bytes(tmp_path):
     assert out == open(GOLDEN, "rb").read()
 
 
-def test_reader_accepts_the_stream_and_sees_every_command():
+def test_reader_accepts_the_stream_and_sees_every_command(monkeypatch):
+    monkeypatch.setenv("ADHIP_MERGE_SMALL", "0")   # one launch per kernel, so that each shows in the plan by name
     text = lower_describe(every_command_program(), set(KEEP))
     # the program lowers: every kept id has a home buffer, the loop and the branch are there
     for k in KEEP:
