@@ -228,6 +228,14 @@ class HipDevice(Device):
         if rc != 0:
             raise RuntimeError("adhip_execute failed: " + self.last_error())
 
+    def execute_serialized(self, blob: bytes, dep_ids: Iterable[str]) -> None:
+        """`execute` for a procedure that `ir.serialize` has already turned into the wire format (the caller keeps
+        the payload arrays alive): what one `adhip_execute` call costs without the Python serialiser in front."""
+        arr, n = _dep_array(dep_ids)
+        rc = self._lib.adhip_execute(self._ctx, blob, len(blob), arr, n)
+        if rc != 0:
+            raise RuntimeError("adhip_execute failed: " + self.last_error())
+
     def compile(self, proc: IR.IRProcedure, dep_ids: Iterable[str]) -> Program:
         return Program(self, proc, dep_ids)
 

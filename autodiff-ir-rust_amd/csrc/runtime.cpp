@@ -122,6 +122,11 @@ struct adhip_program {
     std::unique_ptr<Plan> plan;
     std::vector<void*> buf_ptr;   // per plan buffer
     std::vector<void*> owned;     // allocations to free
+    // Small home / constant buffers share one allocation, uploaded ones first: their payloads go up in one copy and
+    // the small results come back in one, instead of a copy per buffer (a few microseconds each, and they queue up).
+    char* arena = nullptr;
+    std::vector<size_t> arena_off;   // per plan buffer: offset in the arena, or SIZE_MAX
+    size_t arena_upload_bytes = 0;   // the uploaded buffers occupy [0, arena_upload_bytes)
     std::vector<hipFunction_t> fn;  // per plan kernel
     std::vector<std::shared_ptr<Module>> mods;
     bool profiling = false;
@@ -394,9 +399,38 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
             p->flag_fn = get_function(*m, "adhip_flag");
         }
         p->buf_ptr.resize(plan.buffers.size(), nullptr);
+        p->arena_off.assign(plan.buffers.size(), SIZE_MAX);
+        {
+            // the arena: uploaded small buffers, then small results, then the other small ones, 256-byte aligned each,
+            // as long as everything fits half the staging area
+            std::set<int> result_bufs;
+            for (auto& kv : plan.results) result_bufs.insert(kv.second.buf);
+            size_t total = 0;
+            for (int pass = 0; pass < 3; ++pass) {
+                for (size_t i = 0; i < plan.buffers.size(); ++i) {
+                    const PlanBuffer& b = plan.buffers[i];
+                    if (b.kind == PlanBuffer::TEMP || p->arena_off[i] != SIZE_MAX) continue;
+                    const size_t nb = (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float);
+                    const bool uploaded = b.host && b.host_elems > 0;
+                    const int cls = uploaded ? 0 : (result_bufs.count((int)i) ? 1 : 2);
+                    if (cls != pass || nb > kStageMaxItem || total + nb > kStageBytes / 2) continue;  // half: the rest stages what is not in the arena
+                    p->arena_off[i] = total;
+                    total += (nb + 255) & ~size_t(255);
+                }
+                if (pass == 0) p->arena_upload_bytes = total;
+            }
+            if (total > 0) {
+                void* q = nullptr;
+                HIP_OK(hipMalloc(&q, total));
+                p->owned.push_back(q);
+                p->device_bytes += total;
+                p->arena = (char*)q;
+            }
+        }
         for (size_t i = 0; i < plan.buffers.size(); ++i) {
             const PlanBuffer& b = plan.buffers[i];
             if (b.kind == PlanBuffer::TEMP) { p->buf_ptr[i] = slot_ptr[b.slot]; continue; }
+            if (p->arena_off[i] != SIZE_MAX) { p->buf_ptr[i] = p->arena + p->arena_off[i]; continue; }
             void* q = nullptr;
             HIP_OK(hipMalloc(&q, (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float)));
             p->owned.push_back(q);
@@ -428,14 +462,27 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
     return p.release();
 }
 
-void program_upload(adhip_program* p) {
+// `wait`: return only when the copies are done (a caller of adhip_program_upload may reuse its payload memory then)
+void program_upload(adhip_program* p, bool wait = true) {
     adhip_ctx* ctx = p->ctx;
     HIP_OK(hipSetDevice(ctx->device));
     Plan& plan = *p->plan;
     size_t staged = 0;
+    if (p->arena_upload_bytes > 0) {
+        // the small payloads, laid out as they sit in the arena, in one copy
+        memset(ctx->stage, 0, p->arena_upload_bytes);
+        for (size_t i = 0; i < plan.buffers.size(); ++i) {
+            const PlanBuffer& b = plan.buffers[i];
+            if (p->arena_off[i] < p->arena_upload_bytes && b.host && b.host_elems > 0)
+                memcpy(ctx->stage + p->arena_off[i], b.host, (size_t)b.host_elems * sizeof(float));
+        }
+        HIP_OK(hipMemcpyAsync(p->arena, ctx->stage, p->arena_upload_bytes, hipMemcpyHostToDevice, ctx->stream));
+        staged = p->arena_upload_bytes;
+    }
     for (size_t i = 0; i < plan.buffers.size(); ++i) {
         const PlanBuffer& b = plan.buffers[i];
         if (b.kind == PlanBuffer::TEMP) continue;
+        if (p->arena_off[i] < p->arena_upload_bytes && b.host && b.host_elems > 0) continue;  // went up with the arena
         if (b.host && b.host_elems > 0) {
             const size_t nb = (size_t)b.host_elems * sizeof(float);
             const void* src = b.host;
@@ -454,7 +501,7 @@ void program_upload(adhip_program* p) {
             HIP_OK(hipMemsetAsync(p->buf_ptr[i], 0, (size_t)std::max<int64_t>(b.elems, 1) * sizeof(float), ctx->stream));
         }
     }
-    HIP_OK(hipStreamSynchronize(ctx->stream));
+    if (wait) HIP_OK(hipStreamSynchronize(ctx->stream));
 }
 
 hipEvent_t get_event(adhip_program* p) {
@@ -705,12 +752,27 @@ void program_readback(adhip_program* p) {
     struct Staged { HostResult* r; size_t off, nb; };
     std::vector<Staged> staged;
     size_t used = 0;
+    size_t reserved = 0;  // the head of the staging area that holds the arena's stretch until the last result is out
     auto drain = [&] {
         HIP_OK(hipStreamSynchronize(ctx->stream));
         for (auto& st : staged) memcpy(st.r->data.data(), ctx->stage + st.off, st.nb);
         staged.clear();
-        used = 0;
+        used = reserved;
     };
+    // the small results that live in the arena come back in one copy of the stretch they span
+    size_t span_lo = SIZE_MAX, span_hi = 0;
+    for (auto& kv : p->plan->results) {
+        const size_t off = p->arena_off[(size_t)kv.second.buf];
+        const int64_t ne = numel(kv.second.shape);
+        if (off == SIZE_MAX || ne <= 0) continue;
+        span_lo = std::min(span_lo, off);
+        span_hi = std::max(span_hi, off + (size_t)ne * sizeof(float));
+    }
+    const bool span = span_lo < span_hi && span_hi - span_lo <= kStageBytes;
+    if (span) {
+        HIP_OK(hipMemcpyAsync(ctx->stage, p->arena + span_lo, span_hi - span_lo, hipMemcpyDeviceToHost, ctx->stream));
+        reserved = used = (span_hi - span_lo + 255) & ~size_t(255);
+    }
     for (auto& kv : p->plan->results) {
         HostResult& r = ctx->results[kv.first];
         auto prev = previous.find(kv.first);
@@ -732,6 +794,10 @@ void program_readback(adhip_program* p) {
         r.release();
         r.data.resize((size_t)std::max<int64_t>(ne, 0));
         if (ne <= 0) continue;
+        if (span && p->arena_off[(size_t)kv.second.buf] != SIZE_MAX) {
+            staged.push_back({&r, p->arena_off[(size_t)kv.second.buf] - span_lo, nb});
+            continue;
+        }
         if (nb <= kStageMaxItem) {
             if (used + nb > kStageBytes) drain();
             HIP_OK(hipMemcpyAsync(ctx->stage + used, p->buf_ptr[kv.second.buf], nb, hipMemcpyDeviceToHost, ctx->stream));
@@ -891,8 +957,10 @@ int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, co
                     }
                 }
             }
-            program_upload(p);
-            program_run(p);
+            // one wait for the whole call: uploads, kernels and read-back copies are ordered by the stream, and the
+            // read-back ends with the wait that also covers the staging area both ends use
+            program_upload(p, false);
+            program_run(p, p->profiling);
             program_readback(p);
         } catch (...) {
             // a program that failed is not kept

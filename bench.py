@@ -296,6 +296,15 @@ def main():
         for _ in range(20):
             dev.execute(proc1, deps1)
         us_exec = (time.perf_counter() - t0) / 20 * 1e6
+        # the same call without the Python serialiser in front of it: the C ABI on a stream that is already in wire format
+        from adhip import ir as IR
+        blob1, keepalive1 = IR.serialize(proc1)
+        dev.execute_serialized(blob1, deps1)
+        t0 = time.perf_counter()
+        for _ in range(50):
+            dev.execute_serialized(blob1, deps1)
+        us_abi = (time.perf_counter() - t0) / 50 * 1e6
+        del keepalive1
         p1 = dev.compile(proc1, deps1)
         p1.upload()
         p1.run()
@@ -303,7 +312,7 @@ def main():
         for _ in range(50):
             p1.run()
         us_run = (time.perf_counter() - t0) / 50 * 1e6
-        extra["readme_mlp"] = {"us_per_execute_call": us_exec, "us_per_resident_run": us_run,
+        extra["readme_mlp"] = {"us_per_execute_call": us_exec, "us_per_adhip_execute": us_abi, "us_per_resident_run": us_run,
                                "kernels_per_run": sum(1 for s_ in p1.kernel_stats())}
         p1.close()
         # config 3: reductions
