@@ -914,3 +914,38 @@ def test_loop_flag_latched_by_the_body(case, hip_device):
     for k in keep:
         assert got[k].dim == ref[k].dim, k
         assert_close(got[k].data, ref[k].data, 4 * ELW_RTOL, k)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [501, 502, 503, 504])
+def test_small_programs_one_launch_per_kernel_and_merged_agree(seed, hip_device, monkeypatch):
+    """Programs on tiny tensors run their single-block kernels as the phases of one launch; with ADHIP_MERGE_SMALL=0
+    every kernel is a launch of its own.  Both must give the oracle's result (data-flow programs and programs with
+    loops and branches; the seeds are used nowhere else, so that no kept plan of the other kind is reused)."""
+    print(f"[case] merged and unmerged small programs, seed {seed}", flush=True)
+    from adhip.device import lower_describe
+    from fuzz_control import random_control_program
+    from fuzz_programs import random_program
+    proc, keep, ints = random_control_program(seed)
+    merged_plan = lower_describe(proc, set(keep))
+    monkeypatch.setenv("ADHIP_MERGE_SMALL", "0")
+    assert "[merged]" in merged_plan and "[merged]" not in lower_describe(proc, set(keep))
+    oracle = OracleDevice()
+    oracle.execute(proc, set(keep))
+    hip_device.execute(proc, set(keep))           # one launch per kernel
+    for k in keep:
+        got, ref = hip_device.get_tensor(k), oracle.get_tensor(k)
+        assert got.dim == ref.dim, k
+        if k in ints or k.startswith("i"):
+            assert_exact(got.data, ref.data, f"unmerged {k}")
+        else:
+            assert_close(got.data, ref.data, 2e-5, f"unmerged {k}", scale=max(1.0, float(np.max(np.abs(ref.data)))))
+    got = random_program(hip_device, seed)         # one launch per kernel
+    ref = random_program(OracleDevice(), seed)
+    monkeypatch.delenv("ADHIP_MERGE_SMALL")
+    again = random_program(hip_device, seed + 1000)  # merged, another program
+    ref2 = random_program(OracleDevice(), seed + 1000)
+    for out, want in ((got, ref), (again, ref2)):
+        for k, rv in want.items():
+            assert out[k].dim == rv.dim, k
+            assert_close(out[k].data, rv.data, 2e-4, k)
