@@ -37,10 +37,13 @@ std::string attention_kernel_source(const AttentionConfig& cfg, const std::strin
     std::string params, pick = "switch (problem) {";
     for (int i = 0; i < kAttentionSlots; ++i) {
         params += strf("float* o%d, const float* q%d, const float* k%d, const float* v%d, ", i, i, i, i);
-        pick += strf(" case %d: O = o%d; Q = q%d; K = k%d; V = v%d; break;", i, i, i, i, i);
+        if (cfg.mask) params += strf("const float* m%d, ", i);
+        pick += strf(" case %d: O = o%d; Q = q%d; K = k%d; V = v%d;%s break;", i, i, i, i, i, cfg.mask ? strf(" Mk = m%d;", i).c_str() : "");
     }
     s += "#define GROUP_PARAMS " + params + "\n#define GROUP_PICK " + pick + " default: return; }\n";
-    s += strf("#define KERNEL_NAME %s\n#define D %d\n#define DV %d\n#define BN %d\n#define WG %d\n", entry.c_str(), cfg.d, cfg.dv, cfg.bn, cfg.wg);
+    s += strf("#define KERNEL_NAME %s\n#define D %d\n#define DV %d\n#define BN %d\n#define WG %d\n#define MASK %d\n", entry.c_str(), cfg.d, cfg.dv, cfg.bn,
+              cfg.wg, cfg.mask ? 1 : 0);
+    s += cfg.mask ? "#define MASK_LD long long m_ld,\n" : "#define MASK_LD\n";
     s += "typedef float float4_t __attribute__((ext_vector_type(4)));\n";
     s += R"ATTN(
 #define NT (256 * WG)
@@ -70,7 +73,7 @@ static __device__ __forceinline__ float row16_sum(float x) {
 
 extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     const int* __restrict__ guard, GROUP_PARAMS long long Sq, long long Sk, long long q_ld, long long k_ld, long long v_ld,
-    float scale, int row_blocks, int problems) {
+    MASK_LD float scale, int row_blocks, int problems) {
     if (guard && *guard == 0) return;
     // Blocks are handed to the eight XCDs in turn; renumbering them so that an XCD's blocks are consecutive puts the row
     // blocks of one problem on one XCD, whose L2 then fetches that problem's K and V once.
@@ -84,6 +87,9 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     const float* __restrict__ Q;
     const float* __restrict__ K;
     const float* __restrict__ V;
+#if MASK
+    const float* __restrict__ Mk;
+#endif
     GROUP_PICK
     __shared__ __attribute__((aligned(16))) float lds[2 * STAGE + 4 * WG * 16 * PLD];
     float (*Ps)[16][PLD] = (float (*)[16][PLD])(lds + 2 * STAGE);
@@ -115,6 +121,16 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     float m_i[4], l_i[4];   // running maximum of the row; this lane's share of the running sum (added up at the end)
 #pragma unroll
     for (int r = 0; r < 4; ++r) { m_i[r] = -__builtin_inff(); l_i[r] = 0.0f; }
+#if MASK
+    // where this lane's four accumulator rows start in the mask, at this key group's and lane's column (rows beyond Sq
+    // are never stored: they read the last row)
+    const float* mrow[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const long long row = row_base + 4 * lq + r;
+        mrow[r] = Mk + (row < Sq ? row : Sq - 1) * m_ld + kg * BNW + li;
+    }
+#endif
 
     // The next tile travels through registers.  Where a thread's pieces sit inside a tile, in memory and in LDS, is
     // computed once; a tile's base is uniform.  Keys beyond Sk (last tile only) are fetched from the last valid row
@@ -225,10 +241,23 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
         float mx[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) mx[r] = -__builtin_inff();
+#if MASK
+#pragma unroll
+        for (int nb = 0; nb < BNW / 16; ++nb) {
+            // the scaled score times the mask, in that order, as the caller wrote it; keys beyond Sk read nothing
+            const bool inside = k0 + BN <= Sk || k0 + kg * BNW + 16 * nb + li < Sk;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float mv = inside ? mrow[r][k0 + 16 * nb] : 0.0f;
+                sacc[nb][r] = ((sacc[nb][r] + sodd[nb][r]) * scale) * mv;
+            }
+        }
+#else
 #pragma unroll
         for (int nb = 0; nb < BNW / 16; ++nb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) sacc[nb][r] = (sacc[nb][r] + sodd[nb][r]) * scale;
+#endif
         if (k0 + BN > Sk) {   // the last tile may reach beyond the keys
 #pragma unroll
             for (int nb = 0; nb < BNW / 16; ++nb) {

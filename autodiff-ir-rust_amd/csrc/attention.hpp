@@ -10,6 +10,7 @@ struct AttentionConfig {
     int dv = 128;  // features of a value / result row (multiple of 16, at most 256)
     int bn = 64;   // keys per tile (64 or 32)
     int wg = 2;    // key groups: 1 (a block is 4 wavefronts) or 2 (8 wavefronts, each group takes half of every tile)
+    bool mask = false;  // the scaled scores are multiplied by a [Sq, Sk] mask before the softmax
 };
 
 // bytes of LDS a block of this configuration needs (two stages of K and V tiles and a patch per wavefront)

@@ -1055,16 +1055,19 @@ struct Lowerer {
     }
 
     struct AttentionKey {
-        int64_t sq = 0, sk = 0, d = 0, dv = 0, q_ld = 0, k_ld = 0, v_ld = 0;
+        int64_t sq = 0, sk = 0, d = 0, dv = 0, q_ld = 0, k_ld = 0, v_ld = 0, m_ld = 0;  // m_ld: 0 without a mask
         float scale = 0.f;
         bool operator==(const AttentionKey& o) const {
-            return sq == o.sq && sk == o.sk && d == o.d && dv == o.dv && q_ld == o.q_ld && k_ld == o.k_ld && v_ld == o.v_ld && scale == o.scale;
+            return sq == o.sq && sk == o.sk && d == o.d && dv == o.dv && q_ld == o.q_ld && k_ld == o.k_ld && v_ld == o.v_ld &&
+                   m_ld == o.m_ld && scale == o.scale;
         }
     };
     // shape and strides of an ATTN node's operands, if they are what the kernel reads: unit stride inside a row of Q,
     // K and V, rows of K and V 16-byte aligned
-    static bool attention_key(const Node* n, AttentionKey& k, Affine2D& q, Affine2D& kt, Affine2D& v) {
-        if (n->in.size() != 3 || !tref_affine2d(n->in[0], q) || !tref_affine2d(n->in[1], kt) || !tref_affine2d(n->in[2], v)) return false;
+    // A fourth operand is a [Sq, Sk] mask the scaled scores are multiplied with before the softmax (reference
+    // src/nn/transformer.rs:21-30); `mask` receives its description.
+    static bool attention_key(const Node* n, AttentionKey& k, Affine2D& q, Affine2D& kt, Affine2D& v, Affine2D* mask = nullptr) {
+        if ((n->in.size() != 3 && n->in.size() != 4) || !tref_affine2d(n->in[0], q) || !tref_affine2d(n->in[1], kt) || !tref_affine2d(n->in[2], v)) return false;
         k.sq = n->in[0].shape[0];
         k.d = n->in[0].shape[1];
         k.sk = n->in[1].shape[1];
@@ -1078,6 +1081,14 @@ struct Lowerer {
         k.q_ld = q.s0;
         k.k_ld = kt.s1;
         k.v_ld = v.s0;
+        k.m_ld = 0;
+        if (n->in.size() == 4) {
+            Affine2D m;
+            if (!tref_affine2d(n->in[3], m) || n->in[3].shape != Shape{k.sq, k.sk}) return false;
+            if ((m.s1 != 1 && k.sk > 1) || m.s0 < 1 || m.s0 >= (int64_t(1) << 31)) return false;
+            k.m_ld = m.s0;
+            if (mask) *mask = m;
+        }
         k.scale = n->cval;
         return true;
     }
@@ -1130,22 +1141,34 @@ struct Lowerer {
                 }
             }
             if (!M) continue;
-            // X = scale * (Q K^T)
+            // X = scale * (Q K^T), or that times a mask of the scores' shape
             float scale = 0.f;
             Node* D1 = times_constant(X, scale);
+            Node* X0 = nullptr;   // the scaled scores under a mask
+            const TRef* mask = nullptr;
+            if (!D1 && X->op == Op::MUL && X->in.size() == 2) {
+                for (int k = 0; k < 2 && !D1; ++k) {
+                    Node* x0 = whole_value(X->in[(size_t)k]);
+                    if (!x0 || X->in[(size_t)(1 - k)].shape != Shape{Sq, Sk}) continue;
+                    Node* d1 = times_constant(x0, scale);
+                    if (d1 && d1->op == Op::DOT) { D1 = d1; X0 = x0; mask = &X->in[(size_t)(1 - k)]; }
+                }
+            }
             if (!D1 || D1->op != Op::DOT) continue;
             if (!only_for(P, {O}) || !only_for(E, {P, S}) || !only_for(R, {P}) || !only_for(S, {R}) || !only_for(E1, {E}) ||
-                !only_for(Dn, {E1}) || !only_for(N1, {Dn}) || !only_for(M, {N1}) || !only_for(X, {Dn, M}) || !only_for(D1, {X}))
+                !only_for(Dn, {E1}) || !only_for(N1, {Dn}) || !only_for(M, {N1}) || !only_for(X, {Dn, M}))
                 continue;
+            if (X0 ? (!only_for(X0, {X}) || !only_for(D1, {X0})) : !only_for(D1, {X})) continue;
             // would the kernel accept the operands as they are?
             Node probe;
             probe.in = {D1->in[0], D1->in[1], O->in[1]};
+            if (mask) probe.in.push_back(*mask);
             probe.cval = scale;
             AttentionKey key;
-            Affine2D q, kt, v;
-            if (!attention_key(&probe, key, q, kt, v)) continue;
+            Affine2D q, kt, v, mk;
+            if (!attention_key(&probe, key, q, kt, v, &mk)) continue;
             auto in_memory_able = [](const Affine2D& a) { return op_is_leaf(a.base->op) || op_is_elw(a.base->op) || a.base->root || op_is_reduce(a.base->op) || a.base->op == Op::DOT || a.base->op == Op::ATTN; };
-            if (!in_memory_able(q) || !in_memory_able(kt) || !in_memory_able(v)) continue;
+            if (!in_memory_able(q) || !in_memory_able(kt) || !in_memory_able(v) || (mask && !in_memory_able(mk))) continue;
             O->op = Op::ATTN;
             O->in = probe.in;
             O->cval = scale;
@@ -2503,7 +2526,7 @@ struct Lowerer {
                 if (!attention_key(groups[g].members[0], ak, q, kt, v)) continue;
                 uint32_t sb;
                 memcpy(&sb, &ak.scale, 4);
-                key[g] = {ak.sq, ak.sk, ak.d, ak.dv, ak.q_ld, ak.k_ld, ak.v_ld, (int64_t)sb | (int64_t(1) << 40)};
+                key[g] = {ak.sq, ak.sk, ak.d, ak.dv + (ak.m_ld << 10), ak.q_ld, ak.k_ld, ak.v_ld, (int64_t)sb | (int64_t(1) << 40)};
                 cand[g] = 1;
                 ++ncand;
             }
@@ -2707,6 +2730,7 @@ struct Lowerer {
         AttentionConfig cfg;
         cfg.d = (int)key0.d;
         cfg.dv = (int)key0.dv;
+        cfg.mask = key0.m_ld > 0;
         const int64_t row_blocks = (key0.sq + 63) / 64;
         // A launch with two or more blocks per CU runs blocks of four wavefronts on tiles of 32 keys, two of which fit
         // a CU's LDS while the heads are not too wide; a smaller launch splits every tile between two groups of four
@@ -2716,7 +2740,7 @@ struct Lowerer {
         if (row_blocks * cnt >= 512 && narrow) { cfg.bn = 32; cfg.wg = 1; }
         else { cfg.bn = narrow ? 64 : 32; cfg.wg = 2; }
         ADHIP_CHECK(attention_lds_bytes(cfg) <= 160 * 1024, "internal: attention tiles of %d keys do not fit in LDS", cfg.bn);
-        const std::string entry = strf("adhip_attention_d%d_v%d_k%d_w%d", cfg.d, cfg.dv, cfg.bn, cfg.wg);
+        const std::string entry = strf("adhip_attention_d%d_v%d_k%d_w%d%s", cfg.d, cfg.dv, cfg.bn, cfg.wg, cfg.mask ? "_mask" : "");
         Launch l;
         l.kernel = add_kernel(entry, attention_kernel_source(cfg, entry), "attention");
         l.block[0] = 256u * (unsigned)cfg.wg;
@@ -2734,14 +2758,16 @@ struct Lowerer {
         for (int i = 0; i < kAttentionSlots; ++i) {
             Node* n = atts[(size_t)std::min(i, cnt - 1)];  // unused slots repeat the last problem; no block reads them
             AttentionKey key;
-            Affine2D q, kt, v;
-            ADHIP_CHECK(attention_key(n, key, q, kt, v) && key == key0, "internal: attention problems of one launch differ");
+            Affine2D q, kt, v, mk;
+            ADHIP_CHECK(attention_key(n, key, q, kt, v, &mk) && key == key0, "internal: attention problems of one launch differ");
             l.args.push_back(B(n, 0));
             l.args.push_back(B(q.base, q.offset));
             l.args.push_back(B(kt.base, kt.offset));
             l.args.push_back(B(v.base, v.offset));
+            if (cfg.mask) l.args.push_back(B(mk.base, mk.offset));
         }
         for (int64_t v : {key0.sq, key0.sk, key0.q_ld, key0.k_ld, key0.v_ld}) l.args.push_back(I(v));
+        if (cfg.mask) l.args.push_back(I(key0.m_ld));
         Arg sc;
         sc.kind = Arg::F32;
         sc.fv = key0.scale;
@@ -2749,7 +2775,8 @@ struct Lowerer {
         for (int64_t v : {row_blocks, (int64_t)cnt}) { Arg a; a.kind = Arg::I32; a.iv = v; l.args.push_back(a); }
         l.label = strf("attention_%s_%dx_%lldx%lldx%lldx%lld", atts[0]->name.c_str(), cnt, (long long)key0.sq, (long long)key0.sk,
                        (long long)key0.d, (long long)key0.dv);
-        l.bytes = 4.0 * cnt * ((double)key0.sq * key0.d + (double)key0.sk * key0.d + (double)key0.sk * key0.dv + (double)key0.sq * key0.dv);
+        l.bytes = 4.0 * cnt * ((double)key0.sq * key0.d + (double)key0.sk * key0.d + (double)key0.sk * key0.dv + (double)key0.sq * key0.dv) +
+                  (cfg.mask ? 4.0 * (double)key0.sq * (double)key0.sk : 0.0);
         l.flops = 2.0 * cnt * (double)key0.sq * (double)key0.sk * (double)(key0.d + key0.dv);
         push_launch(out, l, "attention");
     }

@@ -201,10 +201,11 @@ def test_attention_lowers_to_one_kernel(sq, sk, d, dv):
     assert rc == 0, msg
 
 
-@pytest.mark.parametrize("what", ["mask", "scores_kept", "head_of_6", "plain_exp"])
+@pytest.mark.parametrize("what", ["mask_of_another_shape", "scores_kept", "head_of_6", "plain_exp"])
 def test_attention_that_does_not_match_stays_unfused(what, monkeypatch):
-    """A mask between the scaling and the softmax, a softmax somebody else reads, a head width the kernel has no tile
-    for, or the reference's own max-less softmax: none of them is the fused kernel's arithmetic."""
+    """A factor between the scaling and the softmax that is not a mask of the scores' shape, a softmax somebody else
+    reads, a head width the kernel has no tile for, or the reference's own max-less softmax: none of them is the fused
+    kernel's arithmetic."""
     from adhip.core import ValueData
     from adhip.device import Device, lower_describe
 
@@ -217,8 +218,13 @@ def test_attention_that_does_not_match_stays_unfused(what, monkeypatch):
 
     dev = Capture()
     autodiff.set_device(dev)
-    if what == "mask":
-        _attention_program(dev, 64, 64, 16, 16, 64, 0, mask=True)
+    if what == "mask_of_another_shape":
+        rng = np.random.default_rng(0)
+        Q, K, V = (autodiff.tensor(rng.standard_normal((64, 16)).astype(np.float32), [64, 16]) for _ in range(3))
+        row = autodiff.tensor(rng.random(64).astype(np.float32), [64])     # one factor per key, broadcast over the queries
+        o = dot((dot(Q, K.t()) / 8.0 * row).softmax(-1), V)
+        o.forward()
+        o.val().keep()
     elif what == "head_of_6":
         _attention_program(dev, 64, 64, 6, 16, 64, 0)
     else:
@@ -257,6 +263,79 @@ def test_attention_fusion_can_be_switched_off(monkeypatch):
     assert "[attention]" in lower_describe(dev.proc, dev.deps)
     monkeypatch.setenv("ADHIP_FUSE_ATTENTION", "0")
     assert "[attention]" not in lower_describe(dev.proc, dev.deps)
+
+
+_MASKED_SHAPES = [(64, 64, 16, 16), (100, 100, 48, 48), (65, 129, 8, 32), (257, 640, 128, 128), (96, 200, 256, 256),
+                  (1, 7, 4, 16), (33000, 40, 16, 16)]
+
+
+@pytest.mark.parametrize("sq,sk,d,dv", _MASKED_SHAPES)
+def test_masked_attention_lowers_to_one_kernel(sq, sk, d, dv):
+    from adhip.core import ValueData
+    from adhip.device import Device, lower_describe
+    from test_library_cpu import _compile_check
+
+    class Capture(Device):
+        def execute(self, proc, deps):
+            self.proc, self.deps = proc, list(deps)
+
+        def get_tensor(self, id):
+            return ValueData.none()
+
+    dev = Capture()
+    _attention_program(dev, sq, sk, d, dv, 64, 0, mask=True)
+    autodiff.execute()
+    launches = [l for l in lower_describe(dev.proc, dev.deps).splitlines() if l.lstrip().startswith("launch")]
+    assert len(launches) == 1 and "[attention]" in launches[0] and "_mask" in launches[0], launches
+    rc, msg = _compile_check(dev.proc, dev.deps)
+    assert rc == 0, msg
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sq,sk,d,dv", _MASKED_SHAPES)
+def test_fused_masked_attention_matches_oracle_and_float64(sq, sk, d, dv, hip_device):
+    """AttentionMasked (the scaled scores times a 0/1 mask, then softmax: reference src/nn/transformer.rs:21-30) through
+    the fused kernel, against the oracle running the unfused commands and against float64."""
+    print(f"[case] fused masked attention {sq}x{sk} d {d} dv {dv}", flush=True)
+    o, (qn, kn, vn, mn) = _attention_program(hip_device, sq, sk, d, dv, 16, sq + sk, spread=2.0, mask=True)
+    autodiff.execute()
+    got = o.val().get()
+    ro, _ = _attention_program(OracleDevice(), sq, sk, d, dv, 16, sq + sk, spread=2.0, mask=True)
+    autodiff.execute()
+    ref = ro.val().get()
+    assert got.dim == ref.dim == [sq, dv]
+    tol = 4 * RED_RTOL * math.sqrt(max(sk, d))
+    assert_close(got.data, ref.data, tol, "o vs oracle")
+    assert_close(got.data, _attention_float64(qn, kn, vn, 16, mn).reshape(-1), tol, "o vs float64")
+
+
+@pytest.mark.gpu
+def test_masked_multi_head_attention_fused_equals_unfused(hip_device, monkeypatch):
+    """MaskedMultiHeadAttention (every head under the same causal mask) fused and unfused."""
+    print("[case] masked multi-head attention 200x96 heads 3", flush=True)
+    from adhip import nn
+    seq, d_model, heads = 200, 96, 3
+
+    def run():
+        autodiff.set_device(hip_device)
+        rng = np.random.default_rng(5)
+        mask = autodiff.tensor(np.tril(np.ones((seq, seq), dtype=np.float32)), [seq, seq])
+        mha = nn.MaskedMultiHeadAttention(d_model, heads, mask)
+        for group in (mha.wq, mha.wk, mha.wv):
+            for lin in group:
+                lin.w = autodiff.tensor((rng.standard_normal((d_model, d_model // heads)) / 10).astype(np.float32), [d_model, d_model // heads])
+        mha.wo.w = autodiff.tensor((rng.standard_normal((d_model, d_model)) / 10).astype(np.float32), [d_model, d_model])
+        x = autodiff.tensor(rng.standard_normal((seq, d_model)).astype(np.float32), [seq, d_model])
+        y = mha.f(x)
+        y.forward()
+        y.val().keep()
+        autodiff.execute()
+        return y.val().get()
+    fused = run()
+    monkeypatch.setenv("ADHIP_FUSE_ATTENTION", "0")
+    plain = run()
+    assert fused.dim == plain.dim == [seq, d_model]
+    assert_close(fused.data, plain.data, 4 * RED_RTOL * math.sqrt(seq), "fused vs unfused")
 
 
 @pytest.mark.gpu
