@@ -934,7 +934,12 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
     if (spec.latch && vec == 1 && N == 1)
         for (size_t i = 0; i < spec.outputs.size(); ++i)
             if (spec.outputs[i] == spec.latch) latch_output = (int)i;
-    if (latch_output >= 0) { sig += ", int* latch"; k.latch_done = true; }
+    if (latch_output >= 0) {
+        // the flag the kernel latches is the one that guards it: the two parameters name the same word
+        sig.replace(sig.find("const int* __restrict__ guard"), strlen("const int* __restrict__ guard"), "const int* guard");
+        sig += ", int* latch";
+        k.latch_done = true;
+    }
     std::string src = kernel_prelude();
     // Large kernels do not walk through memory block after block.  A block is 16 wavefronts; wavefront w takes a 1 KiB
     // run (64 float4) in band row w, where a band is 16 rows of `band` bytes, and consecutive blocks take consecutive
@@ -1179,7 +1184,11 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         if (epi && spec.latch && V == 1)
             for (size_t i = 0; i < spec.epilogue_outputs.size(); ++i)
                 if (spec.epilogue_outputs[i] == spec.latch) latch_epi = (int)i;
-        if (latch_epi >= 0) { sig += ", int* latch"; k.latch_done = true; }
+        if (latch_epi >= 0) {
+            sig.replace(sig.find("const int* __restrict__ guard"), strlen("const int* __restrict__ guard"), "const int* guard");
+            sig += ", int* latch";
+            k.latch_done = true;
+        }
         src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
         src += "    if (guard && *guard == 0) return;\n";
         src += strf("    const unsigned lane = threadIdx.x %% %du;\n", T);

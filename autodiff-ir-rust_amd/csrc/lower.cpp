@@ -1251,7 +1251,7 @@ struct Lowerer {
                 ++j;
             }
             if (j - i < 2) continue;
-            std::string src, calls, params = "const int* __restrict__ guard";
+            std::string src, calls, params = "const int* guard";
             Launch merged;
             merged.block[0] = 256;
             merged.guard = out[i].launch.guard;
@@ -1260,9 +1260,11 @@ struct Lowerer {
                 const Launch& l = out[q].launch;
                 const KernelDef& kd = plan->kernels[(size_t)l.kernel];
                 std::string body = kd.source;
-                const std::string head = "extern \"C\" __global__", bounds = "__launch_bounds__(";
+                const std::string head = "extern \"C\" __global__", bounds = "__launch_bounds__(", noalias = "__restrict__";
                 for (size_t at = body.find(head); at != std::string::npos; at = body.find(head)) body.replace(at, head.size(), "static __device__");
                 for (size_t at = body.find(bounds); at != std::string::npos; at = body.find(bounds)) body.erase(at, body.find(')', at) + 1 - at);
+                // a buffer one phase writes is another phase's input: no parameter may promise that nothing else names its memory
+                for (size_t at = body.find(noalias); at != std::string::npos; at = body.find(noalias)) body.erase(at, noalias.size());
                 const size_t fn = body.find(" void " + kd.entry + "(");
                 const size_t open = fn == std::string::npos ? fn : body.find('(', fn);
                 const size_t close = open == std::string::npos ? open : body.find(") {", open);
