@@ -38,14 +38,28 @@ const char* kernel_prelude() {
     return R"(
 typedef float float4_t __attribute__((ext_vector_type(4)));
 static __device__ __forceinline__ float u2f(unsigned u) { return __builtin_bit_cast(float, u); }
+// Sums and maxima over a wavefront: within each row of 16 lanes by data-parallel-primitive moves (neighbour, other
+// pair, other quad mirrored, other half mirrored: register-to-register, no LDS round trip), then across the four rows.
+// Every lane ends up with the same bits.
+template <int CTRL> static __device__ __forceinline__ float wave_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
 static __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    v += wave_dpp<0xB1>(v);
+    v += wave_dpp<0x4E>(v);
+    v += wave_dpp<0x141>(v);
+    v += wave_dpp<0x140>(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
     return v;
 }
 static __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    v = fmaxf(v, wave_dpp<0xB1>(v));
+    v = fmaxf(v, wave_dpp<0x4E>(v));
+    v = fmaxf(v, wave_dpp<0x141>(v));
+    v = fmaxf(v, wave_dpp<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
 }
 // sin(x) for |x| <= 2^15 in ~15 instructions: x = k*pi + r with pi split in three floats (each fma is exact or rounds
@@ -680,14 +694,21 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
 }  // namespace
 
 // Rows one block of the column-sum layout covers: 16 (one per wavefront), times the number of rows each wavefront
-// walks, which is 1 until the partial sums would exceed 1024 rows.
-static int64_t elw_colsum_rows_per_wave(int64_t rows) { return std::max<int64_t>(1, (rows + 16 * 1024 - 1) / (16 * 1024)); }
+// walks.  That is 1 until the partial sums would exceed 1024 rows -- except for passes that move few streams (at most
+// three of: results stored, full-size operands read), where a block's closing steps (the sums across the wavefront,
+// the 16 rows through LDS) weigh more against its streaming: two rows per wavefront then, if that still leaves eight
+// blocks per CU.  Measured on 16384 x 4096 with one operand, one result, row and column sums: 103 -> 100 us a step;
+// on the 3-read + 4-write pass over 8192 x 8192 two rows per wavefront cost 4 % instead.
+static int64_t elw_colsum_rows_per_wave(int64_t rows, int64_t cols, int streams) {
+    const int64_t base = std::max<int64_t>(1, (rows + 16 * 1024 - 1) / (16 * 1024));
+    if (base == 1 && streams <= 3 && ((cols / 4 + 63) / 64) * ((rows + 31) / 32) >= 2048) return 2;
+    return base;
+}
 
 int64_t elw_rowsum_runs(int64_t cols) { return (cols / 4 + 63) / 64; }
 
-int64_t elw_colsum_tiles(int64_t rows, int64_t cols) {
-    (void)cols;
-    const int64_t per_block = 16 * elw_colsum_rows_per_wave(rows);
+int64_t elw_colsum_tiles(int64_t rows, int64_t cols, int streams) {
+    const int64_t per_block = 16 * elw_colsum_rows_per_wave(rows, cols, streams);
     return std::max<int64_t>(1, (rows + per_block - 1) / per_block);
 }
 
@@ -710,8 +731,8 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     const int64_t runs = elw_rowsum_runs(C);
     ElwBody b = elw_body(spec, members, Shape{R, C}, 4, wide);
     Gen& g = b.g;
-    const int64_t K = elw_colsum_rows_per_wave(R);
-    const int64_t tiles = elw_colsum_tiles(R, C);
+    const int64_t K = elw_colsum_rows_per_wave(R, C, spec.streams);
+    const int64_t tiles = elw_colsum_tiles(R, C, spec.streams);
     GeneratedKernel k;
     k.kind = "elw_colsum";
     k.entry = spec.name;
@@ -734,8 +755,8 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     src += strf("    const bool col_ok = c1 < %lld%s;\n", (long long)(C / 4), sfx);
     for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("    float cs%zu[4] = {0.f, 0.f, 0.f, 0.f};\n", i);
     if (K == 1) src += strf("    {\n        const %s c0 = (%s)blockIdx.y * 16u + wv;\n", it, it);
-    else src += strf("#pragma unroll 1\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n",
-                     (long long)K, it, it, (long long)(16 * K), sfx);
+    else src += strf("%s\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n",
+                     K <= 2 ? "#pragma unroll" : "#pragma unroll 1", (long long)K, it, it, (long long)(16 * K), sfx);
     for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("        float rs%zu = 0.f;\n", i);
     src += strf("        if (col_ok && c0 < %lld%s) {\n", (long long)R, sfx);
     src += join(g.codeA, "            ");

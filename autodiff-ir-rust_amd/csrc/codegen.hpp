@@ -37,6 +37,9 @@ struct ElwKernelSpec {
     struct RowSum { Node* value; Node* partial; };
     std::vector<RowSum> rowsums;
     int64_t rows = 0, cols = 0;
+    // with column or row sums: how many full-size streams the pass moves (results stored + full-size operands read);
+    // decides how many rows a wavefront walks, so it must be what elw_colsum_tiles is asked with
+    int streams = 8;
     // A one-element output that is the predicate of the device-predicated loop the kernel runs in: the thread that
     // stores it also latches `value != 0` into the loop's flag (a trailing `int* latch` parameter), which saves the
     // one-thread kernel that would do so at the top of the next iteration.  Honoured by the plain kernel form only;
@@ -82,8 +85,9 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
 // Reduce over the last dim of a [V,R] operand.  If the result needs `chunks > 1`, the kernel writes
 // partial sums laid out [chunks][V]; the caller reduces those with a second (column) reduction over the partials.
 GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks = 0);
-// Number of row tiles an element-wise kernel with column sums over [rows, cols] will use.
-int64_t elw_colsum_tiles(int64_t rows, int64_t cols);
+// Number of row tiles an element-wise kernel with column sums over [rows, cols] that moves `streams` full-size
+// streams (ElwKernelSpec::streams) will use.
+int64_t elw_colsum_tiles(int64_t rows, int64_t cols, int streams);
 
 // 2-D strided access description of a matmul operand, if the reference can be expressed that way.
 struct Affine2D {

@@ -250,6 +250,7 @@ struct Group {
     // row are added by a second pass
     std::vector<std::pair<Node*, Node*>> rowsums;
     int64_t cs_rows = 0, cs_cols = 0;  // the [rows, cols] view of the iteration space both kinds of sums refer to
+    int cs_streams = 8;                // full-size streams of a pass with sums (ElwKernelSpec::streams)
     bool rides() const { return !colsums.empty() || !rowsums.empty(); }
     std::vector<std::pair<Node*, Node*>> riders() const {
         std::vector<std::pair<Node*, Node*>> r = colsums;
@@ -1928,9 +1929,15 @@ struct Lowerer {
                 spec.name = name;
                 spec.rows = G.cs_rows;
                 spec.cols = G.cs_cols;
+                if (G.rides()) {
+                    G.cs_streams = (int)G.members.size();
+                    for (auto& rd : greads[g])
+                        if (numel(rd.first->shape) * 2 >= G.cs_rows * G.cs_cols) ++G.cs_streams;
+                    spec.streams = G.cs_streams;
+                }
                 for (auto& cs : G.colsums) {
                     // partial sums [tiles][cols], added by the fixed second-pass kernel
-                    const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
+                    const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols, G.cs_streams);
                     Node* S = cs.second;
                     Node* partial = new_node(Op::COPY, Shape{tiles, G.cs_cols}, {}, S->name + ".partial", 0.f, false);
                     partial->root = true;
@@ -2349,7 +2356,7 @@ struct Lowerer {
                 }
                 // one launch of the fixed second-pass kernel per four sums
                 if (fixed_finalize < 0) fixed_finalize = add_kernel("adhip_colsum_finalize", fixed_kernels_source(), "colsum_finalize");
-                const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols);
+                const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols, G.cs_streams);
                 for (size_t i0 = 0; i0 < G.colsums.size(); i0 += 4) {
                     const size_t cnt = std::min<size_t>(4, G.colsums.size() - i0);
                     Launch lf;

@@ -163,13 +163,20 @@ def test_manip_loop_full_size(hip_device):
     assert_exact(out["gathered"].data, expect.reshape(-1), "gathered")     # data movement: bit-exact
     assert out["i"].data[0] == 10.0
     r = expect.astype(np.float64) * w.astype(np.float64)
+    r0 = r
     for _ in range(10):
         r = r - 0.01 * r.sum(1, keepdims=True)
-    # each iteration multiplies the row sums by (1 - 7.68): compare relative to the row scale
+    # each iteration multiplies the row sums by (1 - 7.68): compare relative to the row scale.  After ten iterations a
+    # row is its first sum times a constant, so that sum's relative error carries through: a float32 sum of 768 terms
+    # is off by up to RED_RTOL * sqrt(768) of its largest term, which for the few rows whose terms nearly cancel
+    # (|sum| down to 2e-4 here, terms up to 1) is large next to the sum whatever the order of the additions
     got = out["r"].numpy().astype(np.float64)
     scale = np.abs(r).max(1, keepdims=True)
     err = np.abs(got - r) / scale
-    assert err.max() <= RED_RTOL * math.sqrt(768) * 10, err.max()
+    cancel = np.abs(r0).max(1, keepdims=True) / np.abs(r0.sum(1, keepdims=True))
+    tol = RED_RTOL * math.sqrt(768) * (10 + cancel)
+    assert (err <= tol).all(), float((err / tol).max())
+    assert np.median(err.max(1)) <= RED_RTOL * math.sqrt(768), "the typical row is far inside the bound"
 
 
 def test_manip_loop_runs_to_the_iteration_limit(hip_device):

@@ -51,7 +51,8 @@ def test_fused_elw_small(rows, cols, hip_device):
     compare_outputs(got, ref, rules, ("close", 4 * ELW_RTOL))
 
 
-@pytest.mark.parametrize("rows,cols", [(128, 64), (100, 36), (1024, 512), (5, 3), (3, 2048), (2048, 3), (300, 260), (77, 1028)])
+@pytest.mark.parametrize("rows,cols", [(128, 64), (100, 36), (1024, 512), (5, 3), (3, 2048), (2048, 3), (300, 260), (77, 1028),
+                                       (4100, 4100)])   # the pass with riding sums walks two rows per wavefront; ragged in both directions
 def test_reductions_small(rows, cols, hip_device):
     print(f"[case] reductions {rows}x{cols}", flush=True)
     got, ref = _both(lambda d: W.reductions(d, rows, cols, seed=2), hip_device)
