@@ -264,8 +264,10 @@ def main():
         t0 = time.perf_counter()
         p5.run()
         ms5 = (time.perf_counter() - t0) * 1e3
+        k5 = profile_once(p5)
+        spin_up(p5)
         print(json.dumps({"metric": "tensor manipulation + data-dependent loop, one run", "value": ms5, "unit": "ms",
-                          "kernels": profile_once(p5)}))
+                          "kernels": k5, "stage_after_spin_up": profile(p5, 5)}))
         return
     if args.workload == "attention":
         print(json.dumps(dict(measure_attention(dev), metric="multi-head attention forward, fp32")))
@@ -344,12 +346,20 @@ def main():
             # kernels' rates are cache rates, not HBM rates
             k["GBps"] = k["bytes"] / (k["avg_ms"] * 1e-3) / 1e9
             k["memory"] = "LLC-resident" if k["launches"] > 1 else "HBM"
+        # The gather stage again, the way every other kernel here is timed (clocks settled, several launches): the
+        # run above follows an upload, during which the compute units idle.  Runs of the resident program repeat the
+        # stage on the same inputs; the loop after it finds its counter at the limit and does not iterate.
+        spin_up(p5)
+        stage = [k for k in profile(p5, 5) if k["bytes"] > 1e8 and not k["kernel"].startswith("reduce")]
         extra["manip_loop"] = {"ms_total": ms5, "kernels": k5,
                                "gather_stage": {"algorithmic_bytes": 150994944 + 301989888, "note": "the gathered regions of p and q read "
-                                                "once (151 MB), r and the kept copy of the gathered tensor written (151 MB each)",
+                                                "once (151 MB), r and the kept copy of the gathered tensor written (151 MB each); "
+                                                "ms: average of 5 launches after the clocks have settled (ms_first_run: the "
+                                                "single launch right after the upload)",
                                                 "traffic": TRAFFIC_BYTES["manip_loop"]["gather_stage"],
-                                                "moved_bytes": sum(k["bytes"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce")),
-                                                "ms": sum(k["avg_ms"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce"))}}
+                                                "moved_bytes": sum(k["bytes"] for k in stage),
+                                                "ms": sum(k["avg_ms"] for k in stage),
+                                                "ms_first_run": sum(k["avg_ms"] for k in k5 if k["launches"] == 1 and k["bytes"] > 1e8 and not k["kernel"].startswith("reduce"))}}
         p5.close()
         # config 4: dense MLP training
         extra["mlp_train"] = measure_mlp(dev, args.mlp_iters)
