@@ -395,6 +395,14 @@ struct Gen {
         return has_lane;
     }
 
+    // A load under a predicate (an element of another concat piece, or outside a slice) is issued unconditionally at
+    // index 0 of the same buffer and its value replaced by 0: a load under a condition becomes a branch, and a branch
+    // keeps the loads behind it from being issued before the ones in front have returned.
+    static std::string guarded_load(const std::string& name, const std::string& pred, const std::string& buf, const std::string& index) {
+        return strf("const float %su = %s[%s ? (%s) : 0]; const float %s = %s ? %su : 0.0f;", name.c_str(), buf.c_str(), pred.c_str(),
+                    index.c_str(), name.c_str(), pred.c_str(), name.c_str());
+    }
+
     Val load(const Node* n, const Aff& idx, const std::string& pred) {
         const bool plane = !pred.empty() && pred_lane[pred];
         std::string key = "L" + std::to_string(n->id) + "@" + aff_key(idx) + "?" + pred;
@@ -424,21 +432,22 @@ struct Gen {
         }
         if (!ilane && !plane) {
             if (pred.empty()) emit(false, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
-            else emit(false, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
+            else emit(false, guarded_load(name, pred, bp, aff_str(idx)));
             v = {name, false};
         } else if (!plane && vectorizable(idx)) {
             Aff base = idx;
             for (auto it2 = base.t.begin(); it2 != base.t.end(); ++it2)
                 if (it2->first == lane_atom) { base.t.erase(it2); break; }
-            std::string addr = nt ? strf("__builtin_nontemporal_load((const float4_t*)(%s + %s))", bp.c_str(), aff_str(base).c_str())
-                                  : strf("*(const float4_t*)(%s + %s)", bp.c_str(), aff_str(base).c_str());
+            const std::string at = pred.empty() ? aff_str(base) : strf("(%s ? (%s) : 0)", pred.c_str(), aff_str(base).c_str());
+            std::string addr = nt ? strf("__builtin_nontemporal_load((const float4_t*)(%s + %s))", bp.c_str(), at.c_str())
+                                  : strf("*(const float4_t*)(%s + %s)", bp.c_str(), at.c_str());
             if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
-            else emit(false, strf("float4_t %sv = {0.f, 0.f, 0.f, 0.f}; if (%s) %sv = %s;", name.c_str(), pred.c_str(), name.c_str(), addr.c_str()));
+            else emit(false, strf("float4_t %sv = %s; if (!(%s)) %sv = float4_t{0.f, 0.f, 0.f, 0.f};", name.c_str(), addr.c_str(), pred.c_str(), name.c_str()));
             emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
             v = {name + "[" + atoms[lane_atom].name + "]", true};
         } else {
             if (pred.empty()) emit(true, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
-            else emit(true, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
+            else emit(true, guarded_load(name, pred, bp, aff_str(idx)));
             v = {name, true};
         }
         val_memo[key] = v;
@@ -870,22 +879,38 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
         else src += strf("    const %s c%zu = bid %% %lld%s;\n    bid /= %lld%s;\n", it, d, (long long)shape[d], sfx.c_str(), (long long)shape[d], sfx.c_str());
     }
     // staging: lane = row within the tile, so that a wavefront reads one 256-byte run of the operand per column
-    src += "#pragma unroll 2\n    for (unsigned k = 0; k < 16u; ++k) {\n";
+    // All 16 loads of a thread are issued before the first value is parked: the loads are unconditional (an element
+    // outside the tensor or the operand's piece reads index 0 and is replaced by 0 afterwards), because a load under
+    // a condition becomes a branch with a wait behind it, and the 16 memory latencies of a block then add up (that
+    // version ran at 0.60 of the HBM peak with every wavefront waiting 88 % of its life).
+    for (auto& st : g.staged) src += strf("    float sv%d[16];\n", st.slot);
+    src += "#pragma unroll\n    for (unsigned k = 0; k < 16u; ++k) {\n";
     src += "        const unsigned lj = tid & 63u, li = (tid >> 6) + 4u * k;\n";
     src += strf("        const %s %s = row0 + lj;\n        const %s ii = col0 + li;\n", it, rowv.c_str(), it);
     src += strf("        const %s %s = ii >> 2;\n        const %s j = ii & 3u;\n", it, colv.c_str(), it);
     src += strf("        const bool inside = %s < %lld%s && ii < %lld%s;\n", rowv.c_str(), (long long)Rws, sfx.c_str(), (long long)I, sfx.c_str());
     src += join(g.index_code, "        ");
     for (auto& st : g.staged) {
-        src += strf("        { float v = 0.0f; if (inside%s%s) v = %s[%s]; tile%d[li][lj] = v; }\n", st.pred.empty() ? "" : " && ",
-                    st.pred.c_str(), st.param.c_str(), st.index.c_str(), st.slot);
+        src += strf("        { const bool ok = inside%s%s; const float v = %s[ok ? (%s) : 0]; sv%d[k] = ok ? v : 0.0f; }\n",
+                    st.pred.empty() ? "" : " && ", st.pred.c_str(), st.param.c_str(), st.index.c_str(), st.slot);
     }
+    src += "    }\n";
+    src += "#pragma unroll\n    for (unsigned k = 0; k < 16u; ++k) {\n";
+    for (auto& st : g.staged) src += strf("        tile%d[(tid >> 6) + 4u * k][tid & 63u] = sv%d[k];\n", st.slot, st.slot);
     src += "    }\n    __syncthreads();\n";
     // compute: a thread owns four adjacent columns of four rows of the tile
     src += "    const unsigned lc = tid & 15u, lr = tid >> 4;\n";
-    src += "#pragma unroll 1\n    for (unsigned k = 0; k < 4u; ++k) {\n";
-    src += strf("        const %s %s = row0 + lr + 16u * k;\n        const %s %s = (col0 >> 2) + lc;\n", it, rowv.c_str(), it, colv.c_str());
-    src += strf("        if (%s >= %lld%s || %s >= %lld%s) continue;\n", rowv.c_str(), (long long)Rws, sfx.c_str(), colv.c_str(), (long long)(I / 4), sfx.c_str());
+    // the four rows' values are computed first and stored afterwards: a result may share its buffer with an operand,
+    // so the compiler cannot move the next row's loads above this row's stores by itself, and the rows' memory
+    // latencies would add up
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("    float keep%zu[4][4];\n", i);
+    src += strf("    %s at[4];\n    bool live[4];\n", it);
+    src += "#pragma unroll\n    for (unsigned k = 0; k < 4u; ++k) {\n";
+    // (a row or column quad beyond the edge works on the last valid one instead and is not stored: no branch)
+    src += strf("        const %s row_k = row0 + lr + 16u * k, quad_k = (col0 >> 2) + lc;\n", it);
+    src += strf("        live[k] = row_k < %lld%s && quad_k < %lld%s;\n", (long long)Rws, sfx.c_str(), (long long)(I / 4), sfx.c_str());
+    src += strf("        const %s %s = row_k < %lld%s ? row_k : %lld%s;\n        const %s %s = quad_k < %lld%s ? quad_k : %lld%s;\n", it, rowv.c_str(),
+                (long long)Rws, sfx.c_str(), (long long)(Rws - 1), sfx.c_str(), it, colv.c_str(), (long long)(I / 4), sfx.c_str(), (long long)(I / 4 - 1), sfx.c_str());
     src += join(g.codeA, "        ");
     for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("        float w%zu[4];\n", i);
     src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
@@ -896,9 +921,13 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
     std::string lin = "c0";
     for (size_t d = 1; d < nd; ++d)
         lin = strf("(%s * %lld%s + c%zu)", lin.c_str(), (long long)(d + 1 == nd ? I / 4 : shape[d]), sfx.c_str(), d);
-    src += strf("        const %s t4 = %s;\n", it, lin.c_str());
+    src += strf("        at[k] = %s;\n", lin.c_str());
     for (size_t i = 0; i < spec.outputs.size(); ++i)
-        src += "        " + store4_stmt(strf("w%zu", i), strf("o%zu + t4 * 4u", i), N >= nontemporal_min_elems()) + "\n";
+        src += strf("#pragma unroll\n        for (int j = 0; j < 4; ++j) keep%zu[k][j] = w%zu[j];\n", i, i);
+    src += "    }\n";
+    src += "#pragma unroll\n    for (unsigned k = 0; k < 4u; ++k) {\n        if (!live[k]) continue;\n";
+    for (size_t i = 0; i < spec.outputs.size(); ++i)
+        src += "        " + store4_stmt(strf("keep%zu[k]", i), strf("o%zu + at[k] * 4u", i), N >= nontemporal_min_elems()) + "\n";
     src += "    }\n}\n";
     k.source = src;
     k.buffer_args = order;
