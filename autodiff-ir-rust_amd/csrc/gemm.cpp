@@ -31,8 +31,8 @@ std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry, 
         }
         s += m + "\n";
     }
-    s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n#define SPLITK %d\n#define GROUPED %d\n", cfg.a_kcontig ? 1 : 0,
-              cfg.b_kcontig ? 1 : 0, cfg.edge ? 1 : 0, cfg.split_k ? 1 : 0, cfg.grouped ? 1 : 0);
+    s += strf("#define A_KCONTIG %d\n#define B_KCONTIG %d\n#define EDGE %d\n#define EDGE_VEC %d\n#define SPLITK %d\n#define GROUPED %d\n", cfg.a_kcontig ? 1 : 0,
+              cfg.b_kcontig ? 1 : 0, cfg.edge ? 1 : 0, cfg.edge && cfg.edge_vec ? 1 : 0, cfg.split_k ? 1 : 0, cfg.grouped ? 1 : 0);
     if (cfg.grouped) {
         // one parameter triple per problem slot, and the (wave-uniform) choice among them by blockIdx.y
         std::string params, pick = "switch (blockIdx.y) {";
@@ -63,6 +63,38 @@ std::string gemm_kernel_source(const GemmConfig& cfg, const std::string& entry, 
 #define B_LOADS (BN * BK / 4 / NT)      /* float4 loads of the B tile per thread */
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+// 128 bits of an operand that is only known to be 4-byte aligned (an odd leading dim or offset): still one
+// global_load_dwordx4, which the hardware splits where it crosses a cache line
+typedef float4_t float4_ua __attribute__((aligned(4)));
+
+#if EDGE
+// Four operand elements p[off + j * step], j = 0..3, of which the first `valid` (any integer; <= 0: none) exist; the
+// others read as 0.  `step` is the operand's unit stride (the four run along its contiguous dim).  With EDGE_VEC
+// (the operands' contiguous extents are at least 4) a thread whose
+// four elements all exist takes them with one 128-bit load, as the kernel without EDGE does, and only the threads on
+// the ragged rim fall back to single elements.  The common load sits under no condition (a thread of the rim reads
+// the operand's first elements there, and an element that does not exist is read at the first element and replaced),
+// so that the loads of a tile are in flight together.  With EDGE_VEC the kernel calls this only for the last,
+// ragged k-tile and for quads that straddle the end of M or N: everywhere else a row or column beyond the product
+// is replaced by one inside it (what it contributes to is never stored) and the load is the plain 128-bit one.
+static __device__ __forceinline__ float4_t edge_load4(const float* p, long long off, long long step, long long valid) {
+    float4_t v;
+#if EDGE_VEC
+    const bool whole = valid >= 4;
+    v = *(const float4_ua*)(p + (whole ? off : 0));
+    if (!whole)
+#endif
+    {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool ok = j < valid;
+            const float x = p[ok ? off + j * step : 0];
+            v[j] = ok ? x : 0.0f;
+        }
+    }
+    return v;
+}
+#endif
 
 // A is [M,K] with element strides (a_sm, a_sk); B is [K,N] with (b_sk, b_sn); C dense [M,N].
 // A_KCONTIG: a_sk == 1 (else a_sm == 1).  B_KCONTIG: b_sk == 1 (else b_sn == 1).
@@ -155,13 +187,9 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
             const unsigned kq = tid & 3u, mr = (tid >> 2) + (NT / 4) * i;
             const long long m = bm + mr, k = k0 + 4 * kq;
 #if EDGE
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (m < M) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (k + j < k_hi) v[j] = A[m * a_sm + (k + j) * a_sk];
-            }
-            ra[i] = v;
+            // rows beyond M only feed rows of the product that are never stored: they read the last row instead
+            if (EDGE_VEC && k0 + BK <= k_hi) ra[i] = *(const float4_ua*)(A + min(m, M - 1) * a_sm + k);
+            else ra[i] = edge_load4(A, m * a_sm + k * a_sk, a_sk, m < M ? k_hi - k : 0);
 #else
             ra[i] = *(const float4_t*)(A + m * a_sm + k);
 #endif
@@ -169,13 +197,10 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
             const unsigned mq = tid % (BM / 4), kr = tid / (BM / 4) + (NT / (BM / 4)) * i;
             const long long m = bm + 4 * mq, k = k0 + kr;
 #if EDGE
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (k < k_hi) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (m + j < M) v[j] = A[(m + j) * a_sm + k * a_sk];
-            }
-            ra[i] = v;
+            // a quad of rows that lies wholly beyond M reads the last whole quad instead; one that straddles M is
+            // taken element by element
+            if (EDGE_VEC && k0 + BK <= k_hi && (m + 4 <= M || m >= M)) ra[i] = *(const float4_ua*)(A + k * a_sk + min(m, (M - 4) & ~3ll));
+            else ra[i] = edge_load4(A, m * a_sm + k * a_sk, a_sm, k < k_hi ? M - m : 0);
 #else
             ra[i] = *(const float4_t*)(A + k * a_sk + m);
 #endif
@@ -189,13 +214,8 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
             const unsigned kq = tid & 3u, nr = (tid >> 2) + (NT / 4) * i;
             const long long n = bn + nr, k = k0 + 4 * kq;
 #if EDGE
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (n < N) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (k + j < k_hi) v[j] = B[(k + j) * b_sk + n * b_sn];
-            }
-            rb[i] = v;
+            if (EDGE_VEC && k0 + BK <= k_hi) rb[i] = *(const float4_ua*)(B + min(n, N - 1) * b_sn + k);
+            else rb[i] = edge_load4(B, k * b_sk + n * b_sn, b_sk, n < N ? k_hi - k : 0);
 #else
             rb[i] = *(const float4_t*)(B + n * b_sn + k);
 #endif
@@ -203,13 +223,8 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
             const unsigned nq = tid % (BN / 4), kr = tid / (BN / 4) + (NT / (BN / 4)) * i;
             const long long n = bn + 4 * nq, k = k0 + kr;
 #if EDGE
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (k < k_hi) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (n + j < N) v[j] = B[k * b_sk + (n + j) * b_sn];
-            }
-            rb[i] = v;
+            if (EDGE_VEC && k0 + BK <= k_hi && (n + 4 <= N || n >= N)) rb[i] = *(const float4_ua*)(B + k * b_sk + min(n, (N - 4) & ~3ll));
+            else rb[i] = edge_load4(B, k * b_sk + n * b_sn, b_sn, k < k_hi ? N - n : 0);
 #else
             rb[i] = *(const float4_t*)(B + k * b_sk + n);
 #endif

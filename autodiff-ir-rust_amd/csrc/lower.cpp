@@ -45,11 +45,16 @@ extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy(
     float* dst = out + b0 * ob0 + b1 * ob1 + b2 * ob2;
     const unsigned tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;
     const long long u0 = tu * 64, v0 = tv * 64;
-#pragma unroll 4
-    for (unsigned r = ty; r < 64u; r += 4u) {
-        const long long u = u0 + tx, v = v0 + r;
-        if (u < U && v < V) tile[r][tx] = src[v * in_sv + u];
+    // all 16 loads are issued before the first value is parked (an element beyond the edge reads the view's first
+    // element instead: a load under a condition would be a branch with a wait behind it)
+    float q[16];
+#pragma unroll
+    for (unsigned i = 0; i < 16u; ++i) {
+        const long long u = u0 + tx, v = v0 + ty + 4u * i;
+        q[i] = src[(u < U && v < V) ? v * in_sv + u : 0];
     }
+#pragma unroll
+    for (unsigned i = 0; i < 16u; ++i) tile[ty + 4u * i][tx] = q[i];
     __syncthreads();
 #pragma unroll 4
     for (unsigned r = ty; r < 64u; r += 4u) {
@@ -76,13 +81,16 @@ extern "C" __global__ __launch_bounds__(256) void adhip_transpose_copy4(
     float* dst = out + b0 * ob0 + b1 * ob1 + b2 * ob2;
     const unsigned c4 = threadIdx.x & 15u, rr = threadIdx.x >> 4;
     const long long u0 = tu * 64, v0 = tv * 64;
+    f4 q[4];
 #pragma unroll
-    for (unsigned r = rr; r < 64u; r += 16u) {
-        const long long u = u0 + 4 * c4, v = v0 + r;
-        if (u < U && v < V) {
-            const f4 q = *(const f4*)(src + v * in_sv + u);
-            tile[r][4 * c4 + 0] = q.x; tile[r][4 * c4 + 1] = q.y; tile[r][4 * c4 + 2] = q.z; tile[r][4 * c4 + 3] = q.w;
-        }
+    for (unsigned i = 0; i < 4u; ++i) {
+        const long long u = u0 + 4 * c4, v = v0 + rr + 16u * i;
+        q[i] = *(const f4*)(src + ((u < U && v < V) ? v * in_sv + u : 0));
+    }
+#pragma unroll
+    for (unsigned i = 0; i < 4u; ++i) {
+        const unsigned r = rr + 16u * i;
+        tile[r][4 * c4 + 0] = q[i].x; tile[r][4 * c4 + 1] = q[i].y; tile[r][4 * c4 + 2] = q[i].z; tile[r][4 * c4 + 3] = q[i].w;
     }
     __syncthreads();
 #pragma unroll
@@ -2509,10 +2517,18 @@ struct Lowerer {
         tref_affine2d(n->in[0], a);
         tref_affine2d(n->in[1], b);
         const int64_t M = n->shape[0], N = n->shape[1], K = n->in[0].shape[1];
-        const int64_t a_ld = a.s1 == 1 ? a.s0 : a.s1, b_ld = b.s0 == 1 ? b.s1 : b.s0;
-        const bool unaligned = (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
-        key = {M, N, K, a.s0, a.s1, b.s0, b.s1, unaligned ? 1 : 0};
+        key = {M, N, K, a.s0, a.s1, b.s0, b.s1, dot_alignment(a, b, M, N, K)};
         return true;
+    }
+
+    // 0: both operands are 16-byte aligned line by line and k is a multiple of the tile depth (the kernel without
+    // bounds checks, if M and N fit the tile as well); 1: not so, but a line of either operand holds at least four
+    // elements (128-bit reads of whatever alignment, single elements on the ragged rim); 2: single elements only
+    static int dot_alignment(const Affine2D& a, const Affine2D& b, int64_t M, int64_t N, int64_t K) {
+        const bool a_k = a.s1 == 1, b_k = b.s0 == 1;
+        const int64_t a_ld = a_k ? a.s0 : a.s1, b_ld = b_k ? b.s1 : b.s0;
+        if ((a_k ? K : M) < 4 || (b_k ? K : N) < 4) return 2;
+        return ((a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4) || (K % 16)) ? 1 : 0;
     }
 
     template <class ReadsNode, class KeepsEpilogue>
@@ -2651,6 +2667,7 @@ struct Lowerer {
         pl.bn_tile = cfg.bm == 64 ? 64 : 128;
         if (cfg.bm == 128 && blocks128 < 512 && splits_for(blocks128) == 1) { pl.bn_tile = 64; cfg.bn = 64; }
         cfg.edge = key[7] || (M % cfg.bm) || (N % pl.bn_tile);
+        cfg.edge_vec = key[7] != 2;
         const int64_t blocks = ((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile) * cnt;
         const int64_t want = small_whole ? 1 : splits_for(blocks);
         if (want > 1) {
@@ -2676,7 +2693,7 @@ struct Lowerer {
         ADHIP_CHECK(cfg.split_k == (partial != nullptr), "internal: split grouped product and its slice buffer disagree");
         ADHIP_CHECK(!partial || numel(partial->shape) == (int64_t)cnt * pl.splits * M * N, "internal: slice buffer of the wrong size");
         std::string entry = strf("adhip_gemm_%c%c_%d%s%s%s_grouped", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
-                                 cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? "_edge" : "", cfg.split_k ? "_splitk" : "");
+                                 cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? (cfg.edge_vec ? "_rim" : "_edge") : "", cfg.split_k ? "_splitk" : "");
         Launch l;
         l.kernel = add_kernel(entry, gemm_kernel_source(cfg, entry), "dot_mfma");
         l.block[0] = cfg.bm == 64 ? 256u : (unsigned)(cfg.bm * 2);
@@ -2808,8 +2825,8 @@ struct Lowerer {
         GemmConfig& cfg = pl.cfg;
         cfg.a_kcontig = a.s1 == 1;
         cfg.b_kcontig = b.s0 == 1;
-        const int64_t a_ld = cfg.a_kcontig ? a.s0 : a.s1, b_ld = cfg.b_kcontig ? b.s1 : b.s0;
-        const bool unaligned = (K % 16) || (a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4);
+        const int alignment = dot_alignment(a, b, M, N, K);
+        const bool unaligned = alignment != 0;
         // the largest block tile that still puts enough blocks on the chip's 256 CUs: 256x128 (8 waves) with at
         // least two blocks per CU, 128x128 with at least one -- counting the ranges k can be cut into (each at
         // least 256 deep; the slices are added afterwards) -- else 64x64, cut the same way.  A block that has a CU
@@ -2827,6 +2844,7 @@ struct Lowerer {
         // one 128x128 block per CU is too few to hide its own latencies: halve the tile's width for two per CU
         if (cfg.bm == 128 && blocks128 < 512 && splits_for(blocks128) == 1) { pl.bn_tile = 64; cfg.bn = 64; }
         cfg.edge = unaligned || (M % cfg.bm) || (N % pl.bn_tile);
+        cfg.edge_vec = alignment != 2;
         const int64_t blocks = ((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile);
         const int64_t want = cfg.bm == 256 ? 1 : splits_for(blocks);
         if (want > 1) {
@@ -2854,7 +2872,7 @@ struct Lowerer {
             const int bn_tile = pl.bn_tile;
             ADHIP_CHECK(!cfg.split_k || (partial && !epi), "internal: split product without its slice buffer");
             std::string entry = strf("adhip_gemm_%c%c_%d%s%s%s", cfg.a_kcontig ? 'k' : 'm', cfg.b_kcontig ? 'k' : 'n', cfg.bm,
-                                     cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? "_edge" : "", cfg.split_k ? "_splitk" : "");
+                                     cfg.bn == 64 && cfg.bm != 64 ? "x64" : "", cfg.edge ? (cfg.edge_vec ? "_rim" : "_edge") : "", cfg.split_k ? "_splitk" : "");
             Launch l;
             if (epi) {
                 // the element-wise group that followed the product runs on the accumulators; every distinct

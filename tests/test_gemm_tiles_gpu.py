@@ -103,3 +103,54 @@ def test_256_tile_epilogue(layout, kind, hip_device):
         y = 1.0 / (1.0 + np.exp2(-(d + bias) / 64.0))
         # |dy/dh| <= 1/64 * 1/4: the product's error is damped; the chain adds a few roundings of its own
         assert_close(hip_device.get_tensor("y").data, y.reshape(-1), tol * scale / 256.0 + 4e-7, "y", scale=1.0)
+
+
+def _operand(cmds, name, rows, cols, rows_contiguous, gapped, rng):
+    """Defines `name` as a [rows, cols] operand and returns it as float64.  `rows_contiguous`: the rows (not the
+    columns) have unit stride.  `gapped`: the operand is every other line of a tensor twice as large, so its leading
+    dim is a multiple of four elements although its contiguous extent is not, and the last 128-bit quad of every line
+    is only partly inside the operand."""
+    lines, run = (cols, rows) if rows_contiguous else (rows, cols)   # memory: `lines` lines of `run` contiguous elements
+    if gapped:
+        full = rng.standard_normal((lines, 2, run), dtype=np.float32)
+        cmds += [IR.CreateMat(full.reshape(-1), [lines, 2, run], name + "_full"), IR.Index(a=name + "_full", index=0, dim=1, res=name + "_m")]
+        mem = full[:, 0, :]
+    else:
+        mem = rng.standard_normal((lines, run), dtype=np.float32)
+        cmds.append(IR.CreateMat(mem.reshape(-1), [lines, run], name + "_m"))
+    if rows_contiguous:
+        cmds.append(IR.Permute(a=name + "_m", p=[1, 0], res=name))
+        return mem.T.astype(np.float64)
+    cmds.append(IR.Contigious(a=name + "_m", res=name) if False else IR.View(a=name + "_m", target_dim=[rows, cols], res=name))
+    return mem.astype(np.float64)
+
+
+@pytest.mark.parametrize("layout", ["kn", "kk", "mn", "mk"])
+@pytest.mark.parametrize("shape", [(200, 136, 100, False, "rim"),     # multiples of 4 that fit no tile: 128-bit loads, checked rim
+                                   (130, 70, 50, True, "rim"),        # aligned leading dims, extents end inside a quad
+                                   (520, 300, 1030, True, "rim"),     # the same with k cut into slices
+                                   (2100, 2100, 260, False, "128x64_rim"), (2050, 4100, 130, True, "128_rim"),   # the larger tiles
+                                   (203, 131, 77, False, "rim"),      # nothing aligned: 128-bit loads that start at any element
+                                   (2051, 2303, 35, False, "rim"),
+                                   (700, 900, 2, False, None), (515, 3, 300, False, None),   # lines of fewer than four elements: single loads
+                                   (1, 4096, 64, False, None), (4096, 1, 64, False, None)])
+def test_ragged_products(layout, shape, hip_device):
+    """Products whose extents fit no tile, in the four operand layouts: the kernel variant with 128-bit loads inside
+    and checked single elements on the rim, and the variant with single elements only."""
+    m, n, k, gapped, variant = shape
+    print(f"[case] ragged product {m}x{n}x{k} layout {layout} gapped {gapped}", flush=True)
+    rng = np.random.default_rng(m * 7 + n * 3 + k + sum(map(ord, layout)))
+    cmds = []
+    a64 = _operand(cmds, "a", m, k, layout[0] == "m", gapped, rng)
+    b64 = _operand(cmds, "b", k, n, layout[1] == "k", gapped, rng)
+    cmds += [IR.DotProduct(a="a", b="b", res="c"), IR.EX()]
+    proc = IR.IRProcedure("main", cmds)
+    if variant and m > 1 and n > 1:
+        names = _kernels(proc, ["c"])
+        assert names and all(("_" + variant) in x for x in names), names
+    hip_device.execute(proc, {"c"})
+    got = hip_device.get_tensor("c")
+    assert got.dim == [m, n]
+    ref = a64 @ b64
+    scale = float((np.abs(a64) @ np.abs(b64)).max())
+    assert_close(got.data, ref.reshape(-1), RED_RTOL * math.sqrt(k), f"c ({layout})", scale=scale)
