@@ -706,8 +706,9 @@ ElwBody elw_body(const ElwKernelSpec& spec, const std::set<const Node*>& members
 // walks.  That is 1 until the partial sums would exceed 1024 rows -- except for passes that move few streams (at most
 // three of: results stored, full-size operands read), where a block's closing steps (the sums across the wavefront,
 // the 16 rows through LDS) weigh more against its streaming: two rows per wavefront then, if that still leaves eight
-// blocks per CU.  Measured on 16384 x 4096 with one operand, one result, row and column sums: 103 -> 100 us a step;
-// on the 3-read + 4-write pass over 8192 x 8192 two rows per wavefront cost 4 % instead.
+// blocks per CU.  Measured on 16384 x 4096 with one operand, one result, row and column sums: 103 -> 96 us a step
+// (three and four rows: 98 and 100); on the 3-read + 4-write pass over 8192 x 8192 two rows per wavefront cost 1.5 %
+// instead.
 static int64_t elw_colsum_rows_per_wave(int64_t rows, int64_t cols, int streams) {
     const int64_t base = std::max<int64_t>(1, (rows + 16 * 1024 - 1) / (16 * 1024));
     if (base == 1 && streams <= 3 && ((cols / 4 + 63) / 64) * ((rows + 31) / 32) >= 2048) return 2;
@@ -760,31 +761,66 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
     src += "    if (guard && *guard == 0) return;\n";
     if (!spec.colsums.empty()) src += "    __shared__ float4_t part[2][16][64];\n";
     src += "    const unsigned lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;\n";
-    src += strf("    const %s c1 = (%s)blockIdx.x * 64u + lane;\n", it, it);
-    src += strf("    const bool col_ok = c1 < %lld%s;\n", (long long)(C / 4), sfx);
+    src += strf("    const %s %s = (%s)blockIdx.x * 64u + lane;\n", it, (K >= 2 && K <= 4) ? "c1_raw" : "c1", it);
+    src += strf("    const bool col_ok = %s < %lld%s;\n", (K >= 2 && K <= 4) ? "c1_raw" : "c1", (long long)(C / 4), sfx);
     for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("    float cs%zu[4] = {0.f, 0.f, 0.f, 0.f};\n", i);
-    if (K == 1) src += strf("    {\n        const %s c0 = (%s)blockIdx.y * 16u + wv;\n", it, it);
-    else src += strf("%s\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n",
-                     K <= 2 ? "#pragma unroll" : "#pragma unroll 1", (long long)K, it, it, (long long)(16 * K), sfx);
-    for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("        float rs%zu = 0.f;\n", i);
-    src += strf("        if (col_ok && c0 < %lld%s) {\n", (long long)R, sfx);
-    src += join(g.codeA, "            ");
-    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            float w%zu[4];\n", i);
-    src += "#pragma unroll\n            for (int j = 0; j < 4; ++j) {\n";
-    src += join(g.codeB, "                ");
-    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("                w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
-    for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("                cs%zu[j] += %s;\n", i, b.cs_exprs[i].c_str());
-    for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("                rs%zu += %s;\n", i, b.rs_exprs[i].c_str());
-    src += "            }\n";
-    for (size_t i = 0; i < spec.outputs.size(); ++i)
-        src += "            " + store4_stmt(strf("w%zu", i), strf("o%zu + (c0 * %lld%s + c1 * 4u)", i, (long long)C, sfx), nt_out) + "\n";
-    src += "        }\n";
-    // a wavefront's run of a row: lanes outside the columns hold 0; one value per (row, run)
-    for (size_t i = 0; i < spec.rowsums.size(); ++i) {
-        src += strf("        rs%zu = wave_sum(rs%zu);\n", i, i);
-        src += strf("        if (lane == 0u && c0 < %lld%s) r%zu[c0 * %lld%s + blockIdx.x] = rs%zu;\n", (long long)R, sfx, i, (long long)runs, sfx, i);
+    if (K >= 2 && K <= 4) {
+        // A few rows per wavefront, in two phases: all rows' operands are loaded and everything is computed, then all
+        // rows are stored.  A result may share its buffer with an operand, so the compiler cannot move a later
+        // row's loads above an earlier row's stores by itself; and the rows are clamped to the last one rather than
+        // skipped, because loads under a condition would not be issued together either.
+        for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("    float keep%zu[%lld][4];\n", i, (long long)K);
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("    float rsk%zu[%lld];\n", i, (long long)K);
+        src += strf("    const %s c1 = col_ok ? c1_raw : %lld%s;\n", it, (long long)(C / 4 - 1), sfx);
+        src += strf("#pragma unroll\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n", (long long)K);
+        src += strf("        const %s row = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n", it, it, (long long)(16 * K), sfx);
+        src += strf("        const bool live = col_ok && row < %lld%s;\n", (long long)R, sfx);
+        src += strf("        const %s c0 = row < %lld%s ? row : %lld%s;\n", it, (long long)R, sfx, (long long)(R - 1), sfx);
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("        float rs%zu = 0.f;\n", i);
+        src += join(g.codeA, "        ");
+        src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+        src += join(g.codeB, "            ");
+        for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            keep%zu[kk][j] = %s;\n", i, b.out_exprs[i].c_str());
+        for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("            cs%zu[j] += live ? (%s) : 0.0f;\n", i, b.cs_exprs[i].c_str());
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("            rs%zu += live ? (%s) : 0.0f;\n", i, b.rs_exprs[i].c_str());
+        src += "        }\n";
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("        rsk%zu[kk] = rs%zu;\n", i, i);
+        src += "    }\n";
+        src += strf("#pragma unroll\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n", (long long)K);
+        src += strf("        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n", it, it, (long long)(16 * K), sfx);
+        src += strf("        if (col_ok && c0 < %lld%s) {\n", (long long)R, sfx);
+        for (size_t i = 0; i < spec.outputs.size(); ++i)
+            src += "            " + store4_stmt(strf("keep%zu[kk]", i), strf("o%zu + (c0 * %lld%s + c1 * 4u)", i, (long long)C, sfx), nt_out) + "\n";
+        src += "        }\n";
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) {
+            src += strf("        const float rs%zu = wave_sum(rsk%zu[kk]);\n", i, i);
+            src += strf("        if (lane == 0u && c0 < %lld%s) r%zu[c0 * %lld%s + blockIdx.x] = rs%zu;\n", (long long)R, sfx, i, (long long)runs, sfx, i);
+        }
+        src += "    }\n";
+    } else {
+        if (K == 1) src += strf("    {\n        const %s c0 = (%s)blockIdx.y * 16u + wv;\n", it, it);
+        else src += strf("%s\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n        const %s c0 = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n",
+                         K <= 2 ? "#pragma unroll" : "#pragma unroll 1", (long long)K, it, it, (long long)(16 * K), sfx);
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("        float rs%zu = 0.f;\n", i);
+        src += strf("        if (col_ok && c0 < %lld%s) {\n", (long long)R, sfx);
+        src += join(g.codeA, "            ");
+        for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("            float w%zu[4];\n", i);
+        src += "#pragma unroll\n            for (int j = 0; j < 4; ++j) {\n";
+        src += join(g.codeB, "                ");
+        for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("                w%zu[j] = %s;\n", i, b.out_exprs[i].c_str());
+        for (size_t i = 0; i < spec.colsums.size(); ++i) src += strf("                cs%zu[j] += %s;\n", i, b.cs_exprs[i].c_str());
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) src += strf("                rs%zu += %s;\n", i, b.rs_exprs[i].c_str());
+        src += "            }\n";
+        for (size_t i = 0; i < spec.outputs.size(); ++i)
+            src += "            " + store4_stmt(strf("w%zu", i), strf("o%zu + (c0 * %lld%s + c1 * 4u)", i, (long long)C, sfx), nt_out) + "\n";
+        src += "        }\n";
+        // a wavefront's run of a row: lanes outside the columns hold 0; one value per (row, run)
+        for (size_t i = 0; i < spec.rowsums.size(); ++i) {
+            src += strf("        rs%zu = wave_sum(rs%zu);\n", i, i);
+            src += strf("        if (lane == 0u && c0 < %lld%s) r%zu[c0 * %lld%s + blockIdx.x] = rs%zu;\n", (long long)R, sfx, i, (long long)runs, sfx, i);
+        }
+        src += "    }\n";
     }
-    src += "    }\n";
     // the 16 wavefronts' sums, added in wavefront order; two sums per round through LDS (wavefronts 0 and 1 add them)
     for (size_t i0 = 0; i0 < spec.colsums.size(); i0 += 2) {
         const size_t cnt = std::min<size_t>(2, spec.colsums.size() - i0);
