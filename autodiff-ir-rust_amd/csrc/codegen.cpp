@@ -1282,13 +1282,40 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         src += "    const unsigned chunk = blockIdx.y;\n";
         src += strf("    const bool row_ok = x < %lld%s;\n", (long long)V, wide ? "ull" : "u");
         src += strf("    float acc[%d];\n#pragma unroll\n    for (int j = 0; j < %d; ++j) acc[j] = %s;\n", vec, vec, ident);
-        if (chunks == 1) {
+        // A row that is also stored, in a few iterations per lane: every iteration's loads are issued and the values
+        // computed before the first one is stored.  A stored value may share its buffer with an operand, so the
+        // compiler has to keep each iteration's loads behind the previous iteration's store, and the iterations'
+        // memory latencies would add up (the body of the data-dependent loop of the manipulation workload is such a
+        // kernel: three iterations).  Iterations past the end of the row are clamped to its last element, not skipped.
+        const int64_t iters = (RV + T - 1) / T;
+        const bool phased = side && chunks == 1 && vec == 4 && iters * (int64_t)b.side_exprs.size() <= 8;
+        if (phased) {
+            const char* it_t = g.idx_t();
+            for (size_t i = 0; i < b.side_exprs.size(); ++i) src += strf("    float keep%zu[%lld][4];\n", i, (long long)iters);
+            src += "    if (row_ok) {\n";
+            src += strf("#pragma unroll\n    for (unsigned it = 0; it < %lldu; ++it) {\n", (long long)iters);
+            src += strf("        const %s yv_raw = lane + it * %du;\n        const bool live = yv_raw < %lldu;\n        const %s yv = live ? yv_raw : %lldu;\n",
+                        it_t, T, (long long)RV, it_t, (long long)(RV - 1));
+            src += join(g.codeA, "        ");
+            src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+            src += join(g.codeB, "            ");
+            for (size_t i = 0; i < b.side_exprs.size(); ++i) src += strf("            keep%zu[it][j] = %s;\n", i, b.side_exprs[i].c_str());
+            src += strf("            if (live) acc[j] = %s;\n        }\n    }\n", comb("acc[j]", b.value).c_str());
+            src += strf("#pragma unroll\n    for (unsigned it = 0; it < %lldu; ++it) {\n        const %s yv = lane + it * %du;\n        if (yv < %lldu) {\n",
+                        (long long)iters, it_t, T, (long long)RV);
+            for (size_t i = 0; i < b.side_exprs.size(); ++i)
+                src += "            " + store4_stmt(strf("keep%zu[it]", i), strf("w%zu + (%lldu * x + 4u * yv)", i, (long long)R), V * R >= nontemporal_min_elems()) + "\n";
+            src += "        }\n    }\n    }\n";
+        }
+        if (phased) {
+        } else if (chunks == 1) {
             // constant trip count: the loads of several iterations can be in flight together
             src += strf("    if (row_ok)\n#pragma unroll 8\n    for (%s yv = lane; yv < %lldu; yv += %du) {\n", g.idx_t(), (long long)RV, T);
         } else {
             src += strf("    const %s y_end = min((%s)(chunk + 1u) * %lldu, (%s)%lldu);\n", g.idx_t(), g.idx_t(), (long long)CH, g.idx_t(), (long long)RV);
             src += strf("    if (row_ok)\n#pragma unroll 4\n    for (%s yv = (%s)chunk * %lldu + lane; yv < y_end; yv += %du) {\n", g.idx_t(), g.idx_t(), (long long)CH, T);
         }
+        if (!phased) {
         src += join(g.codeA, "        ");
         if (side)
             for (size_t i = 0; i < b.side_exprs.size(); ++i) src += strf("        float sv%zu[4];\n", i);
@@ -1302,6 +1329,7 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
             for (size_t i = 0; i < b.side_exprs.size(); ++i)
                 src += "        " + store4_stmt(strf("sv%zu", i), strf("w%zu + (%lldu * x + 4u * yv)", i, (long long)R), V * R >= nontemporal_min_elems()) + "\n";
         src += "    }\n";
+        }
         if (vec == 4) src += "    float s = " + comb4("acc[0]", "acc[1]", "acc[2]", "acc[3]") + ";\n";
         else src += "    float s = acc[0];\n";
         std::string epilogue;
