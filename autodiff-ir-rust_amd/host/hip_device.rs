@@ -13,7 +13,8 @@
 //! does not use: it lowers the IR itself, behind the C ABI.  `ir_callback` runs after `EX` has been appended and before
 //! anything else (reference src/core/autodiff.rs:108-114), sees the complete IR and keeps a copy; `execute` serialises
 //! that copy.  The crate calls `to_kernel` before `execute` (src/core/ir.rs:180-198); it panics on `Index` and cannot
-//! express `Concat` for its device, so programs that use them need the one-line bypass described in INTEGRATION.md.
+//! express `Concat` for its device, so programs that use them need `ir_b_execute` to skip `to_kernel` for a device that
+//! lowers by itself (one `if` around that call, keyed on a new defaulted trait method such as `lowers_ir() -> bool`).
 
 use std::cell::RefCell;
 use std::ffi::{c_char, c_int, c_void, CStr, CString};
