@@ -7,14 +7,21 @@ from adhip import autodiff
 from adhip.core import concat, constant, dot
 
 
-def random_program(dev, seed: int, n_ops: int = 24):
+def random_program(dev, seed: int, n_ops: int = 24, scale: int = 1):
+    """`scale` multiplies the two basic extents (4 and 6) of the leaf shapes: at 1 every kernel is a few threads, at 16
+    and beyond the 128-bit element-wise forms, sums riding along with element-wise passes, chunked reductions and the
+    matrix-core products (with extents that fit no tile) come into play.  Leaf values shrink with the scale so that
+    sums over the longer dims stay in the range the small programs have."""
     rng = np.random.default_rng(seed)
     autodiff.set_device(dev)
-    shapes = [[4, 6], [6], [4, 1], [2, 3, 4], [6, 4], [3, 4], [1], [8, 4, 6]]
+    p, q = 4 * scale, 6 * scale
+    shapes = [[p, q], [q], [p, 1], [2, q // 2, p], [q, p], [q // 2, p], [1], [8, p, q]]
+    amp = 1.5 / np.sqrt(scale)
+    limit = 4096 * scale * scale
     pool = []
     leaves = []
     for sh in shapes:
-        data = rng.uniform(-1.5, 1.5, size=int(np.prod(sh))).astype(np.float32)
+        data = rng.uniform(-amp, amp, size=int(np.prod(sh))).astype(np.float32)
         t = autodiff.tensor(data, sh)
         pool.append(t)
         leaves.append(t)
@@ -63,7 +70,8 @@ def random_program(dev, seed: int, n_ops: int = 24):
                 out = a.permute([int(x) for x in rng.permutation(len(a.dim()))])
             elif kind == 6:
                 n = int(np.prod(a.dim()))
-                divs = [d for d in range(1, n + 1) if n % d == 0]
+                divs = [d for d in range(1, int(n ** 0.5) + 1) if n % d == 0]
+                divs = sorted(divs + [n // d for d in divs if d * d != n])
                 d0 = divs[rng.integers(len(divs))]
                 out = a.view([d0, n // d0])
             elif kind == 7 and len(a.dim()) >= 1:
@@ -89,7 +97,7 @@ def random_program(dev, seed: int, n_ops: int = 24):
                 out = a.t().contigious() if rng.integers(2) else a.t()
         except (AssertionError, RuntimeError):
             out = None
-        if out is not None and int(np.prod(out.dim())) <= 4096 and int(np.prod(out.dim())) > 0:
+        if out is not None and int(np.prod(out.dim())) <= limit and int(np.prod(out.dim())) > 0:
             pool.append(out)
 
     # a scalar target that touches several recent values, then forward and backward

@@ -228,6 +228,29 @@ def test_random_programs_match_oracle(seed, hip_device):
         assert_close(got[k].data, rv.data, tol, f"seed {seed} {k}")
 
 
+@pytest.mark.parametrize("scale,seed", [(16, s) for s in range(12)] + [(16, 23)] + [(48, s) for s in range(6)])
+def test_random_programs_at_scale(scale, seed, hip_device):
+    """The same generator with every leaf extent multiplied (tests/fuzz_programs.py, `scale`): tensors of 10^4 to 10^6
+    elements, so the kernels are the 128-bit element-wise forms, sums riding along, chunked reductions and matrix-core
+    products with extents that fit no tile.  A value is compared relative to its own largest element, but not below
+    1 % of the largest element of any output: gradients of one-element leaves are sums of thousands of terms of the
+    program's magnitude that may cancel (seed 23 at scale 16: -2.5e-3 from terms of order 1)."""
+    print(f"[case] fuzz scale {scale} seed {seed}", flush=True)
+    from fuzz_programs import random_program
+    got = random_program(hip_device, seed, scale=scale)
+    oracle = OracleDevice()
+    ref = random_program(oracle, seed, scale=scale)
+    assert set(got) == set(ref)
+    tol = RED_RTOL * math.sqrt(oracle.max_terms) * 2
+    finite = [np.asarray(rv.data)[np.isfinite(rv.data)] for rv in ref.values()]
+    largest = max((float(np.max(np.abs(f))) for f in finite if f.size), default=1.0)
+    for k, rv in ref.items():
+        assert got[k].dim == rv.dim, f"{k}: dim {got[k].dim} vs {rv.dim}"
+        f = np.asarray(rv.data)[np.isfinite(rv.data)]
+        own = float(np.max(np.abs(f))) if f.size else 0.0
+        assert_close(got[k].data, rv.data, tol, f"scale {scale} seed {seed} {k}", scale=max(own, 1e-2 * largest))
+
+
 def _run_ir(dev, cmds, keep):
     from adhip import ir as IR
     proc = IR.IRProcedure("main", list(cmds) + [IR.EX()])
