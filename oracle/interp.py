@@ -178,6 +178,16 @@ class OracleDevice(Device):
         self.shape: Dict[str, List[int]] = {}     # id -> logical shape (shape tracker)
         self.const: Dict[str, np.float32] = {}    # id -> inline constant
         self.alias: Dict[str, tuple] = {}         # id -> data command back to another id
+        # a view of a view of ... is resolved recursively (_value); the caller side spells a slice of n lines as n
+        # Index commands joined by a chain of n - 1 Concats, so chains run to thousands of links on larger tensors
+        limit = sys.getrecursionlimit()
+        sys.setrecursionlimit(max(limit, 20000))
+        try:
+            self._execute(proc, dep_ids)
+        finally:
+            sys.setrecursionlimit(limit)
+
+    def _execute(self, proc: IR.IRProcedure, dep_ids: Iterable[str]) -> None:
         try:
             self._run(proc)
         except _Exit:
