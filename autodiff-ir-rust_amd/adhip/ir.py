@@ -316,58 +316,79 @@ class IRBase:
 # wire format
 # --------------------------------------------------------------------------------------
 
+_ENCODED: dict = {}   # string -> its length-prefixed UTF-8 form (ids repeat all over a program)
+_DIMS_STRUCT: dict = {}   # rank -> struct for "<I rank Q..."
+
+
 def _s(out: bytearray, s: str) -> None:
-    b = s.encode("utf-8")
-    out += struct.pack("<I", len(b))
+    b = _ENCODED.get(s)
+    if b is None:
+        e = s.encode("utf-8")
+        if len(_ENCODED) > 200000:
+            _ENCODED.clear()
+        b = _ENCODED[s] = struct.pack("<I", len(e)) + e
     out += b
 
 
 def _dims(out: bytearray, dims) -> None:
-    out += struct.pack("<I", len(dims))
-    for d in dims:
-        out += struct.pack("<Q", int(d))
+    n = len(dims)
+    st = _DIMS_STRUCT.get(n)
+    if st is None:
+        st = _DIMS_STRUCT[n] = struct.Struct("<I%dQ" % n)
+    out += st.pack(n, *[int(d) for d in dims])
+
+
+_THREE_IDS = frozenset((T_ELW_MULTIPLY, T_ELW_ADD, T_DOT_PRODUCT))
+_TWO_IDS_SO = frozenset((T_ELW_MULTIPLY_EQ, T_ELW_ADD_EQ))
+_TWO_IDS_AR = frozenset((T_EQUAL_ZERO, T_MORE_ZERO, T_LESS_ZERO, T_SUM, T_MAX, T_CONTIGIOUS,
+                         T_EXP2, T_LOG2, T_SIN, T_RECIP, T_SQRT))
+_PACK_QQ = struct.Struct("<QQ").pack
+_PACK_Q = struct.Struct("<Q").pack
+_PACK_I = struct.Struct("<I").pack
+_PACK_F = struct.Struct("<f").pack
 
 
 def _proc(out: bytearray, proc: IRProcedure, keepalive: list, offsets: Optional[list] = None) -> None:
     _s(out, proc.id)
-    out += struct.pack("<I", len(proc.main))
+    out += _PACK_I(len(proc.main))
     for cmd in proc.main:
         t = cmd.tag
         out.append(t)
-        if t == T_CREATE_MAT:
-            arr = np.ascontiguousarray(cmd.contents, dtype=np.float32).reshape(-1)
+        if t in _THREE_IDS:
+            _s(out, cmd.a); _s(out, cmd.b); _s(out, cmd.res)
+        elif t in _TWO_IDS_AR:
+            _s(out, cmd.a); _s(out, cmd.res)
+        elif t in _TWO_IDS_SO:
+            _s(out, cmd.s); _s(out, cmd.o)
+        elif t == T_CREATE_MAT:
+            arr = cmd.contents
+            if not (isinstance(arr, np.ndarray) and arr.dtype == np.float32 and arr.ndim == 1 and arr.flags.c_contiguous):
+                arr = np.ascontiguousarray(arr, dtype=np.float32).reshape(-1)
             keepalive.append(arr)
             _s(out, cmd.id)
             _dims(out, cmd.dim)
             if offsets is not None:
                 offsets.append(len(out))
-            out += struct.pack("<QQ", arr.ctypes.data if arr.size else 0, arr.size)
+            out += _PACK_QQ(arr.ctypes.data if arr.size else 0, arr.size)
         elif t == T_CREATE_CONSTANT:
-            out += struct.pack("<f", np.float32(cmd.contents))
+            out += _PACK_F(np.float32(cmd.contents))
             _s(out, cmd.id)
             _dims(out, cmd.dim)
-        elif t in (T_ELW_MULTIPLY, T_ELW_ADD, T_DOT_PRODUCT):
-            _s(out, cmd.a); _s(out, cmd.b); _s(out, cmd.res)
-        elif t in (T_ELW_MULTIPLY_EQ, T_ELW_ADD_EQ):
-            _s(out, cmd.s); _s(out, cmd.o)
-        elif t in (T_EQUAL_ZERO, T_MORE_ZERO, T_LESS_ZERO, T_SUM, T_MAX, T_CONTIGIOUS,
-                   T_EXP2, T_LOG2, T_SIN, T_RECIP, T_SQRT):
-            _s(out, cmd.a); _s(out, cmd.res)
         elif t == T_VIEW:
             _s(out, cmd.a); _dims(out, cmd.target_dim); _s(out, cmd.res)
         elif t == T_INDEX:
-            _s(out, cmd.a); out += struct.pack("<QQ", cmd.index, cmd.dim); _s(out, cmd.res)
+            _s(out, cmd.a); out += _PACK_QQ(cmd.index, cmd.dim); _s(out, cmd.res)
         elif t == T_CONCAT:
-            _s(out, cmd.a); _s(out, cmd.b); out += struct.pack("<Q", cmd.dim); _s(out, cmd.res)
+            _s(out, cmd.a); _s(out, cmd.b); out += _PACK_Q(cmd.dim); _s(out, cmd.res)
         elif t == T_PERMUTE:
             _s(out, cmd.a); _dims(out, cmd.p); _s(out, cmd.res)
         elif t == T_BROADCAST:
-            _s(out, cmd.a); out += struct.pack("<QQ", cmd.dim, cmd.r); _s(out, cmd.res)
+            _s(out, cmd.a); out += _PACK_QQ(cmd.dim, cmd.r); _s(out, cmd.res)
         elif t == T_WHILE:
             _s(out, cmd.conditional_var)
             _proc(out, cmd.block, keepalive, offsets)
         elif t == T_IF:
-            out += struct.pack("<I", len(cmd.conditions))
+            out += _PACK_I(len(cmd.conditions))
             for cond, p in cmd.conditions:
                 _s(out, cond)
                 _proc(out, p, keepalive, offsets)
