@@ -125,16 +125,10 @@ extern "C" __global__ void adhip_flag(int* __restrict__ flags, int slot, int par
 // `tiles` rows of its dense partial buffer [tiles][cols] (cols a multiple of 4), in one launch (blockIdx.y picks the
 // sum).  A block is 16 four-column groups x 64 row groups; the row groups are combined through LDS by a tree of fixed
 // shape, so the result does not depend on scheduling.
-extern "C" __global__ __launch_bounds__(1024) void adhip_colsum_finalize(
-    const int* __restrict__ guard, float* o0, float* o1, float* o2, float* o3, const float* p0, const float* p1,
-    const float* p2, const float* p3, long long tiles, long long cols) {
+static __device__ __forceinline__ void adhip_colsum_finalize_body(float* o, const float* p, long long tiles, long long cols) {
     typedef float f4 __attribute__((ext_vector_type(4)));
-    if (guard && *guard == 0) return;
     __shared__ f4 part[64][16];
     const unsigned lx = threadIdx.x & 15u, ly = threadIdx.x >> 4;
-    const unsigned which = blockIdx.y;
-    const float* p = which == 0 ? p0 : (which == 1 ? p1 : (which == 2 ? p2 : p3));
-    float* o = which == 0 ? o0 : (which == 1 ? o1 : (which == 2 ? o2 : o3));
     const long long x = ((long long)blockIdx.x * 16 + lx) * 4;
     const bool ok = x < cols;
     f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -149,6 +143,51 @@ extern "C" __global__ __launch_bounds__(1024) void adhip_colsum_finalize(
     if (ly < 4) part[ly][lx] = (part[ly][lx] + part[ly + 4][lx]) + (part[ly + 8][lx] + part[ly + 12][lx]);
     __syncthreads();
     if (ly == 0 && ok) *(f4*)(o + x) = (part[0][lx] + part[1][lx]) + (part[2][lx] + part[3][lx]);
+}
+
+extern "C" __global__ __launch_bounds__(1024) void adhip_colsum_finalize(
+    const int* __restrict__ guard, float* o0, float* o1, float* o2, float* o3, const float* p0, const float* p1,
+    const float* p2, const float* p3, long long tiles, long long cols) {
+    if (guard && *guard == 0) return;
+    const unsigned which = blockIdx.y;
+    const float* p = which == 0 ? p0 : (which == 1 ? p1 : (which == 2 ? p2 : p3));
+    float* o = which == 0 ? o0 : (which == 1 ? o1 : (which == 2 ? o2 : o3));
+    adhip_colsum_finalize_body(o, p, tiles, cols);
+}
+
+// Second pass of both kinds of sums that rode along with one element-wise kernel, in one launch.  Blocks
+// [0, col_blocks) along x add column partials as adhip_colsum_finalize does (blockIdx.y picks one of up to four sums);
+// the blocks beyond add the run sums of rows: a thread per row, out[row] = the row's `runs` consecutive partial sums
+// added in ascending order (blockIdx.y picks one of up to two sums).
+extern "C" __global__ __launch_bounds__(1024) void adhip_sums_finalize(
+    const int* __restrict__ guard, float* o0, float* o1, float* o2, float* o3, const float* p0, const float* p1,
+    const float* p2, const float* p3, long long tiles, long long cols, long long n_cols, float* r0, float* r1,
+    const float* q0, const float* q1, long long rows, long long runs, long long n_rows, long long col_blocks) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    if (guard && *guard == 0) return;
+    const unsigned which = blockIdx.y;
+    if ((long long)blockIdx.x >= col_blocks) {
+        if (which >= n_rows) return;
+        const long long row = ((long long)blockIdx.x - col_blocks) * 1024 + threadIdx.x;
+        if (row >= rows) return;
+        const float* src = (which ? q1 : q0) + row * runs;
+        float sum = 0.0f;
+        if ((runs & 3) == 0) {
+#pragma unroll 4
+            for (long long j = 0; j < runs; j += 4) {
+                const f4 v = *(const f4*)(src + j);
+                sum = (((sum + v.x) + v.y) + v.z) + v.w;
+            }
+        } else {
+            for (long long j = 0; j < runs; ++j) sum += src[j];
+        }
+        (which ? r1 : r0)[row] = sum;
+        return;
+    }
+    if (which >= n_cols) return;
+    const float* p = which == 0 ? p0 : (which == 1 ? p1 : (which == 2 ? p2 : p3));
+    float* o = which == 0 ? o0 : (which == 1 ? o1 : (which == 2 ? o2 : o3));
+    adhip_colsum_finalize_body(o, p, tiles, cols);
 }
 
 // out[i] = slices[0][i] + slices[1][i] + ... in that order, i < n; four elements per thread when n allows.
@@ -288,7 +327,7 @@ struct Lowerer {
     std::map<std::string, int> kernel_by_source;
     int kernel_counter = 0;
     std::map<std::pair<int, int>, int> layered_kernels;
-    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sum_slices = -1, fixed_sum_slices_grouped = -1;
+    int fixed_copy = -1, fixed_dot = -1, fixed_transpose = -1, fixed_transpose4 = -1, fixed_finalize = -1, fixed_sums_finalize = -1, fixed_sum_slices = -1, fixed_sum_slices_grouped = -1;
     int dot_epilogue_counter = 0;
     int cur_guard = -1;  // flag slot guarding the block being lowered, or -1
     // The device-predicated loop whose body is being lowered: its block, predicate id and flag.  The last region of the
@@ -1197,8 +1236,7 @@ struct Lowerer {
         bool dot_store = true;     // ... and whether the product itself is still written
         // row sums riding along with an element-wise group: per sum the [rows][runs] partial buffer, the node that
         // stands for the second pass over it, and that pass's kernel
-        std::vector<Node*> row_partials, row_fins;
-        std::vector<GeneratedKernel> row_kernels;
+        std::vector<Node*> row_partials;
         // what the group's kernel was generated from, should it be generated again with a loop flag to latch
         int spec_kind = 0;  // 1: elw_spec + spec_members, 2: red_spec
         ElwKernelSpec elw_spec;
@@ -1953,20 +1991,13 @@ struct Lowerer {
                     gks[g].extra_nodes.push_back(partial);
                 }
                 for (auto& rs : G.rowsums) {
-                    // one partial sum per (row, run of 256 columns), added by a generated row reduction over [rows][runs]
+                    // one partial sum per (row, run of 256 columns), added by the fixed second-pass kernel
                     const int64_t runs = elw_rowsum_runs(G.cs_cols);
                     Node* S = rs.second;
                     Node* partial = new_node(Op::COPY, Shape{G.cs_rows, runs}, {}, S->name + ".runs", 0.f, false);
                     partial->root = true;
-                    Node* fin = new_node(Op::SUM, Shape{G.cs_rows}, {tr_node(partial, Shape{G.cs_rows, runs})}, S->name, 0.f, false);
-                    fin->root = true;
                     spec.rowsums.push_back({rs.first, partial});
-                    ReduceKernelSpec s2;
-                    s2.node = fin;
-                    s2.name = name + strf("_rs%zu", gks[g].row_fins.size());
-                    gks[g].row_kernels.push_back(gen_reduce_kernel(s2, 1));
                     gks[g].row_partials.push_back(partial);
-                    gks[g].row_fins.push_back(fin);
                 }
                 gks[g].k = gen_elw_kernel(spec, members);
                 gks[g].spec_kind = 1;
@@ -2358,21 +2389,50 @@ struct Lowerer {
             GeneratedKernel& k = gks[g].k;
             if (G.kind == Group::ELW && G.rides()) {
                 launch_generated(k);
-                for (size_t i = 0; i < G.rowsums.size(); ++i) {
-                    gks[g].row_fins[i]->buffer = G.rowsums[i].second->buffer;
-                    launch_generated(gks[g].row_kernels[i]);
-                }
-                // one launch of the fixed second-pass kernel per four sums
-                if (fixed_finalize < 0) fixed_finalize = add_kernel("adhip_colsum_finalize", fixed_kernels_source(), "colsum_finalize");
                 const int64_t tiles = elw_colsum_tiles(G.cs_rows, G.cs_cols, G.cs_streams);
-                for (size_t i0 = 0; i0 < G.colsums.size(); i0 += 4) {
+                auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: riding sum without buffer"); q.buf = x->buffer; return q; };
+                auto I = [&](int64_t v) { Arg q; q.kind = Arg::I64; q.iv = v; return q; };
+                size_t cols_done = 0;
+                // row sums: one launch of the fixed second-pass kernel per two of them, which also takes up to four of
+                // the column sums along
+                for (size_t r0 = 0; r0 < G.rowsums.size(); r0 += 2) {
+                    const size_t nr = std::min<size_t>(2, G.rowsums.size() - r0);
+                    const size_t nc = std::min<size_t>(4, G.colsums.size() - cols_done);
+                    const int64_t runs = elw_rowsum_runs(G.cs_cols);
+                    const int64_t col_blocks = nc ? (G.cs_cols + 63) / 64 : 0, row_blocks = (G.cs_rows + 1023) / 1024;
+                    if (fixed_sums_finalize < 0) fixed_sums_finalize = add_kernel("adhip_sums_finalize", fixed_kernels_source(), "sums_finalize");
+                    Launch lf;
+                    lf.kernel = fixed_sums_finalize;
+                    lf.block[0] = 1024;
+                    lf.grid[0] = (unsigned)(col_blocks + row_blocks);
+                    lf.grid[1] = (unsigned)std::max(nr, std::max<size_t>(nc, 1));
+                    // unused slots repeat a valid buffer: the kernel never touches them
+                    for (size_t j = 0; j < 4; ++j) lf.args.push_back(nc ? B(G.colsums[cols_done + std::min(j, nc - 1)].second) : B(G.rowsums[r0].second));
+                    for (size_t j = 0; j < 4; ++j) lf.args.push_back(nc ? B(gks[g].extra_nodes[cols_done + std::min(j, nc - 1)]) : B(gks[g].row_partials[r0]));
+                    lf.args.push_back(I(tiles));
+                    lf.args.push_back(I(G.cs_cols));
+                    lf.args.push_back(I((int64_t)nc));
+                    for (size_t j = 0; j < 2; ++j) lf.args.push_back(B(G.rowsums[r0 + std::min(j, nr - 1)].second));
+                    for (size_t j = 0; j < 2; ++j) lf.args.push_back(B(gks[g].row_partials[r0 + std::min(j, nr - 1)]));
+                    lf.args.push_back(I(G.cs_rows));
+                    lf.args.push_back(I(runs));
+                    lf.args.push_back(I((int64_t)nr));
+                    lf.args.push_back(I(col_blocks));
+                    lf.label = k.entry + "_rs0";
+                    lf.bytes = 4.0 * (double)nc * (double)G.cs_cols * (double)(tiles + 1) + 4.0 * (double)nr * (double)G.cs_rows * (double)(runs + 1);
+                    lf.flops = (double)nc * (double)G.cs_cols * (double)tiles + (double)nr * (double)G.cs_rows * (double)runs;
+                    push_launch(out, lf, "sums_finalize");
+                    cols_done += nc;
+                }
+                // the column sums that are left: one launch of the fixed second-pass kernel per four sums
+                if (cols_done < G.colsums.size() && fixed_finalize < 0) fixed_finalize = add_kernel("adhip_colsum_finalize", fixed_kernels_source(), "colsum_finalize");
+                for (size_t i0 = cols_done; i0 < G.colsums.size(); i0 += 4) {
                     const size_t cnt = std::min<size_t>(4, G.colsums.size() - i0);
                     Launch lf;
                     lf.kernel = fixed_finalize;
                     lf.block[0] = 1024;
                     lf.grid[0] = (unsigned)((G.cs_cols + 63) / 64);
                     lf.grid[1] = (unsigned)cnt;
-                    auto B = [&](Node* x) { Arg q; q.kind = Arg::BUF; ADHIP_CHECK(x->buffer >= 0, "internal: column sum without buffer"); q.buf = x->buffer; return q; };
                     for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(G.colsums[i0 + std::min(j, cnt - 1)].second));
                     for (size_t j = 0; j < 4; ++j) lf.args.push_back(B(gks[g].extra_nodes[i0 + std::min(j, cnt - 1)]));
                     Arg t; t.kind = Arg::I64; t.iv = tiles; lf.args.push_back(t);
