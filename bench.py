@@ -26,13 +26,13 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 # copy kernel of known size (the summaries under profiles/ give the runs).  These counters sit in front of the 256 MiB
 # last-level cache, so they bound HBM traffic from above.  Valid for the full-size workloads only.
 TRAFFIC_BYTES = {
-    # 2 x 393277.1 KiB fetched + 1081824.3 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
-    "fused_elw": {"elw_colsum": int((2 * 393277.1 + 1081824.3) * 1024)},
-    # the one pass of configs[2] (dx with row and column sums riding along): 2 x 131353.0 KiB fetched + 278575.5 KiB
+    # 2 x 393276.6 KiB fetched + 1081844.6 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
+    "fused_elw": {"elw_colsum": int((2 * 393276.6 + 1081844.6) * 1024)},
+    # the one pass of configs[2] (dx with row and column sums riding along): 2 x 131353.0 KiB fetched + 278574.5 KiB
     # written (dx, the [512][4096] partial column sums, one run sum per row and 256 columns)
-    "reductions": {"elw_colsum": int((2 * 131353.0 + 278575.5) * 1024)},
-    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73764.7 KiB fetched + 294912.0 KiB written
-    "manip_loop": {"gather_stage": int((2 * 73764.7 + 294912.0) * 1024)},
+    "reductions": {"elw_colsum": int((2 * 131353.0 + 278574.5) * 1024)},
+    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73766.4 KiB fetched + 294912.0 KiB written
+    "manip_loop": {"gather_stage": int((2 * 73766.4 + 294912.0) * 1024)},
 }
 
 
