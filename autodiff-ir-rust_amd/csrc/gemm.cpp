@@ -98,8 +98,9 @@ static __device__ __forceinline__ float4_t edge_load4(const float* p, long long 
 
 // A is [M,K] with element strides (a_sm, a_sk); B is [K,N] with (b_sk, b_sn); C dense [M,N].
 // A_KCONTIG: a_sk == 1 (else a_sm == 1).  B_KCONTIG: b_sk == 1 (else b_sn == 1).
-// EDGE: M, N or K is not a multiple of the tile, or an operand is not 16-byte aligned; every
-// access is then bounds-checked and scalar.
+// EDGE: M, N or K is not a multiple of the tile, or an operand is not 16-byte aligned.  Stores are bounds-checked;
+// loads go through edge_load4 where an element may not exist (all of them without EDGE_VEC; with it, only the last
+// ragged k-tile and quads that straddle the end of M or N).
 // SPLITK: the block at blockIdx.y multiplies only k in [y*k_chunk, (y+1)*k_chunk) and writes slice y of a
 // [gridDim.y][M][N] buffer; the caller adds the slices in a fixed order.  For products whose output alone gives
 // too few blocks to hide the latency of the operand loads.
