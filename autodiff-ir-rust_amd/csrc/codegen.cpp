@@ -395,14 +395,6 @@ struct Gen {
         return has_lane;
     }
 
-    // A load under a predicate (an element of another concat piece, or outside a slice) is issued unconditionally at
-    // index 0 of the same buffer and its value replaced by 0: a load under a condition becomes a branch, and a branch
-    // keeps the loads behind it from being issued before the ones in front have returned.
-    static std::string guarded_load(const std::string& name, const std::string& pred, const std::string& buf, const std::string& index) {
-        return strf("const float %su = %s[%s ? (%s) : 0]; const float %s = %s ? %su : 0.0f;", name.c_str(), buf.c_str(), pred.c_str(),
-                    index.c_str(), name.c_str(), pred.c_str(), name.c_str());
-    }
-
     Val load(const Node* n, const Aff& idx, const std::string& pred) {
         const bool plane = !pred.empty() && pred_lane[pred];
         std::string key = "L" + std::to_string(n->id) + "@" + aff_key(idx) + "?" + pred;
@@ -432,22 +424,22 @@ struct Gen {
         }
         if (!ilane && !plane) {
             if (pred.empty()) emit(false, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
-            else emit(false, guarded_load(name, pred, bp, aff_str(idx)));
+            else emit(false, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
             v = {name, false};
         } else if (!plane && vectorizable(idx)) {
             Aff base = idx;
             for (auto it2 = base.t.begin(); it2 != base.t.end(); ++it2)
                 if (it2->first == lane_atom) { base.t.erase(it2); break; }
-            const std::string at = pred.empty() ? aff_str(base) : strf("(%s ? (%s) : 0)", pred.c_str(), aff_str(base).c_str());
+            const std::string at = aff_str(base);
             std::string addr = nt ? strf("__builtin_nontemporal_load((const float4_t*)(%s + %s))", bp.c_str(), at.c_str())
                                   : strf("*(const float4_t*)(%s + %s)", bp.c_str(), at.c_str());
             if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
-            else emit(false, strf("float4_t %sv = %s; if (!(%s)) %sv = float4_t{0.f, 0.f, 0.f, 0.f};", name.c_str(), addr.c_str(), pred.c_str(), name.c_str()));
+            else emit(false, strf("float4_t %sv = {0.f, 0.f, 0.f, 0.f}; if (%s) %sv = %s;", name.c_str(), pred.c_str(), name.c_str(), addr.c_str()));
             emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
             v = {name + "[" + atoms[lane_atom].name + "]", true};
         } else {
             if (pred.empty()) emit(true, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
-            else emit(true, guarded_load(name, pred, bp, aff_str(idx)));
+            else emit(true, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));
             v = {name, true};
         }
         val_memo[key] = v;

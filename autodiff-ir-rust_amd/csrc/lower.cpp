@@ -298,6 +298,7 @@ struct Group {
     std::vector<std::pair<Node*, Node*>> rowsums;
     int64_t cs_rows = 0, cs_cols = 0;  // the [rows, cols] view of the iteration space both kinds of sums refer to
     int cs_streams = 8;                // full-size streams of a pass with sums (ElwKernelSpec::streams)
+    int64_t loads = 0;                 // places where the members' folded expressions read memory (bounds the kernel's size)
     bool rides() const { return !colsums.empty() || !rowsums.empty(); }
     std::vector<std::pair<Node*, Node*>> riders() const {
         std::vector<std::pair<Node*, Node*>> r = colsums;
@@ -1252,6 +1253,7 @@ struct Lowerer {
         std::map<Node*, std::set<Node*>> folded_in;          // per root: folded nodes it evaluates at its own index
         std::vector<Group> groups;                           // kernels, in launch order
         std::map<Node*, int> group_of;
+        std::map<Node*, int64_t> inline_loads;               // per value: places where its folded expression reads memory
         std::map<Node*, std::string> home_of;                // wanted node -> id
         std::vector<GroupKernels> gks;                       // per group: generated code
         std::vector<std::map<Node*, bool>> greads;           // per group: reads, for hazard analysis
@@ -1373,6 +1375,7 @@ struct Lowerer {
         force_roots(rp);
         if (opt.fuse) plan_transposed_copies(rp);
         keep_shared_values(rp);
+        cut_long_expressions(rp);
         form_groups(rp);
         if (opt.fuse) {
             attach_column_sums(rp);
@@ -1574,6 +1577,43 @@ struct Lowerer {
     }
 
     // ---- 5. group roots into kernels
+    // ---- 4b. A folded expression may not read memory in more than kMaxInlineLoads places.  Slices spelled as one
+    // Index per line joined by Concats, summed up by a backward pass, fold into expressions with thousands of
+    // predicated loads: the compiler needs minutes for the branches, and a kernel with some three hundred loads was
+    // seen to run out of registers (512 per lane and scratch).  Walking producers first, a value whose expression
+    // would exceed the limit gets a buffer and a kernel of its own, so that its consumers read it as one operand.
+    static constexpr int64_t kMaxInlineLoads = 96;
+    void cut_long_expressions(RegionPlan& rp) {
+        if (!opt.fuse) return;
+        auto& loads = rp.inline_loads;
+        for (Node* n : rp.topo) {
+            if (op_is_leaf(n->op)) continue;
+            int64_t c = 0;
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) { c += in_mem(s) ? 1 : std::max<int64_t>(loads[s], 1); });
+            if (!n->root && op_is_elw(n->op) && c > kMaxInlineLoads && numel(n->shape) > 0) {
+                // the cheaper cut is often one level down: root the largest folded operand first, and this value only
+                // if that is not enough
+                std::vector<std::pair<int64_t, Node*>> parts;
+                for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                    if (!in_mem(s) && op_is_elw(s->op) && numel(s->shape) > 0) parts.push_back({loads[s], s});
+                });
+                std::sort(parts.begin(), parts.end(), [](const std::pair<int64_t, Node*>& a, const std::pair<int64_t, Node*>& b) {
+                    return a.first != b.first ? a.first > b.first : a.second->order < b.second->order;
+                });
+                for (auto& pt : parts) {
+                    if (c <= kMaxInlineLoads) break;
+                    if (pt.second->root || pt.first <= 1) continue;
+                    pt.second->root = true;
+                    c -= pt.first - 1;
+                }
+                if (c > kMaxInlineLoads) {
+                    n->root = true;
+                }
+            }
+            loads[n] = c;
+        }
+    }
+
     void form_groups(RegionPlan& rp) {
         auto& topo = rp.topo;
         auto& reads = rp.reads;
@@ -1592,6 +1632,7 @@ struct Lowerer {
             if (op_is_elw(r->op) && opt.fuse && !r->transpose) {
                 for (int g = (int)groups.size() - 1; g >= 0; --g) {
                     if (groups[g].kind != Group::ELW || groups[g].n != numel(r->shape)) continue;
+                    if (groups[g].loads + rp.inline_loads[r] > 2 * kMaxInlineLoads) continue;  // a kernel's size is bounded too
                     bool ok = true;
                     for (auto& rd : reads[r]) {
                         if (op_is_leaf(rd.first->op)) continue;
@@ -1610,6 +1651,7 @@ struct Lowerer {
                 chosen = (int)groups.size() - 1;
             }
             groups[chosen].members.push_back(r);
+            groups[chosen].loads += rp.inline_loads[r];
             group_of[r] = chosen;
         }
         for (auto& w : rp.wanted) rp.home_of[w.second] = w.first;

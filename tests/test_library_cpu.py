@@ -173,6 +173,26 @@ def test_random_programs_lower_and_compile(seed):
     assert not out["target"].is_none
 
 
+@pytest.mark.parametrize("seed", [301, 343])
+def test_folded_expressions_stay_bounded(seed, monkeypatch):
+    """Slices of long dims (one Index per line, joined by Concats) and the sums of their gradients fold into
+    expressions with thousands of predicated loads unless the lowering cuts them: seed 301 at scale 16 is 24 000
+    commands whose largest kernel would read memory in 5 900 places (minutes of compilation); seed 343 gave a kernel
+    with 300 loads that ran out of registers.  No kernel may read memory in more than 2 x 96 places."""
+    from fuzz_programs import random_program
+    monkeypatch.setenv("ADHIP_DUMP_SOURCE", "1")
+    dev = Capture()
+    random_program(dev, seed, scale=16)
+    text = lower_describe(dev.proc, dev.deps)
+    parts = re.split(r"// ===== (\S+) \[(\w+)\] =====\n", text)
+    assert len(parts) > 3
+    for i in range(1, len(parts), 3):
+        if parts[i + 1] not in ("elw", "elw_colsum", "elw_tiled", "reduce_row", "reduce_row_store", "reduce_col", "merged"):
+            continue
+        loads = len(re.findall(r"\bb\d+\[|\(b\d+ \+ ", parts[i + 2]))
+        assert loads <= (192 if parts[i + 1] != "merged" else 2000), (parts[i], loads)
+
+
 def test_generated_sine_is_accurate_on_the_host(tmp_path, monkeypatch):
     """The sine the generated kernels use is plain float arithmetic (fma, rint, a polynomial), so the very text the
     device compiles can be built for the host and compared with float64 sin: at most 2.5 ulp everywhere, including
