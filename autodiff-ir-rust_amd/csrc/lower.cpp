@@ -1577,40 +1577,50 @@ struct Lowerer {
     }
 
     // ---- 5. group roots into kernels
-    // ---- 4b. A folded expression may not read memory in more than kMaxInlineLoads places.  Slices spelled as one
-    // Index per line joined by Concats, summed up by a backward pass, fold into expressions with thousands of
-    // predicated loads: the compiler needs minutes for the branches, and a kernel with some three hundred loads was
-    // seen to run out of registers (512 per lane and scratch).  Walking producers first, a value whose expression
-    // would exceed the limit gets a buffer and a kernel of its own, so that its consumers read it as one operand.
-    static constexpr int64_t kMaxInlineLoads = 96;
+    // ---- 4b. A folded expression may not read more than kMaxInlineLoads distinct values from memory.  Slices spelled
+    // as one Index per line joined by Concats, summed up by a backward pass, fold into expressions with thousands of
+    // predicated loads of as many operands: the compiler needs minutes for the branches, and kernels of a few hundred
+    // loads use all 512 registers of a lane plus scratch (two such kernels were seen to produce wrong elements).
+    // Walking producers first, a value whose expression would exceed the limit gets a buffer and a kernel of its own
+    // (its largest folded operands first, then itself), so that its consumers read it as one operand.  At 32 operands
+    // a kernel stays below 256 registers and needs no scratch.
+    static constexpr int64_t kMaxInlineLoads = 32;
     void cut_long_expressions(RegionPlan& rp) {
         if (!opt.fuse) return;
-        auto& loads = rp.inline_loads;
+        std::map<Node*, std::vector<Node*>> operands;  // per folded value: the in-memory values its expression reads (sorted)
+        auto gather = [&](Node* n) {
+            std::vector<Node*> u;
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                if (in_mem(s)) u.push_back(s);
+                else { auto& o = operands[s]; u.insert(u.end(), o.begin(), o.end()); }
+            });
+            std::sort(u.begin(), u.end());
+            u.erase(std::unique(u.begin(), u.end()), u.end());
+            return u;
+        };
         for (Node* n : rp.topo) {
             if (op_is_leaf(n->op)) continue;
-            int64_t c = 0;
-            for_each_src(n, [&](Node* s, const Piece&, const TRef&) { c += in_mem(s) ? 1 : std::max<int64_t>(loads[s], 1); });
-            if (!n->root && op_is_elw(n->op) && c > kMaxInlineLoads && numel(n->shape) > 0) {
-                // the cheaper cut is often one level down: root the largest folded operand first, and this value only
-                // if that is not enough
-                std::vector<std::pair<int64_t, Node*>> parts;
+            std::vector<Node*> u = gather(n);
+            if (!n->root && op_is_elw(n->op) && (int64_t)u.size() > kMaxInlineLoads && numel(n->shape) > 0) {
+                std::vector<std::pair<size_t, Node*>> parts;
                 for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
-                    if (!in_mem(s) && op_is_elw(s->op) && numel(s->shape) > 0) parts.push_back({loads[s], s});
+                    if (!in_mem(s) && op_is_elw(s->op) && numel(s->shape) > 0) parts.push_back({operands[s].size(), s});
                 });
-                std::sort(parts.begin(), parts.end(), [](const std::pair<int64_t, Node*>& a, const std::pair<int64_t, Node*>& b) {
-                    return a.first != b.first ? a.first > b.first : a.second->order < b.second->order;
+                std::sort(parts.begin(), parts.end(), [](const std::pair<size_t, Node*>& x, const std::pair<size_t, Node*>& y) {
+                    return x.first != y.first ? x.first > y.first : x.second->order < y.second->order;
                 });
+                parts.erase(std::unique(parts.begin(), parts.end()), parts.end());
                 for (auto& pt : parts) {
-                    if (c <= kMaxInlineLoads) break;
+                    if ((int64_t)u.size() <= kMaxInlineLoads) break;
                     if (pt.second->root || pt.first <= 1) continue;
                     pt.second->root = true;
-                    c -= pt.first - 1;
+                    operands.erase(pt.second);
+                    u = gather(n);
                 }
-                if (c > kMaxInlineLoads) {
-                    n->root = true;
-                }
+                if ((int64_t)u.size() > kMaxInlineLoads) n->root = true;
             }
-            loads[n] = c;
+            rp.inline_loads[n] = (int64_t)u.size();
+            if (!n->root) operands[n] = std::move(u);
         }
     }
 
