@@ -337,6 +337,16 @@ hipFunction_t get_function(Module& m, const std::string& entry) {
     hipFunction_t f;
     HIP_OK(hipModuleGetFunction(&f, m.mod, entry.c_str()));
     m.fns[entry] = f;
+    // A generated kernel that spills registers to scratch memory is far outside what the lowering aims for (it bounds
+    // the operands a kernel reads so that kernels stay below 280 registers), and kernels in that regime have been seen
+    // to compute wrong elements: say so once per kernel (ADHIP_QUIET=1 silences it).
+    int scratch = 0;
+    if (hipFuncGetAttribute(&scratch, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, f) == hipSuccess && scratch > 0) {
+        const char* q = getenv("ADHIP_QUIET");
+        if (!(q && *q == '1')) fprintf(stderr, "adhip: kernel %s spills %d bytes per lane to scratch memory\n", entry.c_str(), scratch);
+    } else {
+        (void)hipGetLastError();
+    }
     return f;
 }
 
