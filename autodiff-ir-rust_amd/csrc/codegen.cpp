@@ -435,8 +435,14 @@ struct Gen {
                                   : strf("*(const float4_t*)(%s + %s)", bp.c_str(), at.c_str());
             if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
             else emit(false, strf("float4_t %sv = {0.f, 0.f, 0.f, 0.f}; if (%s) %sv = %s;", name.c_str(), pred.c_str(), name.c_str(), addr.c_str()));
-            emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
-            v = {name + "[" + atoms[lane_atom].name + "]", true};
+            if (pred.empty()) {
+                emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
+                v = {name + "[" + atoms[lane_atom].name + "]", true};
+            } else {
+                // no array of the four elements here: a select between elements of two such arrays under the loads'
+                // own predicates is turned into a load through a selected address, which puts the arrays into scratch
+                v = {name + "v[" + atoms[lane_atom].name + "]", true};
+            }
         } else {
             if (pred.empty()) emit(true, strf("const float %s = %s[%s];", name.c_str(), bp.c_str(), aff_str(idx).c_str()));
             else emit(true, strf("const float %s = %s ? %s[%s] : 0.0f;", name.c_str(), pred.c_str(), bp.c_str(), aff_str(idx).c_str()));

@@ -298,7 +298,6 @@ struct Group {
     std::vector<std::pair<Node*, Node*>> rowsums;
     int64_t cs_rows = 0, cs_cols = 0;  // the [rows, cols] view of the iteration space both kinds of sums refer to
     int cs_streams = 8;                // full-size streams of a pass with sums (ElwKernelSpec::streams)
-    int64_t loads = 0;                 // places where the members' folded expressions read memory (bounds the kernel's size)
     bool rides() const { return !colsums.empty() || !rowsums.empty(); }
     std::vector<std::pair<Node*, Node*>> riders() const {
         std::vector<std::pair<Node*, Node*>> r = colsums;
@@ -1253,7 +1252,6 @@ struct Lowerer {
         std::map<Node*, std::set<Node*>> folded_in;          // per root: folded nodes it evaluates at its own index
         std::vector<Group> groups;                           // kernels, in launch order
         std::map<Node*, int> group_of;
-        std::map<Node*, int64_t> inline_loads;               // per value: places where its folded expression reads memory
         std::map<Node*, std::string> home_of;                // wanted node -> id
         std::vector<GroupKernels> gks;                       // per group: generated code
         std::vector<std::map<Node*, bool>> greads;           // per group: reads, for hazard analysis
@@ -1577,14 +1575,18 @@ struct Lowerer {
     }
 
     // ---- 5. group roots into kernels
-    // ---- 4b. A folded expression may not read more than kMaxInlineLoads distinct values from memory.  Slices spelled
+    // ---- 4b. A folded expression may not read more than kMaxInlineLoads distinct values from memory, and a kernel
+    // may not name more than kMaxKernelPointers buffers (operands and outputs of all its members).  Slices spelled
     // as one Index per line joined by Concats, summed up by a backward pass, fold into expressions with thousands of
-    // predicated loads of as many operands: the compiler needs minutes for the branches, and kernels of a few hundred
-    // loads use all 512 registers of a lane plus scratch (two such kernels were seen to produce wrong elements).
+    // predicated loads of as many operands: the compiler needs minutes for the branches.  A pointer takes two scalar
+    // registers and the lane mask of every predicate two more, of the 102 a wavefront has: kernels of 60 and more
+    // buffers used all 512 vector registers, kept some 200 scalar registers in lanes of vector registers and spilled
+    // vector registers to scratch on top, and three of them were seen to produce wrong elements.
     // Walking producers first, a value whose expression would exceed the limit gets a buffer and a kernel of its own
-    // (its largest folded operands first, then itself), so that its consumers read it as one operand.  At 32 operands
-    // a kernel stays below 256 registers and needs no scratch.
+    // (its largest folded operands first, then itself), so that its consumers read it as one operand.  Within the
+    // bounds a kernel stays below 300 vector registers, spills none of them and needs no scratch.
     static constexpr int64_t kMaxInlineLoads = 32;
+    static constexpr int64_t kMaxKernelPointers = 40;
     void cut_long_expressions(RegionPlan& rp) {
         if (!opt.fuse) return;
         std::map<Node*, std::vector<Node*>> operands;  // per folded value: the in-memory values its expression reads (sorted)
@@ -1619,10 +1621,22 @@ struct Lowerer {
                 }
                 if ((int64_t)u.size() > kMaxInlineLoads) n->root = true;
             }
-            rp.inline_loads[n] = (int64_t)u.size();
             if (!n->root) operands[n] = std::move(u);
         }
     }
+
+    // the buffers a kernel of this group (with one more member, if given) names: distinct operands, outputs, sums
+    int64_t group_pointers(RegionPlan& rp, const Group& G, Node* extra = nullptr) {
+        std::set<Node*> u;
+        for (Node* m : G.members)
+            for (auto& kv : rp.reads[m]) u.insert(kv.first);
+        if (extra)
+            for (auto& kv : rp.reads[extra]) u.insert(kv.first);
+        return (int64_t)(u.size() + G.members.size() + (extra ? 1 : 0) + G.colsums.size() + G.rowsums.size());
+    }
+    // the pass with sums runs 1024 threads a block, which leaves a lane 128 vector registers: a pass that names more
+    // buffers than this would spill them, so its sums get kernels of their own
+    bool can_carry_sums(RegionPlan& rp, const Group& G) { return group_pointers(rp, G) < 20; }
 
     void form_groups(RegionPlan& rp) {
         auto& topo = rp.topo;
@@ -1642,7 +1656,7 @@ struct Lowerer {
             if (op_is_elw(r->op) && opt.fuse && !r->transpose) {
                 for (int g = (int)groups.size() - 1; g >= 0; --g) {
                     if (groups[g].kind != Group::ELW || groups[g].n != numel(r->shape)) continue;
-                    if (groups[g].loads + rp.inline_loads[r] > 2 * kMaxInlineLoads) continue;  // a kernel's size is bounded too
+                    if (group_pointers(rp, groups[g], r) > kMaxKernelPointers) continue;  // a kernel's size is bounded too
                     bool ok = true;
                     for (auto& rd : reads[r]) {
                         if (op_is_leaf(rd.first->op)) continue;
@@ -1661,7 +1675,6 @@ struct Lowerer {
                 chosen = (int)groups.size() - 1;
             }
             groups[chosen].members.push_back(r);
-            groups[chosen].loads += rp.inline_loads[r];
             group_of[r] = chosen;
         }
         for (auto& w : rp.wanted) rp.home_of[w.second] = w.first;
@@ -1734,7 +1747,7 @@ struct Lowerer {
             int target = -1;
             for (size_t g = 0; g < groups.size() && target < 0; ++g) {
                 Group& G = groups[g];
-                if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
+                if (G.dead || G.kind != Group::ELW || G.n != R * C || !can_carry_sums(rp, G)) continue;
                 if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                 for (Node* m : G.members)
                     if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
@@ -1749,7 +1762,7 @@ struct Lowerer {
                 for (auto& kv : er) ident = ident && kv.second;
                 for (size_t g = 0; ident && g < groups.size() && target < 0; ++g) {
                     Group& G = groups[g];
-                    if (G.dead || G.kind != Group::ELW || G.n != R * C) continue;
+                    if (G.dead || G.kind != Group::ELW || G.n != R * C || !can_carry_sums(rp, G)) continue;
                     if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                     bool all = true;
                     for (auto& kv : er) {
@@ -1805,7 +1818,7 @@ struct Lowerer {
             int target = -1;
             for (size_t g = 0; g < groups.size() && target < 0; ++g) {
                 Group& G = groups[g];
-                if (g == gs || G.dead || G.tiled || G.kind != Group::ELW || G.n != R * C || !G.side.empty()) continue;
+                if (g == gs || G.dead || G.tiled || G.kind != Group::ELW || G.n != R * C || !G.side.empty() || !can_carry_sums(rp, G)) continue;
                 if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                 bool computes = false;
                 for (Node* m : G.members) computes = computes || m == E || folded_in[m].count(E);

@@ -313,12 +313,84 @@ std::map<std::string, std::vector<char>> compile_code_objects(const std::vector<
     return out;
 }
 
+// What the compiler wrote into a code object's metadata note (msgpack) about each kernel's register spills: a kernel
+// with more pointers and values in flight than the 102 scalar / 512 vector registers of a lane hold keeps the rest in
+// lanes of spare vector registers and in scratch memory.  The lowering bounds the pointers of a kernel so that vector
+// registers are not spilled: three generated kernels with 512 vector registers, some 200 spilled scalar registers and
+// spilled vector registers on top computed wrong elements, and none without vector spills did.  The keys of a kernel's map
+// are sorted: .name < .private_segment_fixed_size < .sgpr_spill_count < .vgpr_spill_count.
+struct KernelSpills {
+    std::string name;
+    long scalar = 0, vector = 0, scratch_bytes = 0;
+};
+
+std::vector<KernelSpills> code_object_spills(const std::vector<char>& code) {
+    const std::string blob(code.begin(), code.end());
+    auto key = [](const std::string& k) { return std::string(1, (char)(0xa0 + k.size())) + k; };  // fixstr: all < 32 bytes
+    auto uint_at = [&](size_t p) -> long {
+        if (p >= blob.size()) return -1;
+        const unsigned char b = (unsigned char)blob[p];
+        auto be = [&](size_t n) -> long {
+            if (p + n >= blob.size()) return -1;
+            long v = 0;
+            for (size_t i = 1; i <= n; ++i) v = (v << 8) | (unsigned char)blob[p + i];
+            return v;
+        };
+        if (b < 0x80) return b;
+        if (b == 0xcc) return be(1);
+        if (b == 0xcd) return be(2);
+        if (b == 0xce) return be(4);
+        return -1;
+    };
+    auto str_at = [&](size_t p) -> std::string {
+        if (p >= blob.size()) return "";
+        const unsigned char b = (unsigned char)blob[p];
+        size_t len = 0, at = p + 1;
+        if (b >= 0xa0 && b <= 0xbf) len = b - 0xa0;
+        else if (b == 0xd9 && p + 1 < blob.size()) { len = (unsigned char)blob[p + 1]; at = p + 2; }
+        else if (b == 0xda && p + 2 < blob.size()) { len = ((size_t)(unsigned char)blob[p + 1] << 8) | (unsigned char)blob[p + 2]; at = p + 3; }
+        else return "";
+        return at + len <= blob.size() ? blob.substr(at, len) : "";
+    };
+    const std::string k_name = key(".name"), k_priv = key(".private_segment_fixed_size"), k_s = key(".sgpr_spill_count"),
+                      k_v = key(".vgpr_spill_count");
+    std::vector<KernelSpills> out;
+    for (size_t p = blob.find(k_s); p != std::string::npos; p = blob.find(k_s, p + 1)) {
+        KernelSpills ks;
+        ks.scalar = uint_at(p + k_s.size());
+        const size_t nm = blob.rfind(k_name, p), pv = blob.rfind(k_priv, p), vp = blob.find(k_v, p);
+        if (nm != std::string::npos) ks.name = str_at(nm + k_name.size());
+        if (pv != std::string::npos && (nm == std::string::npos || pv > nm)) ks.scratch_bytes = uint_at(pv + k_priv.size());
+        if (vp != std::string::npos) ks.vector = uint_at(vp + k_v.size());
+        out.push_back(ks);
+    }
+    return out;
+}
+
+// everything: also list kernels that only keep scalar registers in lanes of spare vector registers (the compiler's
+// ordinary answer to many lane masks in flight; costs a few instructions) or use scratch memory without spilling
+// (the library sine's reduction of huge arguments does)
+std::string describe_spills(const std::vector<char>& code, bool everything) {
+    std::string text;
+    for (auto& ks : code_object_spills(code))
+        if (ks.vector > 0 || (everything && (ks.scalar > 0 || ks.scratch_bytes > 0)))
+            text += strf("%s%s (%ld scalar, %ld vector registers spilled, %ld bytes of scratch per lane)", text.empty() ? "" : "; ",
+                         ks.name.c_str(), ks.scalar, ks.vector, ks.scratch_bytes);
+    return text;
+}
+
 std::shared_ptr<Module> compile_module(adhip_ctx* ctx, const std::string& source, const std::vector<char>* code_in = nullptr) {
     auto it = ctx->modules.find(source);
     if (it != ctx->modules.end()) return it->second;
     std::vector<char> code = code_in ? *code_in : compile_code_object(source, ctx->arch);
     auto m = std::make_shared<Module>();
     HIP_OK(hipModuleLoadData(&m->mod, code.data()));
+    // say so once per module when a kernel in it spills vector registers (ADHIP_QUIET=1 silences it)
+    const char* quiet = getenv("ADHIP_QUIET");
+    if (!(quiet && *quiet == '1')) {
+        const std::string spills = describe_spills(code, false);
+        if (!spills.empty()) fprintf(stderr, "adhip: kernel %s\n", spills.c_str());
+    }
     // a long-lived context that keeps seeing new programs does not keep every module it ever loaded: beyond a
     // bound, the ones no live program refers to are unloaded (their code objects stay in the on-disk cache)
     if (ctx->modules.size() >= 1024) {
@@ -337,16 +409,6 @@ hipFunction_t get_function(Module& m, const std::string& entry) {
     hipFunction_t f;
     HIP_OK(hipModuleGetFunction(&f, m.mod, entry.c_str()));
     m.fns[entry] = f;
-    // A generated kernel that spills registers to scratch memory is far outside what the lowering aims for (it bounds
-    // the operands a kernel reads so that kernels stay below 280 registers), and kernels in that regime have been seen
-    // to compute wrong elements: say so once per kernel (ADHIP_QUIET=1 silences it).
-    int scratch = 0;
-    if (hipFuncGetAttribute(&scratch, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, f) == hipSuccess && scratch > 0) {
-        const char* q = getenv("ADHIP_QUIET");
-        if (!(q && *q == '1')) fprintf(stderr, "adhip: kernel %s spills %d bytes per lane to scratch memory\n", entry.c_str(), scratch);
-    } else {
-        (void)hipGetLastError();
-    }
     return f;
 }
 
@@ -1130,6 +1192,12 @@ int adhip_compile_check(const uint8_t* program, size_t program_len, const char* 
             }
         }
         text = strf("%zu kernels compiled, %zu bytes of code objects", plan->kernels.size(), bytes);
+        std::string spills;
+        for (auto& o : objects) {
+            const std::string one = describe_spills(o.second, true);
+            if (!one.empty()) spills += (spills.empty() ? "" : "; ") + one;
+        }
+        if (!spills.empty()) text += "; spilling kernels: " + spills;
     });
     if (rc != 0) text = g_tls_error;
     snprintf(out, out_cap, "%s", text.c_str());
