@@ -108,7 +108,9 @@ int adhip_lower_describe(const uint8_t* program, size_t program_len, const char*
                          char* out, size_t out_cap);
 
 /* Lower and compile every generated kernel with hipRTC for `arch` (default "gfx950") without touching a
- * GPU: the build-time check that the device code is valid.  Writes a one-line summary or the error. */
+ * GPU: the build-time check that the device code is valid.  Writes a one-line summary or the error; the
+ * summary ends with "; spilling kernels: <name> (<n> scalar, <n> vector registers spilled, <n> bytes of scratch
+ * per lane); ..." when the compiler's metadata of a code object records any. */
 int adhip_compile_check(const uint8_t* program, size_t program_len, const char* const* dep_ids, size_t n_dep_ids,
                         const char* arch, char* out, size_t out_cap);
 
