@@ -130,6 +130,7 @@ def test_workloads_lower_and_compile_for_gfx950(name):
     SMALL[name](dev).run()
     rc, msg = _compile_check(dev.proc, dev.deps)
     assert rc == 0, msg
+    assert "spilling kernels" not in msg, msg  # no kernel of a workload spills a register or uses scratch memory
 
 
 def test_counted_loop_is_recognised():
