@@ -365,6 +365,9 @@ struct Gen {
     int buffer_of(const Node* n) {
         auto it = buf_index.find(n);
         if (it != buf_index.end()) return it->second;
+        // the lowering bounds what a kernel reads long before this; a kernel that names hundreds of buffers would
+        // take minutes to compile and could only run by spilling registers
+        ADHIP_CHECK(bufs.size() < 192, "internal: a generated kernel names more than 192 operand buffers");
         GenBuffer b;
         b.node = const_cast<Node*>(n);
         b.param = "b" + std::to_string(bufs.size());

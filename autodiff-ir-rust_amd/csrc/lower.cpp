@@ -336,6 +336,15 @@ struct Lowerer {
     std::string latch_id;
     int latch_slot = -1;
     bool latch_region = false, latch_attached = false;
+    // Straight-line regions are numbered in the order they are lowered; the caller may ask for tighter kernel-size
+    // bounds in some of them (LowerOptions::region_shift).
+    int region_counter = 0, cur_region = -1;
+    int region_shift() const {
+        auto it = opt.region_shift.find(cur_region);
+        return it == opt.region_shift.end() ? 0 : std::min(it->second, 8);
+    }
+    int64_t bound(int v) const { return std::max<int64_t>(2, (int64_t)v >> region_shift()); }
+    bool tight() const { return region_shift() > 0; }
 
     // per region
     std::vector<Node*> rnodes;
@@ -968,11 +977,16 @@ struct Lowerer {
             pos = end;
         }
         auto it = kernel_by_source.find(key);
-        if (it != kernel_by_source.end()) return it->second;
+        if (it != kernel_by_source.end()) {
+            std::vector<int>& rg = plan->kernels[(size_t)it->second].regions;
+            if (std::find(rg.begin(), rg.end(), cur_region) == rg.end()) rg.push_back(cur_region);
+            return it->second;
+        }
         KernelDef d;
         d.entry = entry;
         d.source = source;
         d.kind = kind;
+        d.regions.push_back(cur_region);
         plan->kernels.push_back(std::move(d));
         kernel_by_source[key] = (int)plan->kernels.size() - 1;
         return (int)plan->kernels.size() - 1;
@@ -1250,6 +1264,7 @@ struct Lowerer {
         std::vector<Node*> topo;                             // every needed node, producers first
         std::map<Node*, std::map<Node*, bool>> reads;        // per root: in-memory values it reads (true: element for element only)
         std::map<Node*, std::set<Node*>> folded_in;          // per root: folded nodes it evaluates at its own index
+        std::map<Node*, std::set<uint64_t>> sites;           // per value: the places its expression, evaluated in place, loads from
         std::vector<Group> groups;                           // kernels, in launch order
         std::map<Node*, int> group_of;
         std::map<Node*, std::string> home_of;                // wanted node -> id
@@ -1271,6 +1286,7 @@ struct Lowerer {
     }
 
     void flush_region(const IdSet& live, bool final_region, std::vector<Step>& out) {
+        cur_region = region_counter++;
         const size_t first_step = out.size();
         flush_region_launches(live, final_region, out);
         if (opt.fuse && opt.merge_small) merge_single_block_runs(out, first_step);
@@ -1371,6 +1387,7 @@ struct Lowerer {
             order_nodes(rp);
         }
         force_roots(rp);
+        narrow_references(rp);
         if (opt.fuse) plan_transposed_copies(rp);
         keep_shared_values(rp);
         cut_long_expressions(rp);
@@ -1574,22 +1591,157 @@ struct Lowerer {
         }
     }
 
-    // ---- 5. group roots into kernels
-    // ---- 4b. A folded expression may not read more than kMaxInlineLoads distinct values from memory, and a kernel
-    // may not name more than kMaxKernelPointers buffers (operands and outputs of all its members).  Slices spelled
-    // as one Index per line joined by Concats, summed up by a backward pass, fold into expressions with thousands of
-    // predicated loads of as many operands: the compiler needs minutes for the branches.  A pointer takes two scalar
-    // registers and the lane mask of every predicate two more, of the 102 a wavefront has: kernels of 60 and more
-    // buffers used all 512 vector registers, kept some 200 scalar registers in lanes of vector registers and spilled
-    // vector registers to scratch on top, and three of them were seen to produce wrong elements.
-    // Walking producers first, a value whose expression would exceed the limit gets a buffer and a kernel of its own
-    // (its largest folded operands first, then itself), so that its consumers read it as one operand.  Within the
-    // bounds a kernel stays below 300 vector registers, spills none of them and needs no scratch.
-    static constexpr int64_t kMaxInlineLoads = 32;
-    static constexpr int64_t kMaxKernelPointers = 40;
+    // ---- 3a. A tensor reference with many pieces (a Concat of many values, or of many slices that do not continue one
+    // another) costs its reader one predicated load per piece.  A reference with more pieces than the bound is cut,
+    // by planes that no piece straddles (every Concat leaves one), into parts of at most that many pieces; a part with
+    // more than one piece becomes a dense copy of its box, written by a kernel of its own, and the reference reads the
+    // copies.  Repeated until the reference itself is narrow enough.
+    TRef narrow_reference(const TRef& t, int64_t limit, double order, const std::string& name) {
+        if ((int64_t)t.pieces.size() <= limit) return t;
+        struct Part { Shape lo, hi; std::vector<const Piece*> pieces; };
+        std::vector<Part> work, done;
+        {
+            Part whole;
+            whole.lo.assign(t.shape.size(), 0);
+            whole.hi = t.shape;
+            for (const Piece& p : t.pieces) whole.pieces.push_back(&p);
+            work.push_back(std::move(whole));
+        }
+        while (!work.empty()) {
+            Part part = std::move(work.back());
+            work.pop_back();
+            if ((int64_t)part.pieces.size() <= limit) { done.push_back(std::move(part)); continue; }
+            // the plane that divides the part's pieces most evenly
+            int best_dim = -1;
+            int64_t best_at = 0;
+            size_t best_low = 0;
+            for (size_t d = 0; d < t.shape.size(); ++d) {
+                std::vector<int64_t> cuts;
+                for (const Piece* p : part.pieces)
+                    if (p->hi[d] < part.hi[d]) cuts.push_back(p->hi[d]);
+                std::sort(cuts.begin(), cuts.end());
+                cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+                for (int64_t c : cuts) {
+                    size_t low = 0;
+                    bool clean = true;
+                    for (const Piece* p : part.pieces) {
+                        if (p->hi[d] <= c) ++low;
+                        else if (p->lo[d] < c) { clean = false; break; }
+                    }
+                    if (!clean || low == 0 || low == part.pieces.size()) continue;
+                    const size_t half = part.pieces.size() / 2;
+                    auto off = [&](size_t v) { return v > half ? v - half : half - v; };
+                    if (best_dim < 0 || off(low) < off(best_low)) { best_dim = (int)d; best_at = c; best_low = low; }
+                }
+            }
+            if (best_dim < 0) { done.push_back(std::move(part)); continue; }  // no such plane: stays as wide as it is
+            Part lo_part, hi_part;
+            lo_part.lo = hi_part.lo = part.lo;
+            lo_part.hi = hi_part.hi = part.hi;
+            lo_part.hi[(size_t)best_dim] = best_at;
+            hi_part.lo[(size_t)best_dim] = best_at;
+            for (const Piece* p : part.pieces) (p->hi[(size_t)best_dim] <= best_at ? lo_part : hi_part).pieces.push_back(p);
+            work.push_back(std::move(hi_part));
+            work.push_back(std::move(lo_part));
+        }
+        if (done.size() < 2) return t;
+        TRef o;
+        o.shape = t.shape;
+        for (const Part& part : done) {
+            if (part.pieces.size() == 1) { o.pieces.push_back(*part.pieces[0]); continue; }
+            TRef sub;
+            for (size_t d = 0; d < t.shape.size(); ++d) sub.shape.push_back(part.hi[d] - part.lo[d]);
+            for (const Piece* p : part.pieces) {
+                Piece q = *p;
+                for (size_t d = 0; d < t.shape.size(); ++d) { q.lo[d] -= part.lo[d]; q.hi[d] -= part.lo[d]; }
+                sub.pieces.push_back(std::move(q));
+            }
+            Node* c = new_node(Op::COPY, sub.shape, {sub}, name + ".part");
+            c->root = true;
+            c->order = std::min(c->order, order - 0.5);
+            Piece q;
+            q.lo = part.lo;
+            q.hi = part.hi;
+            q.view.st.push_back(contiguous_stage(sub.shape));
+            q.src.kind = Src::NODE;
+            q.src.node = c;
+            o.pieces.push_back(std::move(q));
+        }
+        std::sort(o.pieces.begin(), o.pieces.end(), [](const Piece& x, const Piece& y) { return x.lo < y.lo; });
+        if (o.pieces.size() >= t.pieces.size()) return o;
+        return narrow_reference(o, limit, order, name);
+    }
+
+    void narrow_references(RegionPlan& rp) {
+        const int64_t limit = bound(opt.max_pieces);
+        bool added = false;
+        std::vector<Node*> work = rp.topo;
+        for (size_t i = 0; i < work.size(); ++i) {
+            Node* n = work[i];
+            for (TRef& t : n->in) {
+                if ((int64_t)t.pieces.size() <= limit) continue;
+                const size_t before = arena.size();
+                t = narrow_reference(t, limit, n->order, n->name);
+                n->key.clear();
+                // the copies' own operands are narrow by construction (at most `limit` pieces each)
+                added = added || arena.size() != before;
+            }
+        }
+        if (added) order_nodes(rp);
+    }
+
+    // ---- 4b. A kernel is bounded in what drives its register pressure.  A folded expression may load from at most
+    // max_inline_sites places (a load site: one piece of a tensor reference onto a value in memory, reached along
+    // one chain of views) and from at most max_inline_loads distinct values; a kernel may load from at most
+    // max_kernel_sites places and name at most max_kernel_pointers buffers (operands and outputs of all its members).
+    // Slices spelled as one Index per line joined by Concats, summed up by a backward pass, fold into expressions
+    // with thousands of predicated loads of as many operands: the compiler needs minutes for the branches.  A pointer
+    // takes two scalar registers and the lane mask of every predicate two more, of the 102 a wavefront has: kernels
+    // of 60 and more buffers used all 512 vector registers, kept some 200 scalar registers in lanes of vector
+    // registers and spilled vector registers to scratch on top, and three of them were seen to produce wrong elements.
+    // Walking producers first, a value whose expression would exceed a limit gets a buffer and a kernel of its own
+    // (its largest folded operands first, then itself), so that its consumers read it as one operand.
+    static uint64_t mix(uint64_t h, uint64_t v) {
+        h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
+        return h;
+    }
+    static uint64_t hash_str(const std::string& s) {
+        uint64_t h = 1469598103934665603ull;
+        for (unsigned char c : s) { h ^= c; h *= 1099511628211ull; }
+        return h;
+    }
+    // load sites of the expression of `n` evaluated in place, given those of the folded values below it
+    std::set<uint64_t> expression_sites(Node* n, const std::map<Node*, std::set<uint64_t>>& below) {
+        std::set<uint64_t> out;
+        std::set<std::string> seen_refs;
+        for (const TRef& t : n->in) {
+            if (!seen_refs.insert(tref_str(t)).second) continue;  // x * x: one set of loads
+            for (const Piece& p : t.pieces) {
+                if (p.src.kind != Src::NODE) continue;
+                Node* s = p.src.node;
+                const bool ident = identity_piece(p, t) && numel(s->shape) == numel(n->shape);
+                uint64_t path = 0;
+                if (!ident) {
+                    std::string v = shape_str(p.lo) + shape_str(p.hi);
+                    for (const Stage& st : p.view.st) v += stage_str(st);
+                    path = hash_str(v);
+                }
+                if (in_mem(s)) out.insert(mix((uint64_t)s->id + 1, path));
+                else {
+                    auto it = below.find(s);
+                    if (it == below.end()) continue;
+                    for (uint64_t k : it->second) out.insert(ident ? k : mix(k, path));
+                }
+            }
+        }
+        return out;
+    }
+
     void cut_long_expressions(RegionPlan& rp) {
         if (!opt.fuse) return;
+        const int64_t max_loads = bound(opt.max_inline_loads), max_sites = bound(opt.max_inline_sites);
         std::map<Node*, std::vector<Node*>> operands;  // per folded value: the in-memory values its expression reads (sorted)
+        auto& sites = rp.sites;
         auto gather = [&](Node* n) {
             std::vector<Node*> u;
             for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
@@ -1601,27 +1753,31 @@ struct Lowerer {
             return u;
         };
         for (Node* n : rp.topo) {
-            if (op_is_leaf(n->op)) continue;
+            if (op_is_leaf(n->op) || numel(n->shape) == 0) continue;
             std::vector<Node*> u = gather(n);
-            if (!n->root && op_is_elw(n->op) && (int64_t)u.size() > kMaxInlineLoads && numel(n->shape) > 0) {
+            std::set<uint64_t> st = expression_sites(n, sites);
+            auto too_long = [&] { return (int64_t)u.size() > max_loads || (int64_t)st.size() > max_sites; };
+            if (too_long()) {
                 std::vector<std::pair<size_t, Node*>> parts;
                 for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
-                    if (!in_mem(s) && op_is_elw(s->op) && numel(s->shape) > 0) parts.push_back({operands[s].size(), s});
+                    if (!in_mem(s) && op_is_elw(s->op) && numel(s->shape) > 0) parts.push_back({sites[s].size(), s});
                 });
                 std::sort(parts.begin(), parts.end(), [](const std::pair<size_t, Node*>& x, const std::pair<size_t, Node*>& y) {
                     return x.first != y.first ? x.first > y.first : x.second->order < y.second->order;
                 });
                 parts.erase(std::unique(parts.begin(), parts.end()), parts.end());
                 for (auto& pt : parts) {
-                    if ((int64_t)u.size() <= kMaxInlineLoads) break;
+                    if (!too_long()) break;
                     if (pt.second->root || pt.first <= 1) continue;
                     pt.second->root = true;
                     operands.erase(pt.second);
                     u = gather(n);
+                    st = expression_sites(n, sites);
                 }
-                if ((int64_t)u.size() > kMaxInlineLoads) n->root = true;
+                if (too_long() && op_is_elw(n->op)) n->root = true;
             }
-            if (!n->root) operands[n] = std::move(u);
+            if (!in_mem(n)) operands[n] = std::move(u);
+            sites[n] = std::move(st);
         }
     }
 
@@ -1634,9 +1790,27 @@ struct Lowerer {
             for (auto& kv : rp.reads[extra]) u.insert(kv.first);
         return (int64_t)(u.size() + G.members.size() + (extra ? 1 : 0) + G.colsums.size() + G.rowsums.size());
     }
-    // the pass with sums runs 1024 threads a block, which leaves a lane 128 vector registers: a pass that names more
-    // buffers than this would spill them, so its sums get kernels of their own
-    bool can_carry_sums(RegionPlan& rp, const Group& G) { return group_pointers(rp, G) < 20; }
+    // the places a kernel of this group (with one more member, if given) loads from
+    int64_t group_sites(RegionPlan& rp, const Group& G, Node* extra = nullptr) {
+        std::set<uint64_t> u;
+        auto add = [&](Node* m) {
+            auto it = rp.sites.find(m);
+            if (it != rp.sites.end()) u.insert(it->second.begin(), it->second.end());
+        };
+        for (Node* m : G.members) add(m);
+        for (auto& cs : G.riders()) add(cs.first);
+        if (extra) add(extra);
+        return (int64_t)u.size();
+    }
+    bool group_fits(RegionPlan& rp, const Group& G, Node* extra) {
+        return group_pointers(rp, G, extra) <= bound(opt.max_kernel_pointers) && group_sites(rp, G, extra) <= bound(opt.max_kernel_sites);
+    }
+    // the pass with sums runs 1024 threads a block, which leaves a lane 128 vector registers: a pass that loads from
+    // more places or names more buffers than this would spill them, so its sums get kernels of their own
+    bool can_carry_sums(RegionPlan& rp, const Group& G, Node* value = nullptr) {
+        if (tight()) return false;
+        return group_pointers(rp, G) < bound(opt.max_carrier_pointers) && group_sites(rp, G, value) <= bound(opt.max_carrier_sites);
+    }
 
     void form_groups(RegionPlan& rp) {
         auto& topo = rp.topo;
@@ -1656,7 +1830,7 @@ struct Lowerer {
             if (op_is_elw(r->op) && opt.fuse && !r->transpose) {
                 for (int g = (int)groups.size() - 1; g >= 0; --g) {
                     if (groups[g].kind != Group::ELW || groups[g].n != numel(r->shape)) continue;
-                    if (group_pointers(rp, groups[g], r) > kMaxKernelPointers) continue;  // a kernel's size is bounded too
+                    if (!group_fits(rp, groups[g], r)) continue;  // a kernel's size is bounded too
                     bool ok = true;
                     for (auto& rd : reads[r]) {
                         if (op_is_leaf(rd.first->op)) continue;
@@ -1707,6 +1881,7 @@ struct Lowerer {
         auto& group_of = rp.group_of;
         const auto& home_of = rp.home_of;
         auto reads_node = [&](const Group& H, Node* what) { return group_reads(rp, H, what); };
+        if (tight()) return -1;  // a region asked to keep its kernels small fuses nothing across kernel kinds
         for (size_t ge = g + 1; ge < groups.size(); ++ge) {
             Group& E = groups[ge];
             if (E.dead) continue;
@@ -1747,7 +1922,7 @@ struct Lowerer {
             int target = -1;
             for (size_t g = 0; g < groups.size() && target < 0; ++g) {
                 Group& G = groups[g];
-                if (G.dead || G.kind != Group::ELW || G.n != R * C || !can_carry_sums(rp, G)) continue;
+                if (G.dead || G.kind != Group::ELW || G.n != R * C || !can_carry_sums(rp, G, E)) continue;
                 if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                 for (Node* m : G.members)
                     if (m == E || folded_in[m].count(E)) { target = (int)g; break; }
@@ -1762,7 +1937,7 @@ struct Lowerer {
                 for (auto& kv : er) ident = ident && kv.second;
                 for (size_t g = 0; ident && g < groups.size() && target < 0; ++g) {
                     Group& G = groups[g];
-                    if (G.dead || G.kind != Group::ELW || G.n != R * C || !can_carry_sums(rp, G)) continue;
+                    if (G.dead || G.kind != Group::ELW || G.n != R * C || !can_carry_sums(rp, G, E)) continue;
                     if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                     bool all = true;
                     for (auto& kv : er) {
@@ -1818,7 +1993,7 @@ struct Lowerer {
             int target = -1;
             for (size_t g = 0; g < groups.size() && target < 0; ++g) {
                 Group& G = groups[g];
-                if (g == gs || G.dead || G.tiled || G.kind != Group::ELW || G.n != R * C || !G.side.empty() || !can_carry_sums(rp, G)) continue;
+                if (g == gs || G.dead || G.tiled || G.kind != Group::ELW || G.n != R * C || !G.side.empty() || !can_carry_sums(rp, G, E)) continue;
                 if (G.rides() && (G.cs_rows != R || G.cs_cols != C)) continue;
                 bool computes = false;
                 for (Node* m : G.members) computes = computes || m == E || folded_in[m].count(E);
@@ -1904,6 +2079,7 @@ struct Lowerer {
     void attach_row_sum_operands(RegionPlan& rp) {
         auto& groups = rp.groups;
         auto& group_of = rp.group_of;
+        if (tight()) return;
         for (size_t gs = 1; gs < groups.size(); ++gs) {
             Group& GS = groups[gs];
             if (GS.dead || GS.kind != Group::SUM) continue;
@@ -3432,6 +3608,18 @@ std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::str
     if (const char* e = getenv("ADHIP_LAYER_KERNELS")) opt.layer_kernels = opt.layer_kernels && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_MERGE_SMALL")) opt.merge_small = opt.merge_small && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_FUSE_ATTENTION")) opt.fuse_attention = opt.fuse_attention && atoi(e) != 0;
+    // diagnostic: the seven kernel-size bounds, in the order LowerOptions declares them ("24,48,32,96,40,24,20")
+    if (const char* e = getenv("ADHIP_KERNEL_BOUNDS")) {
+        int* field[7] = {&opt.max_pieces, &opt.max_inline_sites, &opt.max_inline_loads, &opt.max_kernel_sites, &opt.max_kernel_pointers,
+                         &opt.max_carrier_sites, &opt.max_carrier_pointers};
+        for (int i = 0; i < 7 && *e; ++i) {
+            char* end = nullptr;
+            const long v = strtol(e, &end, 10);
+            if (end == e) break;
+            if (v >= 2) *field[i] = (int)std::min<long>(v, 1 << 20);
+            e = *end == ',' ? end + 1 : end;
+        }
+    }
     Lowerer l(prog, dep_ids, opt);
     return l.run();
 }

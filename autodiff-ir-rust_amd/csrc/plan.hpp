@@ -22,6 +22,7 @@ struct KernelDef {
     std::string entry;   // symbol name
     std::string source;  // complete HIP C++ translation unit
     std::string kind;    // "elw", "reduce_row", "reduce_col", "dot", ...
+    std::vector<int> regions;  // the straight-line regions (in lowering order) whose launches use it
 };
 
 struct Arg {

@@ -379,18 +379,53 @@ std::string describe_spills(const std::vector<char>& code, bool everything) {
     return text;
 }
 
+// Lowers a program and compiles the kernels that `have` does not know yet into `objects` (by source text).  A kernel
+// that the compiler could only build by spilling vector registers to scratch memory is never accepted: the regions
+// it belongs to are lowered again with their kernel-size bounds halved (LowerOptions::region_shift), up to four
+// times, and if a kernel still spills then -- or is not one the lowering can cut: a hand-written one -- the program
+// is refused.  `relowered` receives the number of extra lowerings.
+template <class Have>
+std::unique_ptr<Plan> lower_and_compile(const Proc& ir, const std::vector<std::string>& deps, const std::string& arch, Have&& have,
+                                        std::map<std::string, std::vector<char>>& objects, int* relowered = nullptr) {
+    LowerOptions opt;
+    for (int attempt = 0;; ++attempt) {
+        std::unique_ptr<Plan> plan = lower_program(ir, deps, opt);
+        std::vector<std::string> missing;
+        for (const KernelDef& k : plan->kernels)
+            if (!objects.count(k.source) && !have(k.source)) missing.push_back(k.source);
+        for (auto& kv : compile_code_objects(missing, arch)) objects[kv.first] = std::move(kv.second);
+        std::set<int> regions;
+        std::string report;
+        for (const KernelDef& k : plan->kernels) {
+            auto it = objects.find(k.source);
+            if (it == objects.end()) continue;  // loaded before, so accepted before
+            for (const KernelSpills& ks : code_object_spills(it->second)) {
+                if (ks.vector <= 0) continue;
+                report += strf("%s%s [%s] (%ld vector, %ld scalar registers spilled, %ld bytes of scratch per lane)", report.empty() ? "" : "; ",
+                               ks.name.c_str(), k.kind.c_str(), ks.vector, ks.scalar, ks.scratch_bytes);
+                for (int r : k.regions)
+                    if (r >= 0) regions.insert(r);
+            }
+        }
+        if (relowered) *relowered = attempt;
+        if (report.empty()) return plan;
+        bool tighter = false;
+        for (int r : regions) {
+            int& sh = opt.region_shift[r];
+            if (sh < 4) { ++sh; tighter = true; }
+        }
+        ADHIP_CHECK(tighter && attempt < 4,
+                    "refusing to run kernels that spill vector registers to scratch memory (after %d lowerings with tighter bounds): %s",
+                    attempt, report.c_str());
+    }
+}
+
 std::shared_ptr<Module> compile_module(adhip_ctx* ctx, const std::string& source, const std::vector<char>* code_in = nullptr) {
     auto it = ctx->modules.find(source);
     if (it != ctx->modules.end()) return it->second;
     std::vector<char> code = code_in ? *code_in : compile_code_object(source, ctx->arch);
     auto m = std::make_shared<Module>();
     HIP_OK(hipModuleLoadData(&m->mod, code.data()));
-    // say so once per module when a kernel in it spills vector registers (ADHIP_QUIET=1 silences it)
-    const char* quiet = getenv("ADHIP_QUIET");
-    if (!(quiet && *quiet == '1')) {
-        const std::string spills = describe_spills(code, false);
-        if (!spills.empty()) fprintf(stderr, "adhip: kernel %s\n", spills.c_str());
-    }
     // a long-lived context that keeps seeing new programs does not keep every module it ever loaded: beyond a
     // bound, the ones no live program refers to are unloaded (their code objects stay in the on-disk cache)
     if (ctx->modules.size() >= 1024) {
@@ -438,14 +473,11 @@ adhip_program* program_create(adhip_ctx* ctx, const uint8_t* program, size_t len
     const char* genv = getenv("ADHIP_GRAPHS");
     if (genv && *genv == '0') p->use_graphs = false;
     p->ir = parse_program(program, len, payload_offsets);
-    p->plan = lower_program(*p->ir, dep_vector(dep_ids, n));
+    std::map<std::string, std::vector<char>> fresh;
+    // kernels: what the context has not loaded yet is compiled (or fetched from the disk cache) in parallel
+    p->plan = lower_and_compile(*p->ir, dep_vector(dep_ids, n), ctx->arch, [&](const std::string& src) { return ctx->modules.count(src) != 0; }, fresh);
     Plan& plan = *p->plan;
     try {
-        // kernels: what the context has not loaded yet is compiled (or fetched from the disk cache) in parallel
-        std::vector<std::string> missing;
-        for (const KernelDef& k : plan.kernels)
-            if (!ctx->modules.count(k.source)) missing.push_back(k.source);
-        std::map<std::string, std::vector<char>> fresh = compile_code_objects(missing, ctx->arch);
         for (const KernelDef& k : plan.kernels) {
             auto f = fresh.find(k.source);
             auto m = compile_module(ctx, k.source, f != fresh.end() ? &f->second : nullptr);
@@ -1176,12 +1208,11 @@ int adhip_compile_check(const uint8_t* program, size_t program_len, const char* 
     std::string text;
     int rc = guarded(nullptr, [&] {
         auto ir = parse_program(program, program_len);
-        auto plan = lower_program(*ir, dep_vector(dep_ids, n_dep_ids));
         size_t bytes = 0;
         const char* dump_dir = getenv("ADHIP_DUMP_CODE_DIR");
-        std::vector<std::string> sources;
-        for (auto& k : plan->kernels) sources.push_back(k.source);
-        std::map<std::string, std::vector<char>> objects = compile_code_objects(sources, arch && *arch ? arch : "gfx950");
+        std::map<std::string, std::vector<char>> objects;
+        int relowered = 0;
+        auto plan = lower_and_compile(*ir, dep_vector(dep_ids, n_dep_ids), arch && *arch ? arch : "gfx950", [](const std::string&) { return false; }, objects, &relowered);
         for (auto& k : plan->kernels) {
             const std::vector<char>& code = objects[k.source];
             bytes += code.size();
@@ -1192,9 +1223,10 @@ int adhip_compile_check(const uint8_t* program, size_t program_len, const char* 
             }
         }
         text = strf("%zu kernels compiled, %zu bytes of code objects", plan->kernels.size(), bytes);
+        if (relowered) text += strf("; lowered %d more times with tighter kernel bounds", relowered);
         std::string spills;
-        for (auto& o : objects) {
-            const std::string one = describe_spills(o.second, true);
+        for (auto& k : plan->kernels) {
+            const std::string one = describe_spills(objects[k.source], true);
             if (!one.empty()) spills += (spills.empty() ? "" : "; ") + one;
         }
         if (!spills.empty()) text += "; spilling kernels: " + spills;

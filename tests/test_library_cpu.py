@@ -174,26 +174,85 @@ def test_random_programs_lower_and_compile(seed):
     assert not out["target"].is_none
 
 
+def _generated_kernel_sizes(proc, deps, monkeypatch):
+    """(entry, kind, buffers named, places loaded from) of every generated kernel of the lowered program, read off the
+    kernels' text: operands are parameters b<N>, outputs o<N>; a load is `b<N>[...]` or a 128-bit access at `b<N> + ...`."""
+    monkeypatch.setenv("ADHIP_DUMP_SOURCE", "1")
+    text = lower_describe(proc, deps)
+    parts = re.split(r"// ===== (\S+) \[(\w+)\] =====\n", text)
+    out = []
+    for i in range(1, len(parts), 3):
+        if parts[i + 1] not in ("elw", "elw_colsum", "elw_tiled", "reduce_row", "reduce_row_store", "reduce_col"):
+            continue
+        body = parts[i + 2]
+        if re.search(r"_x\d+\(", body) and "blockIdx.z" in body:
+            continue  # the shared-launch wrapper repeats its kernel's parameters once per member
+        operands = set(re.findall(r"\b[bo]\d+\b", body))
+        loads = len(re.findall(r"\bb\d+\[", body)) + len(re.findall(r"\(b\d+ \+ ", body))
+        out.append((parts[i], parts[i + 1], len(operands), loads))
+    return out
+
+
 @pytest.mark.parametrize("seed", [301, 343])
 def test_folded_expressions_stay_bounded(seed, monkeypatch):
     """Slices of long dims (one Index per line, joined by Concats) and the sums of their gradients fold into
     expressions with thousands of predicated loads unless the lowering cuts them: seed 301 at scale 16 is 24 000
     commands whose largest kernel would read memory in 5 900 places (minutes of compilation); seed 343 gave a kernel
-    with 300 loads that ran out of registers.  No generated kernel may name more than 40 buffers."""
+    with 300 loads that ran out of registers.  No generated kernel may name more than 40 buffers or load from more
+    than 96 places."""
     from fuzz_programs import random_program
-    monkeypatch.setenv("ADHIP_DUMP_SOURCE", "1")
     dev = Capture()
     random_program(dev, seed, scale=16)
-    text = lower_describe(dev.proc, dev.deps)
-    parts = re.split(r"// ===== (\S+) \[(\w+)\] =====\n", text)
-    assert len(parts) > 3
-    for i in range(1, len(parts), 3):
-        if parts[i + 1] not in ("elw", "elw_colsum", "elw_tiled", "reduce_row", "reduce_row_store", "reduce_col", "merged"):
-            continue
-        if parts[i + 1] == "merged":
-            continue
-        operands = set(re.findall(r"\b[bo]\d+\b", parts[i + 2]))
-        assert len(operands) <= 40, (parts[i], len(operands))
+    sizes = _generated_kernel_sizes(dev.proc, dev.deps, monkeypatch)
+    assert len(sizes) > 1
+    for entry, kind, operands, loads in sizes:
+        assert operands <= 40 and loads <= 96, (entry, kind, operands, loads)
+
+
+def _vector_spills(msg):
+    return [(name, int(vector)) for name, scalar, vector, scratch in
+            re.findall(r"(\w+) \((\d+) scalar, (\d+) vector registers spilled, (\d+) bytes", msg) if int(vector)]
+
+
+@pytest.mark.parametrize("name,build", [
+    ("200 buffers under one multiplication", lambda: __import__("adversarial_programs").wide_concat(100)),
+    ("one buffer behind 200 pieces", lambda: __import__("adversarial_programs").one_buffer_pieces(200)),
+    ("39 operands gathered against the grain", lambda: __import__("adversarial_programs").gathers(39)),
+    ("a pass of 17 operands that carries a row and a column sum", lambda: __import__("adversarial_programs").rider(17)),
+    ("a pass of 19 operands whose sums are wanted", lambda: __import__("adversarial_programs").rider(19)),
+])
+def test_adversarial_programs_are_cut_into_kernels_that_fit(name, build, monkeypatch):
+    """What drives a kernel's register pressure is the number of places it loads from (every concat piece is a load
+    under a predicate) and the buffers it names, whether or not the value that reads them was going to get a kernel of
+    its own anyway: a reference with more pieces than the bound is copied part by part first, an expression that loads
+    from too many places is cut, sums ride only on small passes.  The compiler's record of every kernel shows no
+    spilled vector register, and no lowering with tighter bounds was needed to get there."""
+    monkeypatch.setenv("ADHIP_CACHE_DIR", "off")
+    proc, keep, _ = build()
+    for entry, kind, operands, loads in _generated_kernel_sizes(proc, keep, monkeypatch):
+        assert operands <= 40 and loads <= 96, (name, entry, kind, operands, loads)
+    monkeypatch.delenv("ADHIP_DUMP_SOURCE")
+    rc, msg = _compile_check(proc, keep)
+    assert rc == 0, msg
+    assert not _vector_spills(msg), msg
+    assert "tighter kernel bounds" not in msg, msg
+
+
+def test_a_kernel_that_spills_vector_registers_is_cut_again_or_refused(monkeypatch):
+    """The library never runs a kernel whose code object records spilled vector registers (three such kernels computed
+    wrong elements).  With the lowering's bounds raised so far that 184 buffers land in one kernel (ADHIP_KERNEL_BOUNDS,
+    a diagnostic switch), the compiler spills; the regions of such a kernel are lowered again with the bounds halved
+    until nothing spills.  Raised so far that four halvings do not help, the program is refused with an error."""
+    from adversarial_programs import wide_concat
+    monkeypatch.setenv("ADHIP_CACHE_DIR", "off")
+    proc, keep, _ = wide_concat(92)
+    monkeypatch.setenv("ADHIP_KERNEL_BOUNDS", "200,200,200,200,200,200,200")
+    rc, msg = _compile_check(proc, keep)
+    assert rc == 0, msg
+    assert "more times with tighter kernel bounds" in msg and not _vector_spills(msg), msg
+    monkeypatch.setenv("ADHIP_KERNEL_BOUNDS", "4000,4000,4000,4000,4000,4000,4000")
+    rc, msg = _compile_check(proc, keep)
+    assert rc != 0 and "refusing to run kernels that spill vector registers" in msg, msg
 
 
 @pytest.mark.parametrize("scale,seed", [(48, 81), (48, 31), (48, 52)])

@@ -254,6 +254,26 @@ def test_random_programs_at_scale(scale, seed, hip_device):
         assert_close(got[k].data, rv.data, tol, f"scale {scale} seed {seed} {k}", scale=max(own, 1e-2 * largest))
 
 
+@pytest.mark.parametrize("name", ["wide_concat", "one_buffer_pieces", "gathers", "rider17", "rider19"])
+def test_adversarial_programs_match_numpy(name, hip_device):
+    """Programs that strain the size of one kernel (tests/adversarial_programs.py) against closed forms in numpy: data
+    movement and a single multiplication are bit-exact, the sum of 39 transposed operands is added in program order on
+    both sides, the sums are compared with float64."""
+    print(f"[case] adversarial {name}", flush=True)
+    import adversarial_programs as A
+    build = {"wide_concat": lambda: A.wide_concat(100), "one_buffer_pieces": lambda: A.one_buffer_pieces(200),
+             "gathers": lambda: A.gathers(39), "rider17": lambda: A.rider(17), "rider19": lambda: A.rider(19)}[name]
+    proc, keep, want = build()
+    hip_device.execute(proc, set(keep))
+    for k, ref in want.items():
+        got = hip_device.get_tensor(k)
+        assert got.dim == list(ref.shape), (k, got.dim)
+        if k in ("rs", "cs"):
+            assert_close(got.data.reshape(ref.shape), ref, RED_RTOL * math.sqrt(2048))
+        else:  # (the riders' product of up to 19 factors is multiplied in program order on both sides)
+            assert_exact(got.data.reshape(ref.shape), ref, f"{name}.{k}")
+
+
 def _run_ir(dev, cmds, keep):
     from adhip import ir as IR
     proc = IR.IRProcedure("main", list(cmds) + [IR.EX()])
