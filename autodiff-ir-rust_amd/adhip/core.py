@@ -431,9 +431,11 @@ class Tensor:
         exp overflows beyond x = 88.  The evident intent is followed: normalise along `dim`, with the maximum along
         `dim` subtracted first.  The maximum carries no gradient: a shift of the argument cancels in the quotient."""
         d = len(self.dim()) + dim if dim < 0 else dim
-        m = self.max(d).stop_grad().unsqueeze(d)
+        keep = list(self.dim())
+        keep[d] = 1   # the reduced dim kept with extent 1 (a vector's reduction has one element, not rank 0)
+        m = self.max(d).stop_grad().view(keep)
         e = (self - m).exp()
-        return e / e.sum(d).unsqueeze(d)
+        return e / e.sum(d).view(keep)
 
     # -- comparisons (src/graph/ops/equality.rs) --------------------------------------
     def equal(self, b: "Tensor"):

@@ -274,6 +274,46 @@ def test_adversarial_programs_match_numpy(name, hip_device):
             assert_exact(got.data.reshape(ref.shape), ref, f"{name}.{k}")
 
 
+MODEL_FUZZ = ([(1, s) for s in range(40)] + [(4, s) for s in range(16)] + [(16, s) for s in range(10)] +
+              [(48, s) for s in range(4)])
+
+
+@pytest.mark.parametrize("scale,seed", MODEL_FUZZ)
+def test_random_model_programs(scale, seed, hip_device):
+    """Random programs out of softmax, row maxima, mean / variance, LayerNorm, RMS, Linear with its in-place bias,
+    tensor `*=` / `-=` / `+=`, Attention and AttentionMasked (fused, and unfused where the probabilities are kept),
+    and Concats of up to 12 distinct values (tests/fuzz_models.py), forward and backward.  Checked twice: against the
+    oracle (same command stream, the reference's arithmetic) and against a float64 torch shadow of the same
+    computation that shares no code with the caller side.  Where a value is the outcome of cancellation (the
+    gradient of a sum of softmax rows is exactly 0), the oracle's own distance from the float64 answer says how well
+    float32 can know it, and the device may be a few times that far from it; otherwise 1e-5 sqrt(N) of the value's own
+    largest element, N = the most terms any Sum or DotProduct of the program adds."""
+    print(f"[case] model fuzz scale {scale} seed {seed}", flush=True)
+    from fuzz_models import random_model_program, shadow_model_program
+    got = random_model_program(hip_device, seed, scale)
+    oracle = OracleDevice()
+    ref = random_model_program(oracle, seed, scale)
+    exact = shadow_model_program(seed, scale)
+    assert set(got) == set(ref)
+    tol = RED_RTOL * math.sqrt(oracle.max_terms) * 2
+    for k, rv in ref.items():
+        assert got[k].dim == rv.dim, f"{k}: dim {got[k].dim} vs {rv.dim}"
+        if k not in exact:
+            continue  # the gradient of a leaf that the shadow holds as a constant
+        e = exact[k].ravel()
+        r = np.asarray(rv.data, np.float64)
+        g = np.asarray(got[k].data, np.float64)
+        assert e.shape == r.shape, f"{k}: {exact[k].shape} vs {rv.dim}"
+        own = float(np.max(np.abs(e))) if e.size else 0.0
+        oracle_err = float(np.max(np.abs(r - e))) if e.size else 0.0
+        assert oracle_err <= tol * max(own, 1e-3 * max(float(np.max(np.abs(x))) for x in exact.values())), \
+            f"scale {scale} seed {seed} {k}: the oracle is {oracle_err:.3e} from float64 (own scale {own:.3e})"
+        allowed = max(tol * own, 8.0 * oracle_err)
+        err = float(np.max(np.abs(g - e))) if e.size else 0.0
+        assert err <= allowed, f"scale {scale} seed {seed} {k}: |device - float64| = {err:.3e} > {allowed:.3e} (own scale {own:.3e}, oracle {oracle_err:.3e})"
+        assert float(np.max(np.abs(g - r))) <= 2 * allowed if e.size else True
+
+
 def _run_ir(dev, cmds, keep):
     from adhip import ir as IR
     proc = IR.IRProcedure("main", list(cmds) + [IR.EX()])
