@@ -1173,10 +1173,11 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
     const Node* n = spec.node;
     ADHIP_CHECK(op_is_reduce(n->op) && n->in.size() == 1 && n->in[0].shape.size() == 2, "internal: malformed reduction");
     // Sum and Max share everything but the combining step: `acc (+)= v`, the identity lanes start from, and how two
-    // partial results are merged.  fmaxf returns the other operand when one is NaN, so a row's maximum is NaN only
-    // if all of it is.
+    // partial results are merged.  fmaxf returns the other operand when one is NaN, so NaN is the identity of the
+    // maximum: a row's maximum is NaN exactly when all of it is (a row of -inf gives -inf), and lanes that hold no
+    // element of the row drop out of every combination.
     const bool mx = n->op == Op::MAX;
-    const char* ident = mx ? "-__builtin_inff()" : "0.0f";
+    const char* ident = mx ? "__builtin_nanf(\"\")" : "0.0f";
     auto comb = [&](const std::string& a, const std::string& b) { return mx ? "fmaxf(" + a + ", " + b + ")" : a + " + " + b; };
     auto comb4 = [&](const std::string& a, const std::string& b, const std::string& c, const std::string& d) {
         return mx ? "fmaxf(fmaxf(" + a + ", " + b + "), fmaxf(" + c + ", " + d + "))" : "(" + a + " + " + b + ") + (" + c + " + " + d + ")";

@@ -637,22 +637,13 @@ void* cur_buf(adhip_program* p, int buf) { return p->use_static ? p->static_buf_
 
 void launch(adhip_program* p, const Launch& l) {
     adhip_ctx* ctx = p->ctx;
-    // argument block: guard pointer, then the plan's arguments; on the stack for all but the widest launches, so
-    // that a run allocates nothing on the host either
+    // argument block: guard pointer, then the plan's arguments; on the stack, so that a run allocates nothing on the
+    // host either
     const void* guard = l.guard >= 0 ? (const void*)(cur_flags(p) + l.guard) : nullptr;
-    constexpr size_t kStackArgs = 192;
-    void* ptr_stack[kStackArgs + 1];
-    uint64_t val_stack[kStackArgs];
-    std::vector<void*> ptr_heap;
-    std::vector<uint64_t> val_heap;
-    void** ptrs = ptr_stack;
-    uint64_t* vals = val_stack;
-    if (l.args.size() > kStackArgs) {
-        ptr_heap.resize(l.args.size() + 1);
-        val_heap.resize(l.args.size());
-        ptrs = ptr_heap.data();
-        vals = val_heap.data();
-    }
+    constexpr size_t kStackArgs = 192;  // merged launches take at most 160 arguments, shared ones 96 pointers
+    void* ptrs[kStackArgs + 1];
+    uint64_t vals[kStackArgs];
+    ADHIP_CHECK(l.args.size() <= kStackArgs, "internal: launch '%s' takes %zu arguments", l.label.c_str(), l.args.size());
     ptrs[0] = (void*)&guard;
     for (size_t i = 0; i < l.args.size(); ++i) {
         const Arg& a = l.args[i];

@@ -192,6 +192,47 @@ def measure_attention(dev, seq=2048, d_model=1024, heads=8):
     return out
 
 
+def measure_reductions_forward(dev, rows=16384, cols=4096):
+    """The stand-alone reduction kernels at HBM size (what a forward-only `x.pow(2).sum(1)` / `x.sum(0)` runs: in the
+    forward + backward step of configs[2] the sums ride on the element-wise pass instead).  Three programs: configs[2]
+    without its backward pass; row sums of three different 256 MiB tensors; column sums of the same three.  With three
+    tensors in turn no launch finds its operand in the 256 MiB last-level cache."""
+    import numpy as np
+    from adhip import autodiff
+    from adhip import workloads as W
+    n = rows * cols
+    out = {"config": {"rows": rows, "cols": cols, "bytes_per_tensor": 4 * n}}
+    wl = W.reductions(dev, rows, cols, seed=0, backward=False)
+    p = compile_resident(dev, wl)
+    ms = timed_runs(p, 10, 2)
+    ks = profile(p, 5)
+    out["configs2_forward"] = {"ms_per_step": ms, "kernels": ks,
+                               "roofline": [hbm_roofline(k, k["bytes"], note="x read once by this launch") for k in ks if k["bytes"] > 2.0 * n]}
+    p.close()
+    rng = np.random.default_rng(0)
+    data = [rng.standard_normal(n, dtype=np.float32) for _ in range(3)]
+    for name, dim in (("row_sums", 1), ("column_sums", 0)):
+        autodiff.set_device(dev)
+        outs = {}
+        for i, d in enumerate(data):
+            s = autodiff.tensor(d, [rows, cols]).sum(dim)
+            s.forward()
+            s.val().keep()
+            outs[f"s{i}"] = s.val()
+        wls = W.Workload(name, outs, {}, algorithmic_bytes=3 * 4.0 * (n + (rows if dim else cols)))
+        p = compile_resident(dev, wls)
+        ms = timed_runs(p, 10, 2)
+        ks = profile(p, 5)
+        big = [k for k in ks if k["bytes"] > 2.0 * n]
+        tensors = sum(round(k["bytes"] / (4.0 * n)) * k["launches_per_run"] for k in big)
+        entry = {"ms_per_step": ms, "GBps_whole_step": wls.algorithmic_bytes / (ms * 1e-3) / 1e9, "kernels": ks, "tensors_per_step": tensors,
+                 "roofline": [hbm_roofline(k, k["bytes"], note=f"{round(k['bytes'] / (4.0 * n))} tensor(s) of {4 * n} bytes read once per launch; "
+                                           "three tensors in turn, so none is found in the last-level cache") for k in big]}
+        out[name] = entry
+        p.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,12 +241,13 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "manip", "attention"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "reductions_forward", "manip", "attention"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by; "
                          "'streammix': only a bare 3-reads + 4-writes kernel over 8192x8192 f32 (the stream mix of the "
                          "headline pass with trivial arithmetic and no column sums: what the memory system gives that mix); "
-                         "'reductions': only configs[2]; 'mlp': only configs[3]; 'manip': only configs[4] (one run: its "
+                         "'reductions': only configs[2]; 'reductions_forward': only the stand-alone row and column reduction "
+                         "kernels on 256 MiB tensors; 'mlp': only configs[3]; 'manip': only configs[4] (one run: its "
                          "loop consumes its counter); 'attention': only multi-head attention forward")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -258,6 +300,9 @@ def main():
         print(json.dumps({"metric": "reductions forward + backward, f32 [16384,4096]", "value": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
                           "unit": "GB/s", "ms_per_step": ms3, "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}))
         return
+    if args.workload == "reductions_forward":
+        print(json.dumps(dict(measure_reductions_forward(dev), metric="stand-alone reductions, f32 [16384,4096]")))
+        return
     if args.workload == "manip":
         wl5 = W.manip_loop(dev)
         p5 = compile_resident(dev, wl5)
@@ -277,7 +322,10 @@ def main():
         return
     wl = W.fused_elw(dev, rows, cols, seed=0)
     prog = compile_resident(dev, wl)
-    ms = timed_runs(prog, args.steps, args.warmup)
+    # five timed loops of exactly `steps` steps each; the reported step time is the median loop's, the others say how
+    # far one 6 ms sample can be off
+    loops = sorted(timed_runs(prog, args.steps, args.warmup if i == 0 else 0, spin=(i == 0)) for i in range(5))
+    ms = loops[len(loops) // 2]
     value = wl.algorithmic_bytes / (ms * 1e-3) / 1e9
     kstats = profile(prog, 5)
     dom = max(kstats, key=lambda k: k["avg_ms"] * k["launches_per_run"])
@@ -285,6 +333,8 @@ def main():
     # algorithmic bytes of the dominant launch: a, b, c, bias read once; y, da, db, dc written once
     dom_alg = 4.0 * (7 * n + cols) if dom["kernel"].startswith("elw") else dom["bytes"]
     roofline = hbm_roofline(dom, dom_alg, TRAFFIC_BYTES["fused_elw"]["elw_colsum"] if dom["kernel"].startswith("elw_colsum") else None)
+    roofline["traffic_source"] = ("hardware counters of a separate rocprofv3 --pmc run of this workload (summary: "
+                                  "profiles/fused_elw_8192x8192.hbm_traffic_pmc.txt); a constant of this script, not read in this run")
     prog.close()
 
     extra = {"fused_elw_kernels": kstats}
@@ -334,6 +384,7 @@ def main():
                 # x read once, dx written once, the row and column sums
                 extra["reductions"]["roofline"].append(hbm_roofline(k, 4.0 * (2 * n3 + 4096 + 16384), TRAFFIC_BYTES["reductions"]["elw_colsum"]))
         p3.close()
+        extra["reductions_forward"] = measure_reductions_forward(dev)
         # config 5: tensor manipulation + data-dependent loop
         wl5 = W.manip_loop(dev)
         p5 = compile_resident(dev, wl5)
@@ -345,7 +396,8 @@ def main():
             # r is 151 MB and is rewritten every iteration: it stays in the 256 MiB last-level cache, so the loop
             # kernels' rates are cache rates, not HBM rates
             k["GBps"] = k["bytes"] / (k["avg_ms"] * 1e-3) / 1e9
-            k["memory"] = "LLC-resident" if k["launches"] > 1 else "HBM"
+            # (that includes the row reduction launched once right behind the gather stage, which wrote r)
+            k["memory"] = "HBM" if k["launches"] == 1 and not k["kernel"].startswith("reduce") else "LLC-resident"
         # The gather stage again, the way every other kernel here is timed (clocks settled, several launches): the
         # run above follows an upload, during which the compute units idle.  Runs of the resident program repeat the
         # stage on the same inputs; the loop after it finds its counter at the limit and does not iterate.
@@ -383,7 +435,7 @@ def main():
     line = {
         "metric": "fused-ELW & reduce GB/s (% HBM peak); fp32 MLP train steps/s, 1 MI355X",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "ms_per_step": ms, "ms_per_step_of_each_timed_loop": loops, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "spin_up_seconds": SPIN_UP_SECONDS,
         "data": "synthetic",
         "config": {"workload": "configs[1]: fused element-wise + broadcast, forward + backward, a,b,c f32 [8192,8192], bias [8192]",

@@ -72,19 +72,23 @@ int adhip_program_run(adhip_program* p);
 int adhip_program_enqueue(adhip_program* p);
 int adhip_program_sync(adhip_program* p);
 
-/* adhip_program_enqueue for callers that cannot allocate device memory while they run (code under HIP graph capture,
- * tight serving loops, harnesses that forbid it).  No counterpart in the reference.
+/* adhip_program_enqueue for callers that cannot allocate device memory while they run (tight serving loops, harnesses
+ * that forbid it; a straight-line program also under HIP stream capture).  No counterpart in the reference.
  * Every temporary of the program (partial sums of reductions, slices of split matrix products, intermediate tensors)
  * and its control-flow flags are placed in a static device array of ADHIP_STATIC_SCRATCH_BYTES that the library holds
  * on every GPU it runs on, instead of in the program's own allocations; inputs, kept tensors and ids that live across
  * control flow stay in the buffers the program got at create time.  The call makes no hipMalloc / hipFree and no
- * allocating library call, launches every kernel directly (no graph capture or instantiation, no profiling events)
- * and returns without waiting, like adhip_program_enqueue.  A program whose temporaries and flags need more than
- * ADHIP_STATIC_SCRATCH_BYTES is refused with an error that names both sizes.  All programs of all contexts on one GPU
- * share that GPU's array and find the last call's contents in it (every kernel writes what it later reads from there,
- * so nothing needs clearing).  Runs queued on one context follow one another on its stream; runs of different
- * contexts on the same GPU that overlap in time race on the array -- wait for one (adhip_program_sync) before a run
- * of another context starts. */
+ * allocating library call, on the device or on the host, and launches every kernel directly (no graph capture or
+ * instantiation, no profiling events).  A straight-line program is queued and the call returns without waiting, like
+ * adhip_program_enqueue.  A program with loops or branches behaves as it does there too: the host reads predicates
+ * back (a 4-byte asynchronous copy into pinned memory the context holds since adhip_create, then a wait on the
+ * stream) -- once for a counted loop, once per batch of iterations for a data-dependent one, once per If -- which
+ * allocates nothing but blocks, and is not legal while the caller captures the stream.  A program whose temporaries
+ * and flags need more than ADHIP_STATIC_SCRATCH_BYTES is refused with an error that names both sizes.  All programs
+ * of all contexts on one GPU share that GPU's array and find the last call's contents in it (every kernel writes
+ * what it later reads from there, so nothing needs clearing).  Runs queued on one context follow one another on its
+ * stream; runs of different contexts on the same GPU that overlap in time race on the array -- wait for one
+ * (adhip_program_sync) before a run of another context starts. */
 #define ADHIP_STATIC_SCRATCH_BYTES (32u << 20)
 int adhip_program_enqueue_noalloc(adhip_program* p);
 /* Copy kept ids to host memory owned by the context (then served by adhip_get_tensor). */

@@ -303,3 +303,30 @@ def test_control_flow_semantics():
     assert dev.get_tensor("y").data[0] == 8.5
     assert dev.get_tensor("c").data[0] == 0.0
     assert dev.get_tensor("zz").is_none
+
+
+def test_reference_softmax_formula_on_a_square_matrix():
+    """The reference's softmax is `x.exp() / x.exp().sum(dim)` (src/nn/activations/softmax.rs:28-30): the sum loses
+    `dim`, and the division broadcasts it back by the trailing-dim rule, so on a square matrix element (i, j) is divided
+    by the sum of row j.  The caller side here normalises along `dim` instead (with the maximum subtracted first).
+    Both formulas spelled out on one 3x3 matrix: they differ, each matches its own closed form, and only the second
+    has rows that add up to 1."""
+    from adhip import autodiff
+    x = np.array([[0.0, 1.0, 2.0], [1.0, 1.0, 1.0], [3.0, 0.0, -1.0]], dtype=np.float32)
+    dev = OracleDevice()
+    autodiff.set_device(dev)
+    t = autodiff.tensor(x.reshape(-1), [3, 3])
+    ours = t.softmax(1)
+    reference = t.exp() / t.exp().sum(1)      # the reference's composition, through the same operators
+    for v in (ours, reference):
+        v.forward()
+        v.val().keep()
+    autodiff.execute()
+    e = np.exp(x.astype(np.float64))
+    got_ours = ours.val().get().numpy()
+    got_ref = reference.val().get().numpy()
+    np.testing.assert_allclose(got_ours, e / e.sum(1, keepdims=True), rtol=1e-6)
+    np.testing.assert_allclose(got_ref, e / e.sum(1)[None, :], rtol=1e-6)       # divided by the sum of row j
+    np.testing.assert_allclose(got_ours.sum(1), 1.0, rtol=1e-6)
+    assert np.abs(got_ref.sum(1) - 1.0).max() > 0.1
+    assert np.abs(got_ours - got_ref).max() > 0.05

@@ -724,6 +724,8 @@ def test_max_rows_and_columns(V, R, hip_device):
     if R > 1:
         x[V - 1, 0] = np.nan
         x[V // 2, :] = -np.inf
+    if V > 3 and R > 1:
+        x[1, :] = np.nan       # a row that is NaN throughout: its maximum is NaN (and so is every column's only if all of it is)
     cmds = [IR.CreateMat(x.reshape(-1), [V, R], "x"), IR.Max(a="x", res="rows"),
             IR.Permute(a="x", p=[1, 0], res="xt"), IR.Max(a="xt", res="cols")]
     got = _run_ir(hip_device, cmds, ["rows", "cols"])
