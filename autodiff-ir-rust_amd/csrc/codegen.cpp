@@ -184,6 +184,7 @@ struct Gen {
     std::vector<GenBuffer> bufs;
     std::set<const Node*> members;  // computed in this kernel, never loaded
     std::map<const Node*, std::string> preset;  // nodes whose value is a variable the kernel already holds
+    std::map<const Node*, std::string> preset_at;  // ... and, where given, the only index (aff_key) that variable stands for
     std::vector<LoadRec> loads;
     std::vector<Aff> recorded;  // every index expression over base atoms, for dim merging
     // Tiled element-wise kernels: loads whose key is in `stage_keys` are not issued by the thread that needs the value;
@@ -198,6 +199,13 @@ struct Gen {
     int row_atom = -1;
     int tmp = 0;
     double flops = 0;  // per lane element
+    // Row-chain kernels: a 128-bit load whose key is in `keep_keys` is held in a per-thread array indexed by the
+    // (fully unrolled) sweep counter `keep_index`, so that a later sweep takes it from registers; `sweep_loads`
+    // collects the keys of the vector loads the current sweep makes.
+    std::set<std::string> keep_keys, sweep_loads;
+    std::map<std::string, std::string> kept_arrays;
+    std::vector<std::string> kept_decls;
+    std::string keep_index;
 
     const char* idx_t() const { return wide ? "unsigned long long" : "unsigned int"; }
 
@@ -436,7 +444,18 @@ struct Gen {
             const std::string at = aff_str(base);
             std::string addr = nt ? strf("__builtin_nontemporal_load((const float4_t*)(%s + %s))", bp.c_str(), at.c_str())
                                   : strf("*(const float4_t*)(%s + %s)", bp.c_str(), at.c_str());
-            if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
+            if (pred.empty()) sweep_loads.insert(key);
+            if (pred.empty() && keep_keys.count(key)) {
+                auto kept = kept_arrays.find(key);
+                if (kept == kept_arrays.end()) {
+                    const std::string arr = "rk" + std::to_string(kept_arrays.size());
+                    kept_arrays[key] = arr;
+                    kept_decls.push_back(arr);
+                    emit(false, strf("const float4_t %sv = (%s[%s] = %s);", name.c_str(), arr.c_str(), keep_index.c_str(), addr.c_str()));
+                } else {
+                    emit(false, strf("const float4_t %sv = %s[%s];", name.c_str(), kept->second.c_str(), keep_index.c_str()));
+                }
+            } else if (pred.empty()) emit(false, strf("const float4_t %sv = %s;", name.c_str(), addr.c_str()));
             else emit(false, strf("float4_t %sv = {0.f, 0.f, 0.f, 0.f}; if (%s) %sv = %s;", name.c_str(), pred.c_str(), name.c_str(), addr.c_str()));
             if (pred.empty()) {
                 emit(false, strf("const float %s[4] = {%sv.x, %sv.y, %sv.z, %sv.w};", name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str()));
@@ -539,7 +558,12 @@ struct Gen {
     Val gen_node(const Node* n, const Aff& l, const std::string& pred) {
         {
             auto ps = preset.find(n);
-            if (ps != preset.end()) return {ps->second, false};
+            if (ps != preset.end()) {
+                auto at = preset_at.find(n);
+                ADHIP_CHECK(at == preset_at.end() || at->second == aff_key(l), "internal: node %d is held for index %s, wanted at %s", n->id,
+                            at->second.c_str(), aff_key(l).c_str());
+                return {ps->second, false};
+            }
         }
         if (in_memory(n)) return load(n, l, pred);
         if (n->op == Op::FILL) return {flit(n->cval), false};
@@ -1420,6 +1444,252 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         k.flops = (g.flops + 1) * (double)V * (double)R;
     }
     k.source = src;
+    return k;
+}
+
+// ---------------------------------------------------------------------------------------
+// row chains
+// ---------------------------------------------------------------------------------------
+
+RowAccess row_access(const TRef& t, int64_t V, int64_t R, bool row_level) {
+    if (!t.single_full() || t.pieces[0].src.kind != Src::NODE) return RowAccess::OTHER;
+    Gen g;
+    g.wide = true;
+    const int ax = g.add_atom("x", V, false);
+    Aff lin = row_level ? aff_atom(ax, 1) : aff_atom(ax, R);
+    int ay = -1;
+    if (!row_level) {
+        ay = g.add_atom("y", R, false);
+        lin = aff_add(lin, aff_atom(ay, 1));
+    }
+    const size_t before = g.atoms.size();
+    Aff idx;
+    try {
+        idx = g.apply_view_from(t.pieces[0].view, 0, lin);
+    } catch (const Error&) {
+        return RowAccess::OTHER;
+    }
+    if (g.atoms.size() != before || idx.c != 0) return RowAccess::OTHER;
+    if (idx.t.size() == 1 && idx.t[0].first == ax && idx.t[0].second == 1) return RowAccess::ROW;
+    if (!row_level && idx.t.size() == 2 && idx.t[0].first == ax && idx.t[0].second == R && idx.t[1].first == ay && idx.t[1].second == 1)
+        return RowAccess::FULL;
+    return RowAccess::OTHER;
+}
+
+bool rowchain_fits(int64_t V, int64_t R) {
+    if (V < 1 || R < 4 || R % 4 != 0) return false;
+    const int64_t RV = R / 4;
+    const int64_t T = RV <= 512 ? 64 : 256;
+    return (RV + T - 1) / T <= 8;
+}
+
+GeneratedKernel gen_rowchain_kernel(const RowChainSpec& spec) {
+    const int64_t V = spec.V, R = spec.R, RV = R / 4;
+    ADHIP_CHECK(rowchain_fits(V, R), "internal: rows of %lld elements do not fit a row-chain kernel", (long long)R);
+    const int T = RV <= 512 ? 64 : 256;             // threads per row: a wavefront, or the whole block
+    const int64_t K = (RV + T - 1) / T;             // sweeps' trip count: 128-bit pieces of the row per thread
+    const int rows_per_block = 256 / T;
+    const bool ragged = RV % T != 0;
+    const bool wide = needs_wide(spec.order) || V * R >= (int64_t(1) << 31) - 1024;
+    const bool nt_out = V * R >= nontemporal_min_elems();
+    int n_reduce = 0;
+    for (Node* m : spec.order) n_reduce += op_is_reduce(m->op) ? 1 : 0;
+
+    struct Sweep {
+        std::vector<std::string> codeA, codeB;
+        std::string value;          // reductions: the operand's value at this element
+        const Node* reduce = nullptr;
+        std::vector<std::string> after;                       // row-uniform statements that follow the sweep
+        std::vector<std::pair<const Node*, std::string>> row_values;  // stored one-per-row members: (node, expression)
+        std::vector<std::pair<const Node*, std::string>> outputs;     // last sweep: stored full-size members
+    };
+    struct Built {
+        Gen g;
+        std::vector<Sweep> sweeps;
+        std::map<std::string, int> load_sweeps;   // vector load key -> number of sweeps that make it
+        std::vector<std::string> head;             // row-uniform statements before the first sweep
+    };
+    auto build = [&](const std::set<std::string>& keep) {
+        Built b;
+        Gen& g = b.g;
+        g.vec = 4;
+        g.wide = wide;
+        g.keep_keys = keep;
+        g.keep_index = "it";
+        const int ax = g.add_atom("x", V, false), ay = g.add_atom("yv", RV, false);
+        g.lane_atom = g.add_atom("j", 4, true);
+        const Aff lin = aff_add(aff_add(aff_atom(ax, R), aff_atom(ay, 4)), aff_atom(g.lane_atom, 1));
+        const Aff at_x = aff_atom(ax, 1);
+        for (Node* m : spec.order) g.members.insert(m);
+        size_t a0 = 0, b0 = 0;
+        auto begin = [&] {
+            g.val_memo.clear();
+            g.atom_memo.clear();
+            g.sweep_loads.clear();
+            a0 = g.codeA.size();
+            b0 = g.codeB.size();
+        };
+        auto take = [&](std::vector<std::string>& A, std::vector<std::string>& B) {
+            A.assign(g.codeA.begin() + (long)a0, g.codeA.end());
+            B.assign(g.codeB.begin() + (long)b0, g.codeB.end());
+            g.codeA.resize(a0);
+            g.codeB.resize(b0);
+            for (const std::string& k : g.sweep_loads) b.load_sweeps[k] += 1;
+        };
+        Sweep* last = nullptr;       // the sweep whose `after` list takes row-uniform values
+        int ri = 0;
+        for (Node* m : spec.order) {
+            if (op_is_reduce(m->op)) {
+                ADHIP_CHECK(m->in.size() == 1 && m->in[0].shape == (Shape{V, R}), "internal: row-chain reduction over another space");
+                b.sweeps.emplace_back();
+                Sweep& sw = b.sweeps.back();
+                sw.reduce = m;
+                begin();
+                sw.value = g.gen_tref(m->in[0], lin, "").expr;
+                take(sw.codeA, sw.codeB);
+                const std::string name = strf("red%d", ri++);
+                g.preset[m] = name;
+                g.preset_at[m] = aff_key(at_x);
+                if (spec.stored.count(m)) sw.row_values.push_back({m, name});
+                last = &sw;
+            } else if (numel(m->shape) == V && V != V * R) {
+                // one value per row: row-uniform code behind the sweep that finished what it needs
+                ADHIP_CHECK(op_is_elw(m->op), "internal: row-chain member of the wrong kind");
+                begin();
+                const int vec_saved = g.vec, lane_saved = g.lane_atom;
+                g.vec = 1;
+                g.lane_atom = -1;
+                const Val v = g.gen_node(m, at_x, "");
+                g.vec = vec_saved;
+                g.lane_atom = lane_saved;
+                std::vector<std::string> A, B;
+                take(A, B);
+                ADHIP_CHECK(B.empty(), "internal: a per-row value produced per-lane code");
+                const std::string name = strf("rv%d", g.tmp++);
+                A.push_back(strf("const float %s = %s;", name.c_str(), v.expr.c_str()));
+                g.preset[m] = name;
+                g.preset_at[m] = aff_key(at_x);
+                std::vector<std::string>& dst = last ? last->after : b.head;
+                dst.insert(dst.end(), A.begin(), A.end());
+                if (spec.stored.count(m)) {
+                    ADHIP_CHECK(last, "internal: a stored per-row value before the first sweep of a row chain");
+                    last->row_values.push_back({m, name});
+                }
+            } else {
+                ADHIP_CHECK(op_is_elw(m->op) && numel(m->shape) == V * R, "internal: row-chain member of the wrong size");
+            }
+        }
+        // the last sweep evaluates and stores the full-size members
+        b.sweeps.emplace_back();
+        Sweep& fin = b.sweeps.back();
+        begin();
+        for (Node* m : spec.order)
+            if (!op_is_reduce(m->op) && numel(m->shape) == V * R && spec.stored.count(m)) fin.outputs.push_back({m, g.gen_node(m, lin, "").expr});
+        take(fin.codeA, fin.codeB);
+        return b;
+    };
+    std::set<std::string> keep;
+    {
+        Built dry = build({});
+        for (auto& kv : dry.load_sweeps)
+            if (kv.second >= 2) keep.insert(kv.first);
+        // a kept stream costs 4 K registers a thread
+        while ((int64_t)keep.size() * 4 * K > 160) keep.erase(std::prev(keep.end()));
+    }
+    Built b = build(keep);
+    Gen& g = b.g;
+    if (b.sweeps.back().outputs.empty()) b.sweeps.pop_back();
+
+    GeneratedKernel k;
+    k.kind = "rowchain";
+    k.entry = spec.name;
+    const char* it_t = g.idx_t();
+    const char* sfx = wide ? "ull" : "u";
+    // no __restrict__: a stored member may share its buffer with an operand it replaces in place
+    std::string sig = "const int* __restrict__ guard";
+    std::vector<Node*> order;
+    std::map<const Node*, std::string> out_param;
+    for (Node* m : spec.order)
+        if (spec.stored.count(m)) {
+            out_param[m] = strf("w%zu", out_param.size());
+            sig += ", float* " + out_param[m];
+            order.push_back(m);
+        }
+    for (auto& gb : g.bufs) { sig += ", const float* " + gb.param; order.push_back(gb.node); }
+    std::string src = kernel_prelude();
+    src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+    src += "    if (guard && *guard == 0) return;\n";
+    if (T == 256 && n_reduce > 0) src += strf("    __shared__ float part[%d][4];\n", n_reduce);
+    src += strf("    const unsigned lane = threadIdx.x %% %du;\n", T);
+    src += strf("    const %s x_raw = (%s)blockIdx.x * %du + threadIdx.x / %du;\n", it_t, it_t, rows_per_block, T);
+    // a row beyond the last one works on the last one and stores nothing: no thread leaves early
+    src += strf("    const bool row_ok = x_raw < %lld%s;\n    const %s x = row_ok ? x_raw : %lld%s;\n", (long long)V, sfx, it_t, (long long)(V - 1), sfx);
+    for (const std::string& arr : g.kept_decls) src += strf("    float4_t %s[%lld];\n", arr.c_str(), (long long)K);
+    src += join(b.head, "    ");
+    int ri = 0;
+    for (size_t si = 0; si < b.sweeps.size(); ++si) {
+        Sweep& sw = b.sweeps[si];
+        const bool mx = sw.reduce && sw.reduce->op == Op::MAX;
+        const char* ident = mx ? "__builtin_nanf(\"\")" : "0.0f";
+        if (sw.reduce) src += strf("    float acc%d[4] = {%s, %s, %s, %s};\n", ri, ident, ident, ident, ident);
+        src += strf("#pragma unroll\n    for (unsigned it = 0; it < %lldu; ++it) {\n", (long long)K);
+        if (ragged) src += strf("        const %s yv_raw = lane + it * %du;\n        const bool live = yv_raw < %lldu;\n        const %s yv = live ? yv_raw : %lldu;\n",
+                                it_t, T, (long long)RV, it_t, (long long)(RV - 1));
+        else src += strf("        const %s yv = lane + it * %du;\n", it_t, T);
+        src += join(sw.codeA, "        ");
+        for (size_t i = 0; i < sw.outputs.size(); ++i) src += strf("        float o%zu[4];\n", i);
+        src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+        src += join(sw.codeB, "            ");
+        if (sw.reduce) {
+            const std::string a = strf("acc%d[j]", ri);
+            const std::string c = mx ? "fmaxf(" + a + ", " + sw.value + ")" : a + " + " + sw.value;
+            src += strf("            %s%s = %s;\n", ragged ? "if (live) " : "", a.c_str(), c.c_str());
+        }
+        for (size_t i = 0; i < sw.outputs.size(); ++i) src += strf("            o%zu[j] = %s;\n", i, sw.outputs[i].second.c_str());
+        src += "        }\n";
+        if (!sw.outputs.empty()) {
+            src += strf("        if (row_ok%s) {\n", ragged ? " && live" : "");
+            for (size_t i = 0; i < sw.outputs.size(); ++i)
+                src += "            " + store4_stmt(strf("o%zu", i), strf("%s + (%lld%s * x + 4u * yv)", out_param[sw.outputs[i].first].c_str(), (long long)R, sfx), nt_out) + "\n";
+            src += "        }\n";
+        }
+        src += "    }\n";
+        if (sw.reduce) {
+            const std::string a = strf("acc%d", ri);
+            const std::string s4 = mx ? strf("fmaxf(fmaxf(%s[0], %s[1]), fmaxf(%s[2], %s[3]))", a.c_str(), a.c_str(), a.c_str(), a.c_str())
+                                      : strf("(%s[0] + %s[1]) + (%s[2] + %s[3])", a.c_str(), a.c_str(), a.c_str(), a.c_str());
+            if (T == 64) {
+                src += strf("    const float red%d = %s(%s);\n", ri, mx ? "wave_max" : "wave_sum", s4.c_str());
+            } else {
+                src += strf("    { const float s = %s(%s); if ((threadIdx.x & 63u) == 0) part[%d][threadIdx.x >> 6] = s; }\n    __syncthreads();\n",
+                            mx ? "wave_max" : "wave_sum", s4.c_str(), ri);
+                src += mx ? strf("    const float red%d = fmaxf(fmaxf(part[%d][0], part[%d][1]), fmaxf(part[%d][2], part[%d][3]));\n", ri, ri, ri, ri, ri)
+                          : strf("    const float red%d = (part[%d][0] + part[%d][1]) + (part[%d][2] + part[%d][3]);\n", ri, ri, ri, ri, ri);
+            }
+            ++ri;
+        }
+        src += join(sw.after, "    ");
+    }
+    // one value per row: stored last, by the row's first lane, when every thread of the row has read what it needed
+    bool any_row_value = false;
+    for (Sweep& sw : b.sweeps) any_row_value = any_row_value || !sw.row_values.empty();
+    if (any_row_value) {
+        if (T == 256) src += "    __syncthreads();\n";
+        src += "    if (lane == 0u && row_ok) {\n";
+        for (Sweep& sw : b.sweeps)
+            for (auto& rv : sw.row_values) src += strf("        %s[x] = %s;\n", out_param[rv.first].c_str(), rv.second.c_str());
+        src += "    }\n";
+    }
+    src += "}\n";
+    k.source = src;
+    k.buffer_args = order;
+    k.block[0] = 256;
+    k.grid[0] = (unsigned)((V + rows_per_block - 1) / rows_per_block);
+    k.bytes = 0;
+    for (Node* m : spec.order)
+        if (spec.stored.count(m)) k.bytes += 4.0 * (double)numel(m->shape);
+    for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), V * R);
+    k.flops = (g.flops + n_reduce) * (double)V * (double)R;
     return k;
 }
 

@@ -85,6 +85,28 @@ GeneratedKernel gen_elw_kernel(const ElwKernelSpec& spec, const std::set<const N
 // Reduce over the last dim of a [V,R] operand.  If the result needs `chunks > 1`, the kernel writes
 // partial sums laid out [chunks][V]; the caller reduces those with a second (column) reduction over the partials.
 GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_chunks = 0);
+// A chain of row reductions and element-wise values over one [V, R] space that depend on one another row by row (max ->
+// exp(x - max) -> sum -> divide; mean -> x - mean -> variance -> normalise): one kernel in which a wavefront (rows of
+// up to 2048 elements) or a block owns a row.  Every reduction is a sweep over the row; what a sweep loads that a later
+// sweep needs again stays in registers, so the row is read from memory once and each stored value written once.
+struct RowChainSpec {
+    int64_t V = 0, R = 0;
+    std::string name;
+    // every member, producers first: reductions of a [V, R] operand, element-wise values of V elements (one per row)
+    // and element-wise values of V * R elements
+    std::vector<Node*> order;
+    std::set<const Node*> stored;  // the members that are written to memory; the others only exist inside the kernel
+};
+// How a tensor reference, evaluated at the element (x, y) of a [V, R] space (or, with `row_level`, at row x alone),
+// addresses its source: FULL -- element x * R + y of it (the same element); ROW -- element x (one value per row);
+// OTHER -- anything else.
+enum class RowAccess { FULL, ROW, OTHER };
+RowAccess row_access(const TRef& t, int64_t V, int64_t R, bool row_level);
+// whether rows of R elements fit the kernel (a thread holds at most 8 x 4 elements of each operand)
+bool rowchain_fits(int64_t V, int64_t R);
+// buffer_args: the stored members in the order of `order`, then the operands
+GeneratedKernel gen_rowchain_kernel(const RowChainSpec& spec);
+
 // Number of row tiles an element-wise kernel with column sums over [rows, cols] that moves `streams` full-size
 // streams (ElwKernelSpec::streams) will use.
 int64_t elw_colsum_tiles(int64_t rows, int64_t cols, int streams);

@@ -290,7 +290,7 @@ using RegionKey = std::pair<const Proc*, size_t>;
 struct Group {
     std::vector<Node*> members;
     int64_t n = 0;
-    enum Kind { ELW, SUM, DOT, TRANSPOSE, ATTN } kind = ELW;
+    enum Kind { ELW, SUM, DOT, TRANSPOSE, ATTN, ROWCHAIN } kind = ELW;
     // column sums computed by this element-wise kernel: (value node, SUM node that wanted it)
     std::vector<std::pair<Node*, Node*>> colsums;
     // row sums computed by this element-wise kernel, likewise: every wavefront adds up its run of a row, the runs of a
@@ -308,6 +308,8 @@ struct Group {
     std::vector<Node*> side;
     // element-wise values of the result's size that the reduction evaluates and stores right after summing
     std::vector<Node*> epi;
+    // ROWCHAIN: members that only exist inside the kernel (nobody outside the chain reads them, no id holds them)
+    std::set<Node*> unstored;
     bool dead = false;  // its only member was absorbed by another group
     bool tiled = false; // fetches an operand read against the grain through LDS tiles (takes no sums along)
     int lead = -1;      // >= 0: runs inside the launches of that group (same kernels on other buffers), which it follows directly
@@ -1298,7 +1300,7 @@ struct Lowerer {
     // in order with a block-wide barrier in between, which is also what makes one phase's global writes visible to the
     // next.  Only kernel kinds in which no thread leaves before a barrier the others still reach.
     void merge_single_block_runs(std::vector<Step>& out, size_t from) {
-        static const std::set<std::string> mergeable = {"elw", "reduce_row", "reduce_row_store", "reduce_col", "dot_naive", "copy"};
+        static const std::set<std::string> mergeable = {"elw", "reduce_row", "reduce_row_store", "reduce_col", "dot_naive", "copy", "rowchain"};
         auto single_block = [&](const Step& st) {
             if (st.kind != Step::LAUNCH) return false;
             const Launch& l = st.launch;
@@ -1394,6 +1396,7 @@ struct Lowerer {
         form_groups(rp);
         if (opt.fuse) {
             attach_column_sums(rp);
+            if (opt.row_chains) form_row_chains(rp);
             attach_row_sum_operands(rp);
             fold_transposed_copies(rp);
             attach_row_sums(rp);
@@ -2074,6 +2077,144 @@ struct Lowerer {
         }
     }
 
+    // ---- 5b''. Row chains: a row reduction whose result the following kernels use row by row -- a softmax (max, the
+    // sum of the exponentials, the division), a LayerNorm (mean, the centred value, the variance, the scaling), the
+    // backward pass of either -- runs as one kernel in which a wavefront or a block owns a row (gen_rowchain_kernel):
+    // the row is read from memory once, and what only the chain itself uses is never written.  A chain is a run of
+    // consecutive kernels over one [V, R] space: plain row reductions, element-wise kernels of V * R elements and
+    // element-wise kernels of V elements, each of which reads what the chain produced before it only at its own row
+    // (the same element of a full-size value, element x of a per-row value).
+    bool chain_reads_rowwise(RegionPlan& rp, Node* m, const std::set<Node*>& produced, int64_t V, int64_t R) {
+        bool ok = true;
+        std::function<bool(Node*)> reaches = [&](Node* n) {
+            bool r = false;
+            for_each_src(n, [&](Node* s, const Piece&, const TRef&) {
+                if (r) return;
+                if (produced.count(s)) r = true;
+                else if (!in_mem(s)) r = reaches(s);
+            });
+            return r;
+        };
+        std::set<std::pair<Node*, bool>> seen;
+        std::function<void(Node*, bool)> walk = [&](Node* n, bool row_level) {
+            for (const TRef& t : n->in) {
+                for (const Piece& p : t.pieces) {
+                    if (!ok || p.src.kind != Src::NODE) continue;
+                    Node* s = p.src.node;
+                    const bool mine = produced.count(s) != 0;
+                    if (!mine && in_mem(s)) continue;                       // an operand from outside: read however it likes
+                    const RowAccess ra = row_access(t, V, R, row_level);
+                    const int64_t ns = numel(s->shape);
+                    const bool aligned = (ra == RowAccess::FULL && ns == V * R) || (ra == RowAccess::ROW && ns == V);
+                    if (mine) { if (!aligned) ok = false; continue; }
+                    // a folded value: followed at the coordinates it is evaluated at, if those are a row's
+                    if (aligned) { if (seen.insert({s, ra == RowAccess::ROW}).second) walk(s, ra == RowAccess::ROW); }
+                    else if (reaches(s)) ok = false;
+                }
+            }
+        };
+        walk(m, !op_is_reduce(m->op) && numel(m->shape) == V);
+        (void)rp;
+        return ok;
+    }
+
+    void form_row_chains(RegionPlan& rp) {
+        if (tight()) return;
+        auto& groups = rp.groups;
+        auto& reads = rp.reads;
+        auto plain_reduction = [&](const Group& H, int64_t& V, int64_t& R) {
+            if (H.dead || H.kind != Group::SUM || H.members.size() != 1 || !H.side.empty() || !H.epi.empty() || H.lead >= 0) return false;
+            const Node* n = H.members[0];
+            if (!op_is_reduce(n->op) || n->in.size() != 1 || n->in[0].shape.size() != 2) return false;
+            V = n->in[0].shape[0];
+            R = n->in[0].shape[1];
+            return true;
+        };
+        for (size_t g0 = 0; g0 < groups.size(); ++g0) {
+            int64_t V = 0, R = 0;
+            if (!plain_reduction(groups[g0], V, R) || V < 2 || !rowchain_fits(V, R)) continue;
+            std::vector<size_t> run;
+            std::set<Node*> produced, streamed;
+            auto acceptable = [&](const Group& H) {
+                int64_t v2 = 0, r2 = 0;
+                if (H.kind == Group::SUM) {
+                    if (!plain_reduction(H, v2, r2) || v2 != V || r2 != R) return false;
+                } else if (H.kind == Group::ELW) {
+                    if (H.rides() || H.tiled || !H.side.empty() || H.lead >= 0 || (H.n != V * R && H.n != V)) return false;
+                } else {
+                    return false;
+                }
+                for (Node* m : H.members)
+                    if (!chain_reads_rowwise(rp, m, produced, V, R)) return false;
+                // it belongs to the chain if it uses what the chain made, or streams a full-size operand the chain
+                // streams anyway; independent work on other data stays a kernel of its own
+                if (produced.empty()) return true;
+                for (Node* m : H.members)
+                    for (auto& rd : reads[m])
+                        if (produced.count(rd.first) || (streamed.count(rd.first) && numel(rd.first->shape) * 2 >= V * R)) return true;
+                return false;
+            };
+            for (size_t h = g0; h < groups.size(); ++h) {
+                if (groups[h].dead) continue;
+                if (!acceptable(groups[h])) break;
+                run.push_back(h);
+                for (Node* m : groups[h].members) {
+                    produced.insert(m);
+                    for (auto& rd : reads[m]) streamed.insert(rd.first);
+                }
+            }
+            // the chain pays when something that works on whole rows uses what the chain made before it; it ends with
+            // the last such kernel (per-row arithmetic that follows gains nothing from sharing the launch)
+            auto members_of = [&](size_t upto) {
+                std::vector<Node*> ms;
+                for (size_t i = 0; i < upto; ++i) {
+                    std::vector<Node*> part = groups[run[i]].members;
+                    std::stable_sort(part.begin(), part.end(), [](Node* a, Node* b) { return a->order < b->order; });
+                    ms.insert(ms.end(), part.begin(), part.end());
+                }
+                return ms;
+            };
+            size_t len = run.size();
+            for (; len >= 2; --len) {
+                std::vector<Node*> ms = members_of(len);
+                std::set<Node*> earlier(ms.begin(), ms.end());
+                for (Node* m : groups[run[len - 1]].members) earlier.erase(m);
+                Node* tail = ms.back();
+                bool uses = false;
+                if (op_is_reduce(tail->op) || numel(tail->shape) == V * R)
+                    for (Node* m : groups[run[len - 1]].members)
+                        for (auto& rd : reads[m]) uses = uses || earlier.count(rd.first) != 0;
+                if (!uses) continue;
+                // the kernel's size is bounded like any other's
+                Group probe;
+                probe.members = ms;
+                if (!group_fits(rp, probe, nullptr)) continue;
+                // and it has to generate (a reference the generator cannot follow ends the attempt, not the lowering)
+                RowChainSpec spec;
+                spec.V = V;
+                spec.R = R;
+                spec.name = "probe";
+                spec.order = ms;
+                for (Node* m : ms) spec.stored.insert(m);
+                try {
+                    (void)gen_rowchain_kernel(spec);
+                } catch (const Error&) {
+                    continue;
+                }
+                break;
+            }
+            if (len < 2) continue;
+            Group& G = groups[g0];
+            G.kind = Group::ROWCHAIN;
+            G.members = members_of(len);
+            G.n = V * R;
+            G.cs_rows = V;
+            G.cs_cols = R;
+            for (size_t i = 1; i < len; ++i) groups[run[i]].dead = true;
+            for (Node* m : G.members) rp.group_of[m] = (int)g0;
+        }
+    }
+
     // ---- 5c. a row sum over an element-wise value produced by the kernel just before it: the
     // reduction computes, stores and sums that value in one pass
     void attach_row_sum_operands(RegionPlan& rp) {
@@ -2311,6 +2452,21 @@ struct Lowerer {
                         gks[g].dot_store = needed;
                     }
                 }
+            } else if (G.kind == Group::ROWCHAIN) {
+                // a member is written to memory only if an id holds it or a kernel outside the chain reads it
+                RowChainSpec spec;
+                spec.V = G.cs_rows;
+                spec.R = G.cs_cols;
+                spec.name = name;
+                spec.order = G.members;
+                for (Node* m : G.members) {
+                    bool needed = home_of.count(m) != 0;
+                    for (size_t g2 = 0; g2 < groups.size() && !needed; ++g2)
+                        if (g2 != g && !groups[g2].dead && group_reads(rp, groups[g2], m)) needed = true;
+                    if (needed) spec.stored.insert(m);
+                    else G.unstored.insert(m);
+                }
+                gks[g].k = gen_rowchain_kernel(spec);
             } else if (G.kind == Group::SUM) {
                 ReduceKernelSpec spec;
                 spec.node = G.members[0];
@@ -2382,7 +2538,7 @@ struct Lowerer {
         std::map<std::vector<int64_t>, std::vector<size_t>> by_signature;
         for (size_t g = 0; g < n_groups; ++g) {
             Group& H = groups[g];
-            if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM) || H.rides() || updates_in_place(H)) continue;
+            if (H.dead || (H.kind != Group::ELW && H.kind != Group::SUM && H.kind != Group::ROWCHAIN) || H.rides() || updates_in_place(H)) continue;
             std::vector<int64_t> sig;
             bool ok = true;
             auto add = [&](const GeneratedKernel& k) {
@@ -2489,6 +2645,8 @@ struct Lowerer {
             for (Node* sd : groups[g].side) produced.push_back(sd);
             for (Node* ep : groups[g].epi) produced.push_back(ep);
             if (groups[g].kind == Group::DOT && !gks[g].dot_store) produced.erase(produced.begin());  // lives in registers only
+            if (groups[g].kind == Group::ROWCHAIN)
+                produced.erase(std::remove_if(produced.begin(), produced.end(), [&](Node* m) { return groups[g].unstored.count(m) != 0; }), produced.end());
             for (Node* m : produced) {
                 auto ho = home_of.find(m);
                 bool direct = false;
@@ -2502,12 +2660,18 @@ struct Lowerer {
                                              std::find(groups[g].epi.begin(), groups[g].epi.end(), m) != groups[g].epi.end();
                         const bool is_member = is_side || (groups[g].kind == Group::ELW &&
                             std::find(groups[g].members.begin(), groups[g].members.end(), m) != groups[g].members.end());
+                        // a row chain reads all it needs of a row before it stores any of it: it may overwrite a value
+                        // that its members read only at the row (and element) they work on
+                        bool chain_in_place = groups[g].kind == Group::ROWCHAIN;
+                        if (chain_in_place)
+                            for (Node* cm : groups[g].members)
+                                chain_in_place = chain_in_place && chain_reads_rowwise(rp, cm, std::set<Node*>{old}, groups[g].cs_rows, groups[g].cs_cols);
                         for (size_t g2 = 0; g2 < groups.size(); ++g2) {
                             if (groups[g2].dead) continue;
                             auto it = greads[g2].find(old);
                             if (it == greads[g2].end()) continue;
                             if (g2 > g) direct = false;
-                            if (g2 == g && !(it->second && is_member)) {
+                            if (g2 == g && !(it->second && is_member) && !chain_in_place) {
                                 // a reduction may still update its result in place when it reads the old result only
                                 // at the position it is about to write (s = Sum(f(x, s broadcast along the reduced
                                 // dim))): the block that owns an output element loads before it stores, and a
@@ -3608,6 +3772,7 @@ std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::str
     if (const char* e = getenv("ADHIP_LAYER_KERNELS")) opt.layer_kernels = opt.layer_kernels && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_MERGE_SMALL")) opt.merge_small = opt.merge_small && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_FUSE_ATTENTION")) opt.fuse_attention = opt.fuse_attention && atoi(e) != 0;
+    if (const char* e = getenv("ADHIP_ROW_CHAINS")) opt.row_chains = opt.row_chains && atoi(e) != 0;
     // diagnostic: the seven kernel-size bounds, in the order LowerOptions declares them ("24,48,32,96,40,24,20")
     if (const char* e = getenv("ADHIP_KERNEL_BOUNDS")) {
         int* field[7] = {&opt.max_pieces, &opt.max_inline_sites, &opt.max_inline_loads, &opt.max_kernel_sites, &opt.max_kernel_pointers,

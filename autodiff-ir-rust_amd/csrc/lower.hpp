@@ -19,6 +19,7 @@ struct LowerOptions {
     bool layer_kernels = true;  // groups that run the same generated kernels on other buffers share their launches
     bool merge_small = true;    // consecutive single-block launches of a region run as phases of one launch
     bool fuse_attention = true;  // dot(softmax(scale * dot(Q, K^T)), V) runs as one kernel
+    bool row_chains = true;      // row reductions and the element-wise values between them run as one kernel per row
     // Bounds on the size of one generated kernel, in what drives its register pressure: the places it loads from
     // (a tensor reference with several concat pieces loads once per piece, under a predicate) and the buffers it
     // names.  Beyond them values are cut out into kernels of their own.

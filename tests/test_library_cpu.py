@@ -515,10 +515,10 @@ def test_layered_launches_plan_and_compile():
     for seed in range(30):
         proc, keep = random_layered_program(seed)
         text = lower_describe(proc, set(keep))
-        counts = [int(c) for c in re.findall(r"launch \w+_x(\d+) \[", text)]
+        counts = [int(c) for c in re.findall(r"launch k\w+_x(\d+) \[", text)]
         assert all(2 <= c <= 16 for c in counts), text
         for line in text.splitlines():
-            m = re.search(r"launch \w+_x(\d+) \[\w+\] kernel=\w+ grid=\((\d+),(\d+),(\d+)\)", line)
+            m = re.search(r"launch k\w+_x(\d+) \[\w+\] kernel=\w+ grid=\((\d+),(\d+),(\d+)\)", line)
             if m:
                 assert m.group(1) == m.group(4), line
         layered += len(counts)

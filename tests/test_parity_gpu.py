@@ -287,7 +287,8 @@ def test_random_model_programs(scale, seed, hip_device):
     computation that shares no code with the caller side.  Where a value is the outcome of cancellation (the
     gradient of a sum of softmax rows is exactly 0), the oracle's own distance from the float64 answer says how well
     float32 can know it, and the device may be a few times that far from it; otherwise 1e-5 sqrt(N) of the value's own
-    largest element, N = the most terms any Sum or DotProduct of the program adds."""
+    largest element, N = the most terms any Sum or DotProduct of the program adds -- and never less than that fraction
+    of a thousandth of the program's largest value, below which a number is the rounding noise of larger terms."""
     print(f"[case] model fuzz scale {scale} seed {seed}", flush=True)
     from fuzz_models import random_model_program, shadow_model_program
     got = random_model_program(hip_device, seed, scale)
@@ -306,9 +307,10 @@ def test_random_model_programs(scale, seed, hip_device):
         assert e.shape == r.shape, f"{k}: {exact[k].shape} vs {rv.dim}"
         own = float(np.max(np.abs(e))) if e.size else 0.0
         oracle_err = float(np.max(np.abs(r - e))) if e.size else 0.0
-        assert oracle_err <= tol * max(own, 1e-3 * max(float(np.max(np.abs(x))) for x in exact.values())), \
+        largest = max(float(np.max(np.abs(x))) for x in exact.values())
+        assert oracle_err <= tol * max(own, 1e-3 * largest), \
             f"scale {scale} seed {seed} {k}: the oracle is {oracle_err:.3e} from float64 (own scale {own:.3e})"
-        allowed = max(tol * own, 8.0 * oracle_err)
+        allowed = max(tol * own, 8.0 * oracle_err, tol * 1e-3 * largest)
         err = float(np.max(np.abs(g - e))) if e.size else 0.0
         assert err <= allowed, f"scale {scale} seed {seed} {k}: |device - float64| = {err:.3e} > {allowed:.3e} (own scale {own:.3e}, oracle {oracle_err:.3e})"
         assert float(np.max(np.abs(g - r))) <= 2 * allowed if e.size else True
