@@ -196,6 +196,7 @@ struct Gen {
     std::vector<Staged> staged;
     std::vector<std::string> index_code;
     std::string tile_row_origin, tile_col_origin;  // expressions of the tile's first row / first column
+    int tile_rows = 64, tile_cols = 64;
     int row_atom = -1;
     int tmp = 0;
     double flops = 0;  // per lane element
@@ -881,12 +882,29 @@ static GeneratedKernel gen_elw_colsum_kernel(const ElwKernelSpec& spec, const st
 // staging phase evaluates the very index expression the body would have used, at the coordinates of the element it
 // fetches, so whatever view or concat piece the operand sits behind is handled by construction.
 // Returns false (and leaves `k` alone) when the pass has no such operand or not the shape for it.
+// Tile of the tiled element-wise kernel: 64 rows x 64 columns of the two innermost iteration extents.  The staged
+// operand is read in runs of the tile's rows, the results are written in runs of its columns.  Measured on the gather
+// stage of the manipulation workload (1 staged operand, 2 results, 453 MB): 64x64 77.3 us, 64x128 77.0, 128x64 77.9,
+// 128x128 77.5, 64x256 80.3 -- the length of the runs is not what bounds it.  ADHIP_TILED_SHAPE=<rows>x<cols>
+// (64 or 128 rows; 64, 128 or 256 columns) picks another tile, as a diagnostic.
+static void tiled_shape(int64_t& TR, int64_t& TC) {
+    TR = 64;
+    TC = 64;
+    if (const char* e = getenv("ADHIP_TILED_SHAPE")) {
+        long r = 0, c = 0;
+        if (sscanf(e, "%ldx%ld", &r, &c) == 2 && (r == 64 || r == 128) && (c == 64 || c == 128 || c == 256)) { TR = r; TC = c; }
+    }
+}
+
 static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const Node*>& members, const Shape& shape, bool wide,
                                  GeneratedKernel& k) {
     const size_t nd = shape.size();
     if (nd < 2) return false;
     const int64_t I = shape[nd - 1], Rws = shape[nd - 2];
-    if (I % 4 != 0 || I < 32 || Rws < 32) return false;   // tiles are 64x64: smaller extents leave most of a block idle
+    if (I % 4 != 0 || I < 32 || Rws < 32) return false;   // tiles are at least 64x64: smaller extents leave most of a block idle
+    int64_t TR = 64, TC = 64;
+    tiled_shape(TR, TC);
+    if ((TR * TC / 1024) * (int64_t)spec.outputs.size() > 32) { TR = 64; TC = 64; }   // a thread's share of the results stays in registers
     const int64_t N = numel(spec.outputs[0]->shape);
     std::set<std::string> keys;
     {
@@ -904,12 +922,15 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
         }
     }
     if (keys.empty() || keys.size() > 2) return false;
+    if (keys.size() * (size_t)(TC * (TR + 1) * 4) > 80 * 1024) { TR = 64; TC = 64; }   // two blocks' staging tiles fit a CU's 160 KB
     const std::string sfx = wide ? "ull" : "u";
     ElwBody b = elw_body(spec, members, shape, 4, wide, [&](Gen& g) {
         g.stage_keys = keys;
         g.row_atom = (int)nd - 2;
         g.tile_row_origin = "row0";
         g.tile_col_origin = "col0";
+        g.tile_rows = (int)TR;
+        g.tile_cols = (int)TC;
     });
     Gen& g = b.g;
     if (g.staged.empty()) return false;
@@ -921,7 +942,11 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
     std::vector<Node*> order;
     for (size_t i = 0; i < spec.outputs.size(); ++i) { sig += strf(", float* o%zu", i); order.push_back(spec.outputs[i]); }
     for (auto& gb : g.bufs) { sig += ", const float* " + gb.param; order.push_back(gb.node); }
-    const int64_t TI = (I + 63) / 64, TJ = (Rws + 63) / 64;
+    const int64_t TI = (I + TC - 1) / TC, TJ = (Rws + TR - 1) / TR;
+    const int64_t NS = TR * TC / 256;          // staging loads per thread
+    const int64_t QC = TC / 4;                 // float4 columns of a tile
+    const int64_t RP = 256 / QC;               // rows of a tile that one pass of the block covers
+    const int64_t NP = TR / RP;                // passes
     int64_t outer = 1;
     for (size_t d = 0; d + 2 < nd; ++d) outer *= shape[d];
     const int64_t blocks = TI * TJ * outer;
@@ -930,11 +955,11 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
     std::string src = kernel_prelude();
     src += strf("extern \"C\" __global__ __launch_bounds__(256) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
     src += "    if (guard && *guard == 0) return;\n";
-    for (auto& st : g.staged) src += strf("    __shared__ float tile%d[64][65];\n", st.slot);
+    for (auto& st : g.staged) src += strf("    __shared__ float tile%d[%lld][%lld];\n", st.slot, (long long)TC, (long long)(TR + 1));
     src += "    const unsigned tid = threadIdx.x;\n";
     src += strf("    %s bid = blockIdx.x;\n", it);
-    src += strf("    const %s col0 = (bid %% %lld%s) * 64u;\n    bid /= %lld%s;\n", it, (long long)TI, sfx.c_str(), (long long)TI, sfx.c_str());
-    src += strf("    const %s row0 = (bid %% %lld%s) * 64u;\n    bid /= %lld%s;\n", it, (long long)TJ, sfx.c_str(), (long long)TJ, sfx.c_str());
+    src += strf("    const %s col0 = (bid %% %lld%s) * %lldu;\n    bid /= %lld%s;\n", it, (long long)TI, sfx.c_str(), (long long)TC, (long long)TI, sfx.c_str());
+    src += strf("    const %s row0 = (bid %% %lld%s) * %lldu;\n    bid /= %lld%s;\n", it, (long long)TJ, sfx.c_str(), (long long)TR, (long long)TJ, sfx.c_str());
     for (size_t d = nd - 2; d-- > 0;) {
         if (d == 0) src += strf("    const %s c0 = bid;\n", it);
         else src += strf("    const %s c%zu = bid %% %lld%s;\n    bid /= %lld%s;\n", it, d, (long long)shape[d], sfx.c_str(), (long long)shape[d], sfx.c_str());
@@ -944,9 +969,9 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
     // outside the tensor or the operand's piece reads index 0 and is replaced by 0 afterwards), because a load under
     // a condition becomes a branch with a wait behind it, and the 16 memory latencies of a block then add up (that
     // version ran at 0.60 of the HBM peak with every wavefront waiting 88 % of its life).
-    for (auto& st : g.staged) src += strf("    float sv%d[16];\n", st.slot);
-    src += "#pragma unroll\n    for (unsigned k = 0; k < 16u; ++k) {\n";
-    src += "        const unsigned lj = tid & 63u, li = (tid >> 6) + 4u * k;\n";
+    for (auto& st : g.staged) src += strf("    float sv%d[%lld];\n", st.slot, (long long)NS);
+    src += strf("#pragma unroll\n    for (unsigned k = 0; k < %lldu; ++k) {\n", (long long)NS);
+    src += strf("        const unsigned lj = tid %% %lldu, li = tid / %lldu + %lldu * k;\n", (long long)TR, (long long)TR, (long long)(256 / TR));
     src += strf("        const %s %s = row0 + lj;\n        const %s ii = col0 + li;\n", it, rowv.c_str(), it);
     src += strf("        const %s %s = ii >> 2;\n        const %s j = ii & 3u;\n", it, colv.c_str(), it);
     src += strf("        const bool inside = %s < %lld%s && ii < %lld%s;\n", rowv.c_str(), (long long)Rws, sfx.c_str(), (long long)I, sfx.c_str());
@@ -956,19 +981,19 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
                     st.pred.empty() ? "" : " && ", st.pred.c_str(), st.param.c_str(), st.index.c_str(), st.slot);
     }
     src += "    }\n";
-    src += "#pragma unroll\n    for (unsigned k = 0; k < 16u; ++k) {\n";
-    for (auto& st : g.staged) src += strf("        tile%d[(tid >> 6) + 4u * k][tid & 63u] = sv%d[k];\n", st.slot, st.slot);
+    src += strf("#pragma unroll\n    for (unsigned k = 0; k < %lldu; ++k) {\n", (long long)NS);
+    for (auto& st : g.staged) src += strf("        tile%d[tid / %lldu + %lldu * k][tid %% %lldu] = sv%d[k];\n", st.slot, (long long)TR, (long long)(256 / TR), (long long)TR, st.slot);
     src += "    }\n    __syncthreads();\n";
     // compute: a thread owns four adjacent columns of four rows of the tile
-    src += "    const unsigned lc = tid & 15u, lr = tid >> 4;\n";
+    src += strf("    const unsigned lc = tid %% %lldu, lr = tid / %lldu;\n", (long long)QC, (long long)QC);
     // the four rows' values are computed first and stored afterwards: a result may share its buffer with an operand,
     // so the compiler cannot move the next row's loads above this row's stores by itself, and the rows' memory
     // latencies would add up
-    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("    float keep%zu[4][4];\n", i);
-    src += strf("    %s at[4];\n    bool live[4];\n", it);
-    src += "#pragma unroll\n    for (unsigned k = 0; k < 4u; ++k) {\n";
+    for (size_t i = 0; i < spec.outputs.size(); ++i) src += strf("    float keep%zu[%lld][4];\n", i, (long long)NP);
+    src += strf("    %s at[%lld];\n    bool live[%lld];\n", it, (long long)NP, (long long)NP);
+    src += strf("#pragma unroll\n    for (unsigned k = 0; k < %lldu; ++k) {\n", (long long)NP);
     // (a row or column quad beyond the edge works on the last valid one instead and is not stored: no branch)
-    src += strf("        const %s row_k = row0 + lr + 16u * k, quad_k = (col0 >> 2) + lc;\n", it);
+    src += strf("        const %s row_k = row0 + lr + %lldu * k, quad_k = (col0 >> 2) + lc;\n", it, (long long)RP);
     src += strf("        live[k] = row_k < %lld%s && quad_k < %lld%s;\n", (long long)Rws, sfx.c_str(), (long long)(I / 4), sfx.c_str());
     src += strf("        const %s %s = row_k < %lld%s ? row_k : %lld%s;\n        const %s %s = quad_k < %lld%s ? quad_k : %lld%s;\n", it, rowv.c_str(),
                 (long long)Rws, sfx.c_str(), (long long)(Rws - 1), sfx.c_str(), it, colv.c_str(), (long long)(I / 4), sfx.c_str(), (long long)(I / 4 - 1), sfx.c_str());
@@ -986,7 +1011,7 @@ static bool gen_elw_tiled_kernel(const ElwKernelSpec& spec, const std::set<const
     for (size_t i = 0; i < spec.outputs.size(); ++i)
         src += strf("#pragma unroll\n        for (int j = 0; j < 4; ++j) keep%zu[k][j] = w%zu[j];\n", i, i);
     src += "    }\n";
-    src += "#pragma unroll\n    for (unsigned k = 0; k < 4u; ++k) {\n        if (!live[k]) continue;\n";
+    src += strf("#pragma unroll\n    for (unsigned k = 0; k < %lldu; ++k) {\n        if (!live[k]) continue;\n", (long long)NP);
     for (size_t i = 0; i < spec.outputs.size(); ++i)
         src += "        " + store4_stmt(strf("keep%zu[k]", i), strf("o%zu + at[k] * 4u", i), N >= nontemporal_min_elems()) + "\n";
     src += "    }\n}\n";
@@ -1393,6 +1418,53 @@ GeneratedKernel gen_reduce_kernel(const ReduceKernelSpec& spec, int64_t force_ch
         Gen& g = b.g;
         const int64_t XV = V / vec;
         const int64_t bx = (XV + 63) / 64;
+        // Large inputs: blocks of 16 wavefronts that live for one or two rows each, as in the element-wise pass with
+        // column sums riding along (gen_elw_colsum_kernel) -- wavefront w adds up row 16 k + w of the block's rows over
+        // 256 columns (four per lane), the 16 wavefronts' sums are added through LDS in a fixed order, and one partial
+        // row per block goes to the second pass.  The chip then streams through the operand front to back; threads
+        // that walk down 32 rows each in a loop reached 0.62 of the HBM peak on 16384 x 4096 where this form reaches
+        // what the riding sums do.
+        const int64_t KW = elw_colsum_rows_per_wave(R, V, 1);
+        const int64_t tiles = (R + 16 * KW - 1) / (16 * KW);
+        if (force_chunks == 0 && vec == 4 && KW <= 4 && tiles >= 2 && bx * tiles >= 512) {
+            k.kind = "reduce_col";
+            std::string sig = "const int* __restrict__ guard, float* out";
+            std::vector<Node*> order{const_cast<Node*>(n)};
+            for (auto& gb : g.bufs) { sig += ", const float* " + gb.param; order.push_back(gb.node); }
+            const char* it = g.idx_t();
+            const char* sfx = wide ? "ull" : "u";
+            src += strf("extern \"C\" __global__ __launch_bounds__(1024) void %s(%s) {\n", k.entry.c_str(), sig.c_str());
+            src += "    if (guard && *guard == 0) return;\n";
+            src += "    __shared__ float4_t part[16][64];\n";
+            src += "    const unsigned lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;\n";
+            src += strf("    const %s xv_raw = (%s)blockIdx.x * 64u + lane;\n", it, it);
+            src += strf("    const bool col_ok = xv_raw < %lld%s;\n    const %s xv = col_ok ? xv_raw : %lld%s;\n", (long long)XV, sfx, it, (long long)(XV - 1), sfx);
+            src += strf("    float acc[4] = {%s, %s, %s, %s};\n", ident, ident, ident, ident);
+            // rows beyond the last one are clamped to it and left out of the sum: every load is unconditional, so a
+            // wavefront's loads are all in flight together
+            src += strf("#pragma unroll\n    for (unsigned kk = 0; kk < %lldu; ++kk) {\n", (long long)KW);
+            src += strf("        const %s y_raw = (%s)blockIdx.y * %lld%s + kk * 16u + wv;\n", it, it, (long long)(16 * KW), sfx);
+            src += strf("        const bool live = col_ok && y_raw < %lld%s;\n        const %s y = y_raw < %lld%s ? y_raw : %lld%s;\n", (long long)R, sfx, it,
+                        (long long)R, sfx, (long long)(R - 1), sfx);
+            src += join(g.codeA, "        ");
+            src += "#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+            src += join(g.codeB, "            ");
+            src += strf("            if (live) acc[j] = %s;\n        }\n    }\n", comb("acc[j]", b.value).c_str());
+            src += "    part[wv][lane] = float4_t{acc[0], acc[1], acc[2], acc[3]};\n    __syncthreads();\n";
+            src += "    if (wv == 0u && col_ok) {\n        float4_t s = part[0][lane];\n#pragma unroll\n        for (int r = 1; r < 16; ++r) {\n            const float4_t q = part[r][lane];\n";
+            src += "#pragma unroll\n            for (int j = 0; j < 4; ++j) s[j] = " + comb("s[j]", "q[j]") + ";\n        }\n";
+            src += strf("        *(float4_t*)(out + ((%s)blockIdx.y * %lld%s + xv * 4u)) = s;\n    }\n}\n", it, (long long)V, sfx);
+            k.buffer_args = order;
+            k.block[0] = 1024;
+            k.grid[0] = (unsigned)bx;
+            k.grid[1] = (unsigned)tiles;
+            k.chunks = tiles;
+            k.bytes = 4.0 * (double)V * (double)tiles;
+            for (auto& gb : g.bufs) k.bytes += 4.0 * (double)std::min<int64_t>(numel(gb.node->shape), V * R);
+            k.flops = (g.flops + 1) * (double)V * (double)R;
+            k.source = src;
+            return k;
+        }
         int64_t chunks = 1;
         if (force_chunks > 0) chunks = force_chunks;
         else {
