@@ -206,8 +206,10 @@ def measure_reductions_forward(dev, rows=16384, cols=4096):
     p = compile_resident(dev, wl)
     ms = timed_runs(p, 10, 2)
     ks = profile(p, 5)
+    # algorithmic bytes of a reduction launch: its operand read once (what it writes -- a vector, or the partial sums
+    # of a two-stage reduction -- is not priced; `bytes` in the kernel list is what the launch moves, partials included)
     out["configs2_forward"] = {"ms_per_step": ms, "kernels": ks,
-                               "roofline": [hbm_roofline(k, k["bytes"], note="x read once by this launch") for k in ks if k["bytes"] > 2.0 * n]}
+                               "roofline": [hbm_roofline(k, 4.0 * n, note="x read once by this launch") for k in ks if k["bytes"] > 2.0 * n]}
     p.close()
     rng = np.random.default_rng(0)
     data = [rng.standard_normal(n, dtype=np.float32) for _ in range(3)]
@@ -226,7 +228,7 @@ def measure_reductions_forward(dev, rows=16384, cols=4096):
         big = [k for k in ks if k["bytes"] > 2.0 * n]
         tensors = sum(round(k["bytes"] / (4.0 * n)) * k["launches_per_run"] for k in big)
         entry = {"ms_per_step": ms, "GBps_whole_step": wls.algorithmic_bytes / (ms * 1e-3) / 1e9, "kernels": ks, "tensors_per_step": tensors,
-                 "roofline": [hbm_roofline(k, k["bytes"], note=f"{round(k['bytes'] / (4.0 * n))} tensor(s) of {4 * n} bytes read once per launch; "
+                 "roofline": [hbm_roofline(k, round(k["bytes"] / (4.0 * n)) * 4.0 * n, note=f"{round(k['bytes'] / (4.0 * n))} tensor(s) of {4 * n} bytes read once per launch; "
                                            "three tensors in turn, so none is found in the last-level cache") for k in big]}
         out[name] = entry
         p.close()

@@ -20,7 +20,8 @@ SHAPES = [[4, 6], [6, 4], [6], [4], [1]]
 
 
 class _Gen:
-    def __init__(self, seed):
+    def __init__(self, seed, extended=False):
+        self.extended = extended   # also draw row maxima, a softmax spelled in commands and a maximum of integers
         self.rng = np.random.default_rng(seed)
         self.n = 0
         self.counters = 0
@@ -45,8 +46,26 @@ class _Gen:
     # ---- one straight-line command group appended to `out`
     def compute(self, out, depth):
         rng = self.rng
-        kind = int(rng.integers(10))
-        if kind == 0:      # real: a = 0.5 * (b + c)
+        kind = int(rng.integers(13 if self.extended else 10))
+        if kind == 10:     # real: the largest element of every row of a [4,6], written to a [4]
+            a = self.pick(self.reals, [4])
+            b = self.pick(self.reals, [4, 6])
+            out.append(IR.Max(a=b, res=a))
+        elif kind == 11:   # real: softmax over the rows of a [4,6] spelled in commands (in place when a == b)
+            a = self.pick(self.reals, [4, 6])
+            b = self.pick(self.reals, [4, 6])
+            m, mv, mb, n, d, e1, e, sm, r, rv, rb = (self.fresh("t") for _ in range(11))
+            out += [IR.Max(a=b, res=m), IR.View(a=m, target_dim=[4, 1], res=mv), IR.Broadcast(a=mv, dim=1, r=6, res=mb),
+                    IR.ElwMultiply(a=mb, b=self.const(out, -1.0, [4, 6]), res=n), IR.ElwAdd(a=b, b=n, res=d),
+                    IR.ElwMultiply(a=d, b=self.const(out, 1.4426950408889634, [4, 6]), res=e1), IR.Exp2(a=e1, res=e),
+                    IR.Sum(a=e, res=sm), IR.Recip(a=sm, res=r), IR.View(a=r, target_dim=[4, 1], res=rv),
+                    IR.Broadcast(a=rv, dim=1, r=6, res=rb), IR.ElwMultiply(a=e, b=rb, res=a)]
+        elif kind == 12:   # int: scalar k[1] = the largest element of a [4] (exact)
+            a = self.pick(self.ints, [1])
+            b = self.pick(self.ints, [4])
+            v = self.fresh("t")
+            out += [IR.View(a=b, target_dim=[1, 4], res=v), IR.Max(a=v, res=a)]
+        elif kind == 0:    # real: a = 0.5 * (b + c)
             a = self.pick(self.reals)
             sh = self.reals[a]
             b, c = self.pick(self.reals, sh), self.pick(self.reals, sh)
@@ -182,9 +201,10 @@ class _Gen:
         out.append(IR.If(conditions=arms, else_proc=else_proc))
 
 
-def random_control_program(seed: int):
-    """Returns (procedure, keep list, names of the integer-valued ids)."""
-    g = _Gen(seed)
+def random_control_program(seed: int, extended: bool = False):
+    """Returns (procedure, keep list, names of the integer-valued ids).  `extended` adds row maxima, a softmax spelled in
+    commands and integer maxima to the operations drawn (the plain form keeps the programs of its seeds as they were)."""
+    g = _Gen(seed, extended)
     rng = g.rng
     for sh in SHAPES:
         for _ in range(2):

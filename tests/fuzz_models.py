@@ -148,6 +148,10 @@ def _build(dev, seed, scale, n_ops, shadow, kinds=None):
             if K is not None and V is not None:
                 s2 = K.dim()[0]
                 keep_p = int(rng.integers(3)) == 0
+                if int(rng.integers(2)):
+                    # inference: no gradient flows back through the attention, so nothing but the product reads the
+                    # probabilities and the fused kernel applies (head widths permitting)
+                    a, K, V = (apply(lambda u: u.detach(), lambda u: u.detach(), x) for x in (a, K, V))
                 if kind == 9:
                     mask = leaf([s1, s2], 0.25, 1.25, grad=False)
 

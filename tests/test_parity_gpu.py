@@ -464,14 +464,16 @@ def test_repeated_execute_rebinds_payloads(hip_device):
         assert_close(out["s"].data, v.reshape(2, width).astype(np.float64).sum(1), RED_RTOL * math.sqrt(width), f"width {width}")
 
 
-@pytest.mark.parametrize("seed", list(range(40)) + [257, 266, 290, 311])   # the last four: an arm reads an id an earlier arm dropped
-def test_random_control_flow_matches_oracle(seed, hip_device):
+@pytest.mark.parametrize("seed,extended", [(s, False) for s in list(range(40)) + [257, 266, 290, 311]] +   # the last four: an arm reads an id an earlier arm dropped
+                         [(s, True) for s in range(40)])
+def test_random_control_flow_matches_oracle(seed, extended, hip_device):
     """Random programs with nested counted loops, data-dependent loops and branches (tests/fuzz_control.py):
     integer-valued tensors (which drive every predicate) bit-exact, the others within the element-wise / reduction
-    tolerance."""
-    print(f"[case] control fuzz seed {seed}", flush=True)
+    tolerance.  The extended form also draws row maxima, a softmax spelled in commands (inside loops and branches, in
+    place too) and maxima of integer-valued tensors."""
+    print(f"[case] control fuzz seed {seed}{' extended' if extended else ''}", flush=True)
     from fuzz_control import random_control_program
-    proc, keep, ints = random_control_program(seed)
+    proc, keep, ints = random_control_program(seed, extended)
     ref_dev = OracleDevice()
     ref_dev.execute(proc, set(keep))
     ref = {k: ref_dev.get_tensor(k) for k in keep}
