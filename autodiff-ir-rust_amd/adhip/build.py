@@ -38,5 +38,19 @@ def build_cxx_smoke(verbose: bool = False) -> str:
     return out
 
 
+def build_overlap_probe(verbose: bool = False) -> str:
+    """Compile tests/cxx/mfma_valu_overlap.cpp (a hardware premise of the matrix kernels, measured) for gfx950."""
+    root = os.path.dirname(os.path.dirname(_PKG_DIR))
+    src = os.path.join(root, "tests", "cxx", "mfma_valu_overlap.cpp")
+    out = os.path.join(root, "tests", "cxx", "mfma_valu_overlap")
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-o", out, src]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))

@@ -3308,10 +3308,22 @@ struct Lowerer {
         pl.bn_tile = cfg.bm == 64 ? 64 : 128;
         // one 128x128 block per CU is too few to hide its own latencies: halve the tile's width for two per CU
         if (cfg.bm == 128 && blocks128 < 512 && splits_for(blocks128) == 1) { pl.bn_tile = 64; cfg.bn = 64; }
+        // diagnostic: ADHIP_DOT_PLAN=<bm>,<bn>,<splits> forces tile and k ranges of every aligned product the tile divides
+        int64_t forced_splits = 0;
+        if (const char* e = getenv("ADHIP_DOT_PLAN")) {
+            long fbm = 0, fbn = 0, fs = 0;
+            if (sscanf(e, "%ld,%ld,%ld", &fbm, &fbn, &fs) == 3 && !unaligned && (fbm == 256 || fbm == 128 || fbm == 64) &&
+                (fbn == 128 || fbn == 64) && M % fbm == 0 && N % fbn == 0 && fs >= 1 && !(fbm == 256 && fbn != 128) && !(fbm == 64 && fbn != 64)) {
+                cfg.bm = (int)fbm;
+                pl.bn_tile = (int)fbn;
+                cfg.bn = (fbm == 128 && fbn == 64) ? 64 : 0;
+                forced_splits = fs;
+            }
+        }
         cfg.edge = unaligned || (M % cfg.bm) || (N % pl.bn_tile);
         cfg.edge_vec = alignment != 2;
         const int64_t blocks = ((M + cfg.bm - 1) / cfg.bm) * ((N + pl.bn_tile - 1) / pl.bn_tile);
-        const int64_t want = cfg.bm == 256 ? 1 : splits_for(blocks);
+        const int64_t want = forced_splits ? std::min<int64_t>(forced_splits, std::max<int64_t>(K / 64, 1)) : (cfg.bm == 256 ? 1 : splits_for(blocks));
         if (want > 1) {
             pl.k_chunk = (((K + want - 1) / want) + 15) / 16 * 16;
             pl.splits = (K + pl.k_chunk - 1) / pl.k_chunk;

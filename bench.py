@@ -235,6 +235,33 @@ def measure_reductions_forward(dev, rows=16384, cols=4096):
     return out
 
 
+def measure_last_layer_products(dev):
+    """The three products of configs[3]'s last layer (4096 -> 1024, batch 4096) on their own, without epilogues:
+    y = x W (A rows contiguous), dW = x^T dy (A columns contiguous), dx = dy W^T (both along k).  With
+    ADHIP_DOT_PLAN=<bm>,<bn>,<splits> in the environment the library launches them with that tile and that many ranges
+    of k instead of its own choice, which is how the alternatives in DESIGN.md were timed."""
+    import numpy as np
+    from adhip import ir as IR
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(4096 * 4096).astype(np.float32)
+    w = rng.standard_normal(4096 * 1024).astype(np.float32)
+    dy = rng.standard_normal(4096 * 1024).astype(np.float32)
+    cmds = [IR.CreateMat(x, [4096, 4096], "x"), IR.CreateMat(w, [4096, 1024], "w"), IR.CreateMat(dy, [4096, 1024], "dy"),
+            IR.DotProduct(a="x", b="w", res="y"),
+            IR.Permute(a="x", p=[1, 0], res="xt"), IR.DotProduct(a="xt", b="dy", res="dw"),
+            IR.Permute(a="w", p=[1, 0], res="wt"), IR.DotProduct(a="dy", b="wt", res="dx"), IR.EX()]
+    prog = dev.compile(IR.IRProcedure("main", cmds), {"y", "dw", "dx"})
+    prog.upload()
+    ms = timed_runs(prog, 10, 2)
+    ks = profile(prog, 5)
+    prog.close()
+    for k in ks:
+        if k["flops"] > 1e9:
+            k["TFLOPs"] = k["flops"] / (k["avg_ms"] * 1e-3) / 1e12
+            k["frac_of_fp32_mfma_peak"] = k["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS
+    return {"plan": os.environ.get("ADHIP_DOT_PLAN", "library's choice"), "ms_per_step": ms, "kernels": ks}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -243,13 +270,14 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "reductions_forward", "manip", "attention"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "reductions_forward", "manip", "attention", "last_layer_products"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by; "
                          "'streammix': only a bare 3-reads + 4-writes kernel over 8192x8192 f32 (the stream mix of the "
                          "headline pass with trivial arithmetic and no column sums: what the memory system gives that mix); "
                          "'reductions': only configs[2]; 'reductions_forward': only the stand-alone row and column reduction "
-                         "kernels on 256 MiB tensors; 'mlp': only configs[3]; 'manip': only configs[4] (one run: its "
+                         "kernels on 256 MiB tensors; 'last_layer_products': the three 4096x1024x4096-shaped products of "
+                         "configs[3]'s last layer on their own (honours ADHIP_DOT_PLAN); 'mlp': only configs[3]; 'manip': only configs[4] (one run: its "
                          "loop consumes its counter); 'attention': only multi-head attention forward")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -301,6 +329,9 @@ def main():
         ms3 = timed_runs(p3, args.steps, args.warmup)
         print(json.dumps({"metric": "reductions forward + backward, f32 [16384,4096]", "value": wl3.algorithmic_bytes / (ms3 * 1e-3) / 1e9,
                           "unit": "GB/s", "ms_per_step": ms3, "algorithmic_bytes": wl3.algorithmic_bytes, "kernels": profile(p3, 3)}))
+        return
+    if args.workload == "last_layer_products":
+        print(json.dumps(dict(measure_last_layer_products(dev), metric="products of the 4096 -> 1024 layer, fp32")))
         return
     if args.workload == "reductions_forward":
         print(json.dumps(dict(measure_reductions_forward(dev), metric="stand-alone reductions, f32 [16384,4096]")))
