@@ -178,3 +178,50 @@ def test_chained_equals_unchained(kind, hip_device, monkeypatch):
     for k in plain:
         s = float(np.abs(plain[k]).max())
         assert float(np.abs(chained[k] - plain[k]).max()) <= 4 * RED_RTOL * math.sqrt(cols) * s, k
+
+
+def _in_place_normalise_program(rows, cols, iters, seed=5):
+    """x [rows, cols] is replaced by its row softmax `iters` times inside a counted loop, spelled in commands: the chain
+    reads the old x and writes the new one into the same buffer."""
+    from adhip import ir as IR
+    rng = np.random.default_rng(seed)
+    xn = rng.standard_normal((rows, cols)).astype(np.float32)
+    c = lambda v, id, sh: IR.CreateConstant(float(v), id, list(sh))  # noqa: E731
+    body = [
+        IR.Max(a="x", res="m"), IR.View(a="m", target_dim=[rows, 1], res="mv"), IR.Broadcast(a="mv", dim=1, r=cols, res="mb"),
+        c(-1.0, "neg", [rows, cols]), IR.ElwMultiply(a="mb", b="neg", res="n"), IR.ElwAdd(a="x", b="n", res="d"),
+        c(1.4426950408889634, "l2e", [rows, cols]), IR.ElwMultiply(a="d", b="l2e", res="e1"), IR.Exp2(a="e1", res="e"),
+        IR.Sum(a="e", res="s"), IR.Recip(a="s", res="r"), IR.View(a="r", target_dim=[rows, 1], res="rv"),
+        IR.Broadcast(a="rv", dim=1, r=cols, res="rb"), IR.ElwMultiply(a="e", b="rb", res="x"),
+        c(1.0, "one", [1]), IR.ElwAddEq(s="i", o="one"), c(-float(iters), "lim", [1]), IR.ElwAdd(a="i", b="lim", res="t"),
+        IR.LessZero(a="t", res="go"),
+    ]
+    cmds = [IR.CreateMat(xn.reshape(-1), [rows, cols], "x"), IR.CreateMat(np.zeros(1, np.float32), [1], "i"),
+            c(-float(iters), "lim0", [1]), IR.ElwAdd(a="i", b="lim0", res="t0"), IR.LessZero(a="t0", res="go"),
+            IR.While(conditional_var="go", block=IR.IRProcedure("body", body)), IR.EX()]
+    want = xn.astype(np.float64)
+    for _ in range(iters):
+        e = np.exp(want - want.max(1, keepdims=True))
+        want = e / e.sum(1, keepdims=True)
+    return IR.IRProcedure("main", cmds), {"x", "i"}, want
+
+
+def test_in_place_chain_needs_no_copy():
+    """The softmax that overwrites its own operand inside a loop is one row-chain launch per iteration, with no copy
+    behind it: a chain reads all it needs of a row before it stores any of it."""
+    proc, keep, _ = _in_place_normalise_program(512, 256, 3)
+    text = lower_describe(proc, keep)
+    body = text[text.index("while "):]
+    assert body.count("[rowchain]") == 1 and "[copy]" not in body, body
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols", [(512, 256), (100, 2052), (37, 8192)])
+def test_in_place_chain_in_a_loop_matches_float64(rows, cols, hip_device):
+    print(f"[case] in-place row chain in a loop {rows}x{cols}", flush=True)
+    proc, keep, want = _in_place_normalise_program(rows, cols, 3)
+    hip_device.execute(proc, keep)
+    assert hip_device.get_tensor("i").data[0] == 3.0
+    got = hip_device.get_tensor("x").numpy().astype(np.float64)
+    assert np.abs(got - want).max() <= RED_RTOL * math.sqrt(cols) * np.abs(want).max()
+    np.testing.assert_allclose(got.sum(1), 1.0, rtol=1e-5)
