@@ -343,7 +343,7 @@ struct Lowerer {
     int region_counter = 0, cur_region = -1;
     int region_shift() const {
         auto it = opt.region_shift.find(cur_region);
-        return it == opt.region_shift.end() ? 0 : std::min(it->second, 8);
+        return std::min(std::max(it == opt.region_shift.end() ? 0 : it->second, opt.min_shift), 8);
     }
     int64_t bound(int v) const { return std::max<int64_t>(2, (int64_t)v >> region_shift()); }
     bool tight() const { return region_shift() > 0; }
@@ -3778,6 +3778,17 @@ std::string Plan::describe() const {
     return o;
 }
 
+std::string lowering_switches() {
+    std::string out;
+    for (const char* name : {"ADHIP_GROUP_DOTS", "ADHIP_LAYER_KERNELS", "ADHIP_MERGE_SMALL", "ADHIP_FUSE_ATTENTION", "ADHIP_ROW_CHAINS",
+                             "ADHIP_TIGHTEN", "ADHIP_KERNEL_BOUNDS", "ADHIP_DOT_PLAN", "ADHIP_TILED_SHAPE", "ADHIP_GRAPHS"}) {
+        const char* e = getenv(name);
+        out += e ? e : "";
+        out.push_back(';');
+    }
+    return out;
+}
+
 std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids, const LowerOptions& opt_in) {
     LowerOptions opt = opt_in;
     if (const char* e = getenv("ADHIP_GROUP_DOTS")) opt.group_dots = opt.group_dots && atoi(e) != 0;
@@ -3785,6 +3796,8 @@ std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::str
     if (const char* e = getenv("ADHIP_MERGE_SMALL")) opt.merge_small = opt.merge_small && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_FUSE_ATTENTION")) opt.fuse_attention = opt.fuse_attention && atoi(e) != 0;
     if (const char* e = getenv("ADHIP_ROW_CHAINS")) opt.row_chains = opt.row_chains && atoi(e) != 0;
+    // diagnostic: every region lowered the way a region is after that many kernels of it spilled vector registers
+    if (const char* e = getenv("ADHIP_TIGHTEN")) opt.min_shift = std::max(0, std::min(atoi(e), 4));
     // diagnostic: the seven kernel-size bounds, in the order LowerOptions declares them ("24,48,32,96,40,24,20")
     if (const char* e = getenv("ADHIP_KERNEL_BOUNDS")) {
         int* field[7] = {&opt.max_pieces, &opt.max_inline_sites, &opt.max_inline_loads, &opt.max_kernel_sites, &opt.max_kernel_pointers,

@@ -34,10 +34,15 @@ struct LowerOptions {
     // there.  A region at shift >= 1 also takes no fused epilogues and no sums riding along.  The runtime raises the
     // shift of a region whose kernel the compiler could only build by spilling vector registers, and lowers again.
     std::map<int, int> region_shift;
+    int min_shift = 0;              // diagnostic (ADHIP_TIGHTEN): every region is lowered at this shift at least
 };
 
 std::unique_ptr<Plan> lower_program(const Proc& prog, const std::vector<std::string>& dep_ids,
                                     const LowerOptions& opt = LowerOptions());
+
+// The current values of the environment switches that change what lower_program makes of a program, as one string:
+// part of the key under which a context remembers a lowered program.
+std::string lowering_switches();
 
 // Fixed (not generated) kernels
 const char* fixed_kernels_source();

@@ -999,6 +999,8 @@ int adhip_execute(adhip_ctx* ctx, const uint8_t* program, size_t program_len, co
                 memset(&key[o], 0, 8);
             }
             for (const std::string& d : dep_vector(dep_ids, n_dep_ids)) { key.push_back('\0'); key += d; }
+            key.push_back('\0');
+            key += lowering_switches();  // a plan made under other switches is another program
             for (size_t i = 0; i < ctx->exec_cache.size(); ++i) {
                 if (ctx->exec_cache[i].key != key) continue;
                 adhip_program* q = ctx->exec_cache[i].prog;

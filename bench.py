@@ -262,6 +262,31 @@ def measure_last_layer_products(dev):
     return {"plan": os.environ.get("ADHIP_DOT_PLAN", "library's choice"), "ms_per_step": ms, "kernels": ks}
 
 
+def measure_encoder(dev, kernels=False):
+    """One transformer encoder layer, forward + backward, [2048, 1024] activations, 8 heads, feed-forward width 4096;
+    `kernels`: also the per-launch-site list (each with its rate by the bytes or flops the lowering prices it at)."""
+    from adhip import workloads as W
+    wl6 = W.encoder_layer(dev, 2048, 1024, 8, 4096, seed=0)
+    p6 = compile_resident(dev, wl6)
+    ms6 = timed_runs(p6, 5, 2)
+    k6 = profile(p6, 2)
+    dot6 = sum(k["avg_ms"] * k["launches_per_run"] for k in k6 if k["kernel"].startswith("dot"))
+    all6 = sum(k["avg_ms"] * k["launches_per_run"] for k in k6)
+    out = {"ms_per_step": ms6, "matmul_flops_per_step": wl6.flops,
+           "matmul_TFLOPs_whole_step": wl6.flops / (ms6 * 1e-3) / 1e12,
+           "matmul_kernels_ms": dot6, "other_kernels_ms": all6 - dot6,
+           "launches_per_step": sum(k["launches_per_run"] for k in k6)}
+    if kernels:
+        for k in k6:
+            if k["kernel"].startswith("dot") and k.get("flops"):
+                k["TFLOPs"] = k["flops"] / (k["avg_ms"] * 1e-3) / 1e12
+            elif k["bytes"]:
+                k["GBps"] = k["bytes"] / (k["avg_ms"] * 1e-3) / 1e9
+        out["kernels"] = sorted(k6, key=lambda k: -k["avg_ms"] * k["launches_per_run"])
+    p6.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -270,7 +295,7 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="measure only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mlp-iters", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "reductions_forward", "manip", "attention", "last_layer_products"],
+    ap.add_argument("--workload", default="all", choices=["all", "copy", "streammix", "mlp", "reductions", "reductions_forward", "manip", "attention", "last_layer_products", "encoder"],
                     help="'copy': only a plain 8192x8192 f32 copy kernel (256 MiB read + 256 MiB written per launch), "
                          "the known-size reference that hardware byte counters are scaled by; "
                          "'streammix': only a bare 3-reads + 4-writes kernel over 8192x8192 f32 (the stream mix of the "
@@ -278,7 +303,8 @@ def main():
                          "'reductions': only configs[2]; 'reductions_forward': only the stand-alone row and column reduction "
                          "kernels on 256 MiB tensors; 'last_layer_products': the three 4096x1024x4096-shaped products of "
                          "configs[3]'s last layer on their own (honours ADHIP_DOT_PLAN); 'mlp': only configs[3]; 'manip': only configs[4] (one run: its "
-                         "loop consumes its counter); 'attention': only multi-head attention forward")
+                         "loop consumes its counter); 'attention': only multi-head attention forward; 'encoder': only the encoder "
+                         "layer, with its per-kernel list")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the device path is single-device (run with --gpus 1)", file=sys.stderr)
@@ -349,6 +375,9 @@ def main():
         return
     if args.workload == "attention":
         print(json.dumps(dict(measure_attention(dev), metric="multi-head attention forward, fp32")))
+        return
+    if args.workload == "encoder":
+        print(json.dumps(dict(measure_encoder(dev, kernels=True), metric="transformer encoder layer forward + backward, fp32")))
         return
     if args.workload == "mlp":
         print(json.dumps(dict(measure_mlp(dev, args.mlp_iters), metric="fp32 MLP train steps/s")))
@@ -450,15 +479,7 @@ def main():
         extra["mlp_train"] = measure_mlp(dev, args.mlp_iters)
         # beyond BASELINE.json's configs: one transformer encoder layer (the caller side's attention modules),
         # forward + backward, [2048, 1024] activations, 8 heads, feed-forward width 4096
-        wl6 = W.encoder_layer(dev, 2048, 1024, 8, 4096, seed=0)
-        p6 = compile_resident(dev, wl6)
-        ms6 = timed_runs(p6, 5, 2)
-        k6 = profile(p6, 2)
-        dot6 = sum(k["avg_ms"] * k["launches_per_run"] for k in k6 if k["kernel"].startswith("dot"))
-        extra["encoder_layer"] = {"ms_per_step": ms6, "matmul_flops_per_step": wl6.flops,
-                                  "matmul_TFLOPs_whole_step": wl6.flops / (ms6 * 1e-3) / 1e12,
-                                  "matmul_kernels_ms": dot6, "launches_per_step": sum(k["launches_per_run"] for k in k6)}
-        p6.close()
+        extra["encoder_layer"] = measure_encoder(dev)
         extra["attention_forward"] = measure_attention(dev)
 
     cpu = None

@@ -669,3 +669,25 @@ def test_full_size_workloads_lower(name):
         assert "[elw_tiled]" in text and "[transpose]" not in text
     if name == "mlp_train":
         assert "adhip_gemm_kn_256" in text and "adhip_gemm_kk_256" in text and "adhip_gemm_mn_256" in text
+
+
+@pytest.mark.parametrize("shift", [1, 2, 4])
+def test_tightened_lowering_compiles(shift, monkeypatch):
+    """ADHIP_TIGHTEN lowers every region the way a region is lowered after kernels of it spilled vector registers (the
+    bounds halved `shift` times, no epilogues, no riding sums): more and smaller kernels, all of which compile for
+    gfx950 without spills."""
+    from fuzz_models import random_model_program
+    monkeypatch.setenv("ADHIP_CACHE_DIR", "off")
+    dev = Capture()
+    try:
+        random_model_program(dev, 3, 16)
+    except AttributeError:
+        pass
+    plain = lower_describe(dev.proc, dev.deps).count("\nlaunch ") + lower_describe(dev.proc, dev.deps).count("  launch ")
+    monkeypatch.setenv("ADHIP_TIGHTEN", str(shift))
+    text = lower_describe(dev.proc, dev.deps)
+    tight = text.count("\nlaunch ") + text.count("  launch ")
+    assert tight > plain, (plain, tight)
+    rc, msg = _compile_check(dev.proc, dev.deps)
+    assert rc == 0, msg
+    assert not _vector_spills(msg), msg

@@ -13,6 +13,19 @@ from programs import KATS, ROUNDED, check_golden
 
 pytestmark = pytest.mark.gpu
 
+
+def _sweep(generator):
+    """More seeds for a generator's test, for sweeps on a GPU box.  ADHIP_FUZZ_SWEEP holds comma-separated
+    `generator:scale:first:last` entries (generator = models | programs | control; for control, scale 1 draws the
+    extended command set and 0 the plain one); each adds (scale, seed) for first <= seed < last.  Example:
+    ADHIP_FUZZ_SWEEP=models:16:0:200 python -m pytest tests/test_parity_gpu.py -m gpu -x -k random_model_programs"""
+    out = []
+    for entry in filter(None, os.environ.get("ADHIP_FUZZ_SWEEP", "").split(",")):
+        name, scale, first, last = entry.split(":")
+        if name == generator:
+            out += [(int(scale), s) for s in range(int(first), int(last))]
+    return out
+
 EXACT_KATS = {"grd", "eq", "if_ctrl", "if_else_ctrl", "for_ctrl", "evrty_ctrl", "everything"}
 
 
@@ -228,7 +241,8 @@ def test_random_programs_match_oracle(seed, hip_device):
         assert_close(got[k].data, rv.data, tol, f"seed {seed} {k}")
 
 
-@pytest.mark.parametrize("scale,seed", [(16, s) for s in range(12)] + [(16, 23), (16, 122), (16, 343)] + [(48, s) for s in range(6)] + [(48, 31), (48, 81)])
+@pytest.mark.parametrize("scale,seed", [(16, s) for s in range(12)] + [(16, 23), (16, 122), (16, 343)] + [(48, s) for s in range(6)] + [(48, 31), (48, 81)] +
+                         _sweep("programs"))
 def test_random_programs_at_scale(scale, seed, hip_device):
     """The same generator with every leaf extent multiplied (tests/fuzz_programs.py, `scale`): tensors of 10^4 to 10^6
     elements, so the kernels are the 128-bit element-wise forms, sums riding along, chunked reductions and matrix-core
@@ -278,7 +292,7 @@ def test_adversarial_programs_match_numpy(name, hip_device):
 
 
 MODEL_FUZZ = ([(1, s) for s in range(40)] + [(4, s) for s in range(16)] + [(16, s) for s in range(10)] +
-              [(48, s) for s in range(4)])
+              [(48, s) for s in range(4)]) + _sweep("models")
 
 
 @pytest.mark.parametrize("scale,seed", MODEL_FUZZ)
@@ -468,7 +482,7 @@ def test_repeated_execute_rebinds_payloads(hip_device):
 
 
 @pytest.mark.parametrize("seed,extended", [(s, False) for s in list(range(40)) + [257, 266, 290, 311]] +   # the last four: an arm reads an id an earlier arm dropped
-                         [(s, True) for s in range(40)])
+                         [(s, True) for s in range(40)] + [(s, bool(e)) for e, s in _sweep("control")])
 def test_random_control_flow_matches_oracle(seed, extended, hip_device):
     """Random programs with nested counted loops, data-dependent loops and branches (tests/fuzz_control.py):
     integer-valued tensors (which drive every predicate) bit-exact, the others within the element-wise / reduction
@@ -1045,3 +1059,52 @@ def test_small_programs_one_launch_per_kernel_and_merged_agree(seed, hip_device,
         for k, rv in want.items():
             assert out[k].dim == rv.dim, k
             assert_close(out[k].data, rv.data, 2e-4, k)
+
+
+TIGHT_CASES = ([("models", 1, s) for s in range(8)] + [("models", 16, s) for s in range(4)] + [("models", 48, 0)] +
+               [("programs", 16, s) for s in range(3)] + [("programs", 48, 1)] + [("control", 1, s) for s in range(6)])
+
+
+@pytest.mark.parametrize("shift", [1, 3])
+@pytest.mark.parametrize("generator,scale,seed", TIGHT_CASES)
+def test_tightened_lowering_matches_oracle(generator, scale, seed, shift, hip_device, monkeypatch):
+    """What a program is lowered to after kernels of it spilled vector registers -- every kernel-size bound halved
+    `shift` times, no epilogues, no sums riding along -- is a path no known program takes on its own, so it is forced
+    here (ADHIP_TIGHTEN) and held against the oracle like the ordinary lowering."""
+    print(f"[case] tightened x{shift}: {generator} scale {scale} seed {seed}", flush=True)
+    monkeypatch.setenv("ADHIP_TIGHTEN", str(shift))
+    if generator == "control":
+        from fuzz_control import random_control_program
+        proc, keep, ints = random_control_program(seed, True)
+        oracle = OracleDevice()
+        oracle.execute(proc, set(keep))
+        hip_device.execute(proc, set(keep))
+        for k in keep:
+            got, ref = hip_device.get_tensor(k), oracle.get_tensor(k)
+            if k in ints or k.startswith("i"):
+                assert_exact(got.data, ref.data, k)
+            else:
+                assert_close(got.data, ref.data, 2e-5, k, scale=max(1.0, float(np.max(np.abs(ref.data)))))
+        return
+    if generator == "models":
+        from fuzz_models import random_model_program
+        got = random_model_program(hip_device, seed, scale)
+        oracle = OracleDevice()
+        ref = random_model_program(oracle, seed, scale)
+    else:
+        from fuzz_programs import random_program
+        got = random_program(hip_device, seed, scale=scale)
+        oracle = OracleDevice()
+        ref = random_program(oracle, seed, scale=scale)
+    tol = RED_RTOL * math.sqrt(oracle.max_terms) * 2
+    finite = [np.asarray(v.data)[np.isfinite(v.data)] for v in ref.values()]
+    largest = max((float(np.max(np.abs(f))) for f in finite if f.size), default=1.0)
+    for k, rv in ref.items():
+        r = np.asarray(rv.data, np.float64)
+        g = np.asarray(got[k].data, np.float64)
+        m = np.isfinite(r)
+        assert (np.isfinite(g) == m).all(), k
+        own = float(np.max(np.abs(r[m]))) if m.any() else 0.0
+        floor = max(own, 1e-2 * largest)
+        assert (np.abs(g - r)[m] <= tol * np.maximum(np.abs(r[m]), floor)).all(), \
+            f"{generator} scale {scale} seed {seed} {k}: {float(np.abs(g - r)[m].max()):.3e} > {tol * floor:.3e}"
