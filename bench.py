@@ -26,13 +26,17 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix, published
 # copy kernel of known size (the summaries under profiles/ give the runs).  These counters sit in front of the 256 MiB
 # last-level cache, so they bound HBM traffic from above.  Valid for the full-size workloads only.
 TRAFFIC_BYTES = {
-    # 2 x 393276.6 KiB fetched + 1081844.6 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
-    "fused_elw": {"elw_colsum": int((2 * 393276.6 + 1081844.6) * 1024)},
-    # the one pass of configs[2] (dx with row and column sums riding along): 2 x 131353.0 KiB fetched + 278574.5 KiB
+    # 2 x 393277.1 KiB fetched + 1081785.4 KiB written (the 4 outputs and two [512][8192] partial column-sum buffers)
+    "fused_elw": {"elw_colsum": int((2 * 393277.1 + 1081785.4) * 1024)},
+    # the one pass of configs[2] (dx with row and column sums riding along): 2 x 131353.0 KiB fetched + 278577.4 KiB
     # written (dx, the [512][4096] partial column sums, one run sum per row and 256 columns)
-    "reductions": {"elw_colsum": int((2 * 131353.0 + 278574.5) * 1024)},
-    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73766.4 KiB fetched + 294912.0 KiB written
-    "manip_loop": {"gather_stage": int((2 * 73766.4 + 294912.0) * 1024)},
+    "reductions": {"elw_colsum": int((2 * 131353.0 + 278577.4) * 1024)},
+    # the stand-alone reductions (profiles/reductions_forward_and_row_chains.hbm_traffic_pmc.txt), by kernel kind and
+    # tensors per launch: fetched x 2 + written (the column reduction writes a row of partial sums per 32 rows)
+    "reductions_forward": {("reduce_row", 1): int((2 * 131085.5 + 512.0) * 1024), ("reduce_col", 1): int((2 * 131087.0 + 8192.0) * 1024),
+                           ("reduce_row", 3): int((2 * 393230.0 + 1536.4) * 1024), ("reduce_col", 3): int((2 * 393232.0 + 24576.0) * 1024)},
+    # gather stage of configs[4] (one tiled element-wise launch): 2 x 73777.4 KiB fetched + 294912.0 KiB written
+    "manip_loop": {"gather_stage": int((2 * 73777.4 + 294912.0) * 1024)},
 }
 
 
@@ -202,6 +206,10 @@ def measure_reductions_forward(dev, rows=16384, cols=4096):
     from adhip import workloads as W
     n = rows * cols
     out = {"config": {"rows": rows, "cols": cols, "bytes_per_tensor": 4 * n}}
+
+    def counted_traffic(k, tensors):
+        # counter figures exist for the default size only
+        return TRAFFIC_BYTES["reductions_forward"].get((k["kernel"].split(":")[0], tensors)) if (rows, cols) == (16384, 4096) else None
     wl = W.reductions(dev, rows, cols, seed=0, backward=False)
     p = compile_resident(dev, wl)
     ms = timed_runs(p, 10, 2)
@@ -209,7 +217,7 @@ def measure_reductions_forward(dev, rows=16384, cols=4096):
     # algorithmic bytes of a reduction launch: its operand read once (what it writes -- a vector, or the partial sums
     # of a two-stage reduction -- is not priced; `bytes` in the kernel list is what the launch moves, partials included)
     out["configs2_forward"] = {"ms_per_step": ms, "kernels": ks,
-                               "roofline": [hbm_roofline(k, 4.0 * n, note="x read once by this launch") for k in ks if k["bytes"] > 2.0 * n]}
+                               "roofline": [hbm_roofline(k, 4.0 * n, counted_traffic(k, 1), note="x read once by this launch") for k in ks if k["bytes"] > 2.0 * n]}
     p.close()
     rng = np.random.default_rng(0)
     data = [rng.standard_normal(n, dtype=np.float32) for _ in range(3)]
@@ -228,7 +236,7 @@ def measure_reductions_forward(dev, rows=16384, cols=4096):
         big = [k for k in ks if k["bytes"] > 2.0 * n]
         tensors = sum(round(k["bytes"] / (4.0 * n)) * k["launches_per_run"] for k in big)
         entry = {"ms_per_step": ms, "GBps_whole_step": wls.algorithmic_bytes / (ms * 1e-3) / 1e9, "kernels": ks, "tensors_per_step": tensors,
-                 "roofline": [hbm_roofline(k, round(k["bytes"] / (4.0 * n)) * 4.0 * n, note=f"{round(k['bytes'] / (4.0 * n))} tensor(s) of {4 * n} bytes read once per launch; "
+                 "roofline": [hbm_roofline(k, round(k["bytes"] / (4.0 * n)) * 4.0 * n, counted_traffic(k, round(k["bytes"] / (4.0 * n))), note=f"{round(k['bytes'] / (4.0 * n))} tensor(s) of {4 * n} bytes read once per launch; "
                                            "three tensors in turn, so none is found in the last-level cache") for k in big]}
         out[name] = entry
         p.close()
