@@ -3781,7 +3781,7 @@ std::string Plan::describe() const {
 std::string lowering_switches() {
     std::string out;
     for (const char* name : {"ADHIP_GROUP_DOTS", "ADHIP_LAYER_KERNELS", "ADHIP_MERGE_SMALL", "ADHIP_FUSE_ATTENTION", "ADHIP_ROW_CHAINS",
-                             "ADHIP_TIGHTEN", "ADHIP_KERNEL_BOUNDS", "ADHIP_DOT_PLAN", "ADHIP_TILED_SHAPE", "ADHIP_GRAPHS"}) {
+                             "ADHIP_TIGHTEN", "ADHIP_KERNEL_BOUNDS", "ADHIP_DOT_PLAN", "ADHIP_TILED_SHAPE", "ADHIP_GEMM_AHEAD", "ADHIP_GRAPHS"}) {
         const char* e = getenv(name);
         out += e ? e : "";
         out.push_back(';');
