@@ -294,7 +294,7 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
         }
     };
 
-    const long long KT = (k_hi - k_lo + BK - 1) / BK;
+    const int KT = __builtin_amdgcn_readfirstlane((int)((k_hi - k_lo + BK - 1) / BK));   // (uniform: kept in a scalar register)
 #if AHEAD == 2
     // Global loads run two k-tiles ahead of the MFMAs, in two register sets that take turns: during tile kt the loads
     // of tile kt + 2 are issued into the set that held tile kt (parked in LDS during tile kt - 1), and the set that
@@ -303,28 +303,51 @@ extern "C" __global__ __launch_bounds__(NT) void KERNEL_NAME(
     // memory): 4096 x 1024 x 4096 in 276 / 268 / 251 us instead of 289 / 274 / 257, the MLP workload's step 1.2 % and
     // the encoder layer's 1.3 % shorter.  The loop is unrolled by two so that the sets and the LDS buffers are named,
     // not indexed.
+    // Loads and parkings stand under no condition: beyond the last tile the loads fetch the last tile again and the
+    // parking writes a tile nobody reads.  (Under a condition, the wait in front of a parking also waits for the
+    // newest loads, or the compiler moves the loads down to the parking that consumes them.)
+    int t_at = 0;   // the tile the next loads fetch
+#if EDGE
+    auto load_next = [&](float4_t* ra, float4_t* rb) {
+        load_a(k_lo + (long long)t_at * BK, ra);
+        load_b(k_lo + (long long)t_at * BK, rb);
+        t_at += t_at + 1 < KT ? 1 : 0;
+    };
+#else
+    // Without bounds checks an address is a wave-uniform pointer -- the tile's corner, moved on from tile to tile and
+    // from one of a thread's loads to its next by scalar instructions -- plus one 32-bit offset per thread and
+    // operand that never changes: no vector instruction per load (vector instructions are paid in matrix time).
+    const unsigned oa = A_KCONTIG ? (tid >> 2) * (unsigned)a_sm + 4u * (tid & 3u) : (tid / (BM / 4)) * (unsigned)a_sk + 4u * (tid % (BM / 4));
+    const unsigned ob = B_KCONTIG ? (tid >> 2) * (unsigned)b_sn + 4u * (tid & 3u) : (tid / (BN / 4)) * (unsigned)b_sk + 4u * (tid % (BN / 4));
+    const float* Ab = A + (A_KCONTIG ? bm * a_sm + k_lo : k_lo * a_sk + bm);
+    const float* Bb = B + (B_KCONTIG ? bn * b_sn + k_lo : k_lo * b_sk + bn);
+    const long long ia = A_KCONTIG ? (NT / 4) * a_sm : (NT / (BM / 4)) * a_sk;   // from one of a thread's loads to its next
+    const long long ib = B_KCONTIG ? (NT / 4) * b_sn : (NT / (BN / 4)) * b_sk;
+    const long long step_a = A_KCONTIG ? BK : BK * a_sk, step_b = B_KCONTIG ? BK : BK * b_sk;
+    auto load_next = [&](float4_t* ra, float4_t* rb) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) ra[i] = *(const float4_t*)((const char*)(Ab + i * ia) + (size_t)(4u * oa));
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) rb[i] = *(const float4_t*)((const char*)(Bb + i * ib) + (size_t)(4u * ob));
+        const bool go = t_at + 1 < KT;
+        Ab += go ? step_a : 0;
+        Bb += go ? step_b : 0;
+        t_at += go ? 1 : 0;
+    };
+#endif
     float4_t ra1[A_LOADS], rb1[B_LOADS];
-    load_a(k_lo, ra0);
-    load_b(k_lo, rb0);
+    load_next(ra0, rb0);
     store_tiles(0, ra0, rb0);
-    if (KT > 1) {
-        load_a(k_lo + BK, ra1);
-        load_b(k_lo + BK, rb1);
-    }
+    load_next(ra1, rb1);
     __syncthreads();
-    // (Loads are issued under no condition -- beyond the last tile they fetch the last tile again, into a set nobody
-    // parks -- so that the wait in front of a parking names only the loads of the tile before.)
-    const long long k_last = k_lo + (KT - 1) * BK;
-    long long kt = 0;
+    int kt = 0;
     for (; kt + 1 < KT; kt += 2) {
-        load_a(min(k_lo + (kt + 2) * BK, k_last), ra0);
-        load_b(min(k_lo + (kt + 2) * BK, k_last), rb0);
+        load_next(ra0, rb0);
         compute(0, true, ra1, rb1);
         __syncthreads();
-        load_a(min(k_lo + (kt + 3) * BK, k_last), ra1);
-        load_b(min(k_lo + (kt + 3) * BK, k_last), rb1);
-        compute(1, true, ra0, rb0);   // (behind the last tile this parks a tile nobody reads: a parking under a condition
-        __syncthreads();              //  lets the compiler move the loads it consumes down to it)
+        load_next(ra1, rb1);
+        compute(1, true, ra0, rb0);
+        __syncthreads();
     }
     if (kt < KT) compute(0, false, ra1, rb1);   // an odd number of tiles: the last one sits in buffer 0
 #else

@@ -2993,7 +2993,10 @@ struct Lowerer {
         const bool a_k = a.s1 == 1, b_k = b.s0 == 1;
         const int64_t a_ld = a_k ? a.s0 : a.s1, b_ld = b_k ? b.s1 : b.s0;
         if ((a_k ? K : M) < 4 || (b_k ? K : N) < 4) return 2;
-        return ((a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4) || (K % 16)) ? 1 : 0;
+        // (the kernel without bounds checks addresses a tile by 32-bit offsets from its corner: lines of 2^22 elements
+        // and more take the checked variant, whose index arithmetic is 64 bits wide)
+        const int64_t widest = int64_t(1) << 22;
+        return ((a.offset % 4) || (b.offset % 4) || (a_ld % 4) || (b_ld % 4) || (K % 16) || a_ld >= widest || b_ld >= widest) ? 1 : 0;
     }
 
     template <class ReadsNode, class KeepsEpilogue>
