@@ -247,7 +247,7 @@ def measure_last_layer_products(dev):
     """The three products of configs[3]'s last layer (4096 -> 1024, batch 4096) on their own, without epilogues:
     y = x W (A rows contiguous), dW = x^T dy (A columns contiguous), dx = dy W^T (both along k).  With
     ADHIP_DOT_PLAN=<bm>,<bn>,<splits> in the environment the library launches them with that tile and that many ranges
-    of k instead of its own choice, which is how the alternatives in DESIGN.md were timed."""
+    of k instead of its own choice, which is how alternative tiles are timed."""
     import numpy as np
     from adhip import ir as IR
     rng = np.random.default_rng(0)

@@ -154,3 +154,39 @@ def test_ragged_products(layout, shape, hip_device):
     ref = a64 @ b64
     scale = float((np.abs(a64) @ np.abs(b64)).max())
     assert_close(got.data, ref.reshape(-1), RED_RTOL * math.sqrt(k), f"c ({layout})", scale=scale)
+
+
+def _wide_line_product(dev):
+    """C = A B with A the first 64 columns of a [64, 2^22] tensor: aligned in every respect, but a line of A is 2^22
+    elements long."""
+    from adhip import autodiff
+    from adhip.core import dot
+    autodiff.set_device(dev)
+    rng = np.random.default_rng(11)
+    wide = np.zeros((64, 1 << 22), np.float32)
+    wide[:, :64] = rng.standard_normal((64, 64), dtype=np.float32)
+    bn = rng.standard_normal((64, 128), dtype=np.float32)
+    x = autodiff.tensor(wide.reshape(-1), [64, 1 << 22])
+    b = autodiff.tensor(bn.reshape(-1), [64, 128])
+    c = dot(x.r(range(0, 64), 1), b)
+    c.forward()
+    c.val().keep()
+    return c, wide[:, :64].astype(np.float64) @ bn.astype(np.float64)
+
+
+def test_lines_of_2_to_the_22_take_the_checked_variant(hip_device):
+    """The kernel without bounds checks addresses a tile by 32-bit offsets from its corner; an operand whose lines are
+    2^22 elements apart is therefore given to the checked variant (64-bit index arithmetic), and the product is right."""
+    from adhip import autodiff
+    from test_row_chains import Capture
+    print("[case] product with a leading dim of 2^22", flush=True)
+    cap = Capture()
+    _wide_line_product(cap)
+    autodiff.execute()
+    names = _kernels(cap.proc, cap.deps)
+    assert names and all("_rim" in n or "_edge" in n for n in names), names
+    c, want = _wide_line_product(hip_device)
+    autodiff.execute()
+    got = c.val().get()
+    assert got.dim == [64, 128]
+    assert_close(got.data, want.reshape(-1), RED_RTOL * math.sqrt(64), "c", scale=float(np.abs(want).max()))
