@@ -2661,8 +2661,10 @@ struct Lowerer {
                         const bool is_member = is_side || (groups[g].kind == Group::ELW &&
                             std::find(groups[g].members.begin(), groups[g].members.end(), m) != groups[g].members.end());
                         // a row chain reads all it needs of a row before it stores any of it: it may overwrite a value
-                        // that its members read only at the row (and element) they work on
-                        bool chain_in_place = groups[g].kind == Group::ROWCHAIN;
+                        // of the same extent that its members read only at the row (and element) they work on (an id
+                        // redefined with another extent lays its rows out differently: another row's store could
+                        // land on what this row still has to read)
+                        bool chain_in_place = groups[g].kind == Group::ROWCHAIN && numel(old->shape) == numel(m->shape);
                         if (chain_in_place)
                             for (Node* cm : groups[g].members)
                                 chain_in_place = chain_in_place && chain_reads_rowwise(rp, cm, std::set<Node*>{old}, groups[g].cs_rows, groups[g].cs_cols);

@@ -225,3 +225,36 @@ def test_in_place_chain_in_a_loop_matches_float64(rows, cols, hip_device):
     got = hip_device.get_tensor("x").numpy().astype(np.float64)
     assert np.abs(got - want).max() <= RED_RTOL * math.sqrt(cols) * np.abs(want).max()
     np.testing.assert_allclose(got.sum(1), 1.0, rtol=1e-5)
+
+
+def _redefining_program(rows, cols, seed=9):
+    """`x` [rows, cols] is redefined as the [rows] vector of its rows' sums of exp2(x - max): the chain that reads the
+    old x writes a value of another extent under the same id."""
+    from adhip import ir as IR
+    rng = np.random.default_rng(seed)
+    xn = rng.standard_normal((rows, cols)).astype(np.float32)
+    cmds = [IR.CreateMat(xn.reshape(-1), [rows, cols], "x"),
+            IR.Max(a="x", res="m"), IR.View(a="m", target_dim=[rows, 1], res="mv"), IR.Broadcast(a="mv", dim=1, r=cols, res="mb"),
+            IR.CreateConstant(-1.0, "neg", [rows, cols]), IR.ElwMultiply(a="mb", b="neg", res="n"), IR.ElwAdd(a="x", b="n", res="d"),
+            IR.Exp2(a="d", res="e"), IR.Sum(a="e", res="x"), IR.EX()]
+    x64 = xn.astype(np.float64)
+    return IR.IRProcedure("main", cmds), {"x"}, np.exp2(x64 - x64.max(1, keepdims=True)).sum(1)
+
+
+def test_a_chain_does_not_overwrite_an_operand_of_another_extent():
+    """Row x's sum would land on element x of the buffer, which is element (0, x) of the old value that row 0 may still
+    be reading: the result goes to a buffer of its own and is copied afterwards."""
+    proc, keep, _ = _redefining_program(512, 256)
+    text = lower_describe(proc, keep)
+    assert "[rowchain]" in text and "launch commit_x [copy]" in text, text
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols", [(512, 256), (3000, 2052)])
+def test_redefinition_with_another_extent_matches_float64(rows, cols, hip_device):
+    print(f"[case] row chain redefines its operand's id with another extent {rows}x{cols}", flush=True)
+    proc, keep, want = _redefining_program(rows, cols)
+    hip_device.execute(proc, keep)
+    got = hip_device.get_tensor("x")
+    assert got.dim == [rows]
+    assert np.abs(got.numpy().astype(np.float64) - want).max() <= RED_RTOL * math.sqrt(cols) * np.abs(want).max()
