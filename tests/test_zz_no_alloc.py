@@ -62,6 +62,13 @@ def test_noalloc_with_device_predicated_loop(hip_device):
     _compare(plain, static, "manip_loop")
 
 
+def test_noalloc_with_row_chains_and_grouped_products(hip_device):
+    print("[case] noalloc: encoder layer 128x64, 4 heads (row chains, grouped and split products, layered launches)", flush=True)
+    plain, static, text = _both_ways(hip_device, lambda d: W.encoder_layer(d, 128, 64, 4, 128, seed=26))
+    assert " temp " in text and "[rowchain]" in text
+    _compare(plain, static, "encoder_layer")
+
+
 def test_noalloc_refuses_programs_beyond_the_static_area(hip_device):
     print("[case] noalloc: program with 64 MiB of temporaries", flush=True)
     wl = W.mlp_train(hip_device, 2048, (2048, 2048, 2048, 512), 1, seed=25)
