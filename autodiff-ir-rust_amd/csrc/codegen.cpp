@@ -516,6 +516,22 @@ struct Gen {
             for (size_t d = 0; d < coords.size(); ++d) {
                 const bool partial = p.lo[d] != 0 || p.hi[d] != t.shape[d];
                 if (!partial) { local[d] = coords[d]; continue; }
+                if (vec > 1 && p.lo[d] % vec == 0 && (p.hi[d] - p.lo[d]) % vec == 0 && vectorizable(coords[d])) {
+                    // The elements of one 128-bit access lie on the same side of a boundary at a multiple of four: the
+                    // condition and the piece's own coordinate are the quad's, so the loads under the condition stay
+                    // vector loads (a Concat of heads along the last dim, the gathered halves of a row).
+                    Aff base = coords[d];
+                    for (auto it2 = base.t.begin(); it2 != base.t.end(); ++it2)
+                        if (it2->first == lane_atom) { base.t.erase(it2); break; }
+                    const std::string bs = aff_str(base);
+                    if (p.lo[d] != 0) cond += strf("%s%s >= %lldu", cond.empty() ? "" : " && ", bs.c_str(), (long long)p.lo[d]);
+                    if (p.hi[d] != t.shape[d]) cond += strf("%s%s < %lldu", cond.empty() ? "" : " && ", bs.c_str(), (long long)p.hi[d]);
+                    const std::string code = p.lo[d] != 0 ? strf("(%s - %lld%s) / %d%s", bs.c_str(), (long long)p.lo[d], wide ? "ull" : "u", vec, wide ? "ull" : "u")
+                                                          : strf("%s / %d%s/*<%lld*/", bs.c_str(), vec, wide ? "ull" : "u", (long long)(p.hi[d] / vec));
+                    const int qa = expr_atom(code, (p.hi[d] - p.lo[d]) / vec, false);
+                    local[d] = aff_add(aff_atom(qa, vec), aff_atom(lane_atom, 1));
+                    continue;
+                }
                 clane = clane || aff_lane(coords[d]);
                 std::string cs = aff_str(coords[d]);
                 if (p.lo[d] != 0) cond += strf("%s%s >= %lldu", cond.empty() ? "" : " && ", cs.c_str(), (long long)p.lo[d]);
