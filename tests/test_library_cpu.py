@@ -691,3 +691,22 @@ def test_tightened_lowering_compiles(shift, monkeypatch):
     rc, msg = _compile_check(dev.proc, dev.deps)
     assert rc == 0, msg
     assert not _vector_spills(msg), msg
+
+
+def test_concat_at_a_multiple_of_four_keeps_vector_loads(monkeypatch):
+    """y = concat([a, b], 1) * c with 128-column parts: which part an element comes from is decided per 128-bit quad,
+    so both parts are read with (predicated) 128-bit loads; with a boundary inside a quad the loads are single ones."""
+    import numpy as np
+    monkeypatch.setenv("ADHIP_DUMP_SOURCE", "1")
+
+    def text(wa, wb):
+        z = lambda n: np.zeros(n, np.float32)  # noqa: E731
+        cmds = [IR.CreateMat(z(512 * wa), [512, wa], "a"), IR.CreateMat(z(512 * wb), [512, wb], "b"),
+                IR.CreateMat(z(512 * (wa + wb)), [512, wa + wb], "c"), IR.Concat(a="a", b="b", dim=1, res="ab"),
+                IR.ElwMultiply(a="ab", b="c", res="y"), IR.EX()]
+        return lower_describe(IR.IRProcedure("main", cmds), {"y"})
+    aligned = text(128, 128)
+    assert len(re.findall(r"if \(p\d+\) l\d+v = \*\(const float4_t\*\)", aligned)) == 2, aligned
+    assert not re.search(r"p\d+ \? b\d+\[", aligned)
+    ragged = text(126, 130)
+    assert re.search(r"p\d+ \? b\d+\[", ragged) and not re.search(r"if \(p\d+\) l\d+v = ", ragged)
