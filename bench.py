@@ -32,9 +32,9 @@ TRAFFIC_BYTES = {
     # written (dx, the [512][4096] partial column sums, one run sum per row and 256 columns)
     "reductions": {"elw_colsum": int((2 * 131353.0 + 278577.4) * 1024)},
     # the stand-alone reductions (profiles/reductions_forward_and_row_chains.hbm_traffic_pmc.txt), by kernel kind and
-    # tensors per launch: fetched x 2 + written (the column reduction writes a row of partial sums per 32 rows)
-    "reductions_forward": {("reduce_row", 1): int((2 * 131085.5 + 512.0) * 1024), ("reduce_col", 1): int((2 * 131087.0 + 8192.0) * 1024),
-                           ("reduce_row", 3): int((2 * 393230.0 + 1536.4) * 1024), ("reduce_col", 3): int((2 * 393232.0 + 24576.0) * 1024)},
+    # tensors per launch: fetched x 2 + written (the column reduction writes a row of partial sums per 64 rows)
+    "reductions_forward": {("reduce_row", 1): int((2 * 131085.5 + 512.0) * 1024), ("reduce_col", 1): int((2 * 131088.5 + 4096.0) * 1024),
+                           ("reduce_row", 3): int((2 * 393230.0 + 1536.4) * 1024), ("reduce_col", 3): int((2 * 393233.5 + 12288.0) * 1024)},
     # gather stage of configs[4] (one tiled element-wise launch): 2 x 73777.4 KiB fetched + 294912.0 KiB written
     "manip_loop": {"gather_stage": int((2 * 73777.4 + 294912.0) * 1024)},
 }
