@@ -1460,7 +1460,70 @@ struct Lowerer {
 
     // ---- 3. values that get a kernel and a buffer of their own whatever happens; product operands that are not
     // strided 2-D views of memory are copied first
+    // A product whose left operand is a Concat of row blocks, each of them a strided view of one value in memory (the
+    // heads of an attention layer side by side, transposed: the weight gradient of the projection behind them), would
+    // need the Concat written out first -- against the grain, through transposed copies.  Rows of a product depend on
+    // the same rows of its left operand only: it is computed as one product per block (they share a grouped launch) and
+    // is itself the Concat of their results.
+    void split_row_concat_products(RegionPlan& rp) {
+        if (!opt.fuse || !opt.group_dots) return;
+        bool changed = false;
+        std::vector<Node*> work = rp.topo;
+        for (Node* n : work) {
+            if (n->op != Op::DOT || n->in.size() != 2) continue;
+            const TRef A = n->in[0], B = n->in[1];
+            Affine2D a2, b2;
+            if (tref_affine2d(A, a2) || !tref_affine2d(B, b2)) continue;
+            if (A.pieces.size() < 2 || (int)A.pieces.size() > kGemmGroupSlots) continue;
+            const int64_t M = A.shape[0], K = A.shape[1], N = B.shape[1];
+            std::vector<const Piece*> blocks;
+            for (const Piece& pc : A.pieces) blocks.push_back(&pc);
+            std::sort(blocks.begin(), blocks.end(), [](const Piece* x, const Piece* y) { return x->lo[0] < y->lo[0]; });
+            bool ok = true;
+            int64_t at = 0;
+            std::vector<TRef> parts_a;
+            for (const Piece* pc : blocks) {
+                ok = ok && pc->lo[0] == at && pc->lo[1] == 0 && pc->hi[1] == K && pc->hi[0] - pc->lo[0] >= 64 && pc->src.kind == Src::NODE;
+                if (!ok) break;
+                at = pc->hi[0];
+                TRef ai;
+                ai.shape = {pc->hi[0] - pc->lo[0], K};
+                Piece q = *pc;
+                q.lo = {0, 0};
+                q.hi = ai.shape;
+                ai.pieces.push_back(std::move(q));
+                Affine2D pa;
+                ok = ok && tref_affine2d(ai, pa) && (op_is_leaf(pa.base->op) || op_is_elw(pa.base->op) || op_is_reduce(pa.base->op) ||
+                                                     pa.base->op == Op::DOT || pa.base->op == Op::ATTN || pa.base->root);
+                parts_a.push_back(std::move(ai));
+            }
+            if (!ok || at != M) continue;
+            TRef whole;
+            whole.shape = n->shape;
+            int64_t row = 0;
+            for (size_t i = 0; i < parts_a.size(); ++i) {
+                const Shape sh{parts_a[i].shape[0], N};
+                Node* d = new_node(Op::DOT, sh, {parts_a[i], B}, strf("%s.rows%zu", n->name.c_str(), i));
+                d->order = std::min(d->order, n->order - 0.25 + 0.01 * (double)i);
+                Piece q;
+                q.lo = {row, 0};
+                q.hi = {row + sh[0], N};
+                q.view.st.push_back(contiguous_stage(sh));
+                q.src.kind = Src::NODE;
+                q.src.node = d;
+                whole.pieces.push_back(std::move(q));
+                row += sh[0];
+            }
+            n->op = Op::COPY;
+            n->in = {whole};
+            n->key.clear();
+            changed = true;
+        }
+        if (changed) order_nodes(rp);
+    }
+
     void force_roots(RegionPlan& rp) {
+        split_row_concat_products(rp);
         auto& wanted = rp.wanted;
         auto& topo = rp.topo;
         for (auto& w : wanted) w.second->root = true;

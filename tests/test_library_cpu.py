@@ -710,3 +710,32 @@ def test_concat_at_a_multiple_of_four_keeps_vector_loads(monkeypatch):
     assert not re.search(r"p\d+ \? b\d+\[", aligned)
     ragged = text(126, 130)
     assert re.search(r"p\d+ \? b\d+\[", ragged) and not re.search(r"if \(p\d+\) l\d+v = ", ragged)
+
+
+def _row_concat_product(blocks=3, rows=128, k=256, n=192, seed=2):
+    """C = concat([x_1^T, ..., x_b^T], 0) . B with x_i [k, rows]: the left operand is a Concat of transposed blocks."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    xs = [rng.standard_normal((k, rows), dtype=np.float32) for _ in range(blocks)]
+    bn = rng.standard_normal((k, n), dtype=np.float32)
+    cmds = [IR.CreateMat(bn.reshape(-1), [k, n], "b")]
+    prev = None
+    for i, x in enumerate(xs):
+        cmds += [IR.CreateMat(x.reshape(-1), [k, rows], f"x{i}"), IR.Permute(a=f"x{i}", p=[1, 0], res=f"t{i}")]
+        if prev is None:
+            prev = f"t{i}"
+        else:
+            cmds.append(IR.Concat(a=prev, b=f"t{i}", dim=0, res=f"c{i}"))
+            prev = f"c{i}"
+    cmds += [IR.DotProduct(a=prev, b="b", res="y"), IR.EX()]
+    want = np.concatenate([x.T.astype(np.float64) for x in xs], 0) @ bn.astype(np.float64)
+    return IR.IRProcedure("main", cmds), {"y"}, want
+
+
+def test_a_product_of_concatenated_row_blocks_is_one_grouped_launch():
+    """Rows of a product depend on the same rows of its left operand only: the Concat is never written out (it would
+    need transposed copies of every block); the blocks' products share one launch and the result is their Concat."""
+    proc, keep, _ = _row_concat_product()
+    text = lower_describe(proc, keep)
+    assert re.search(r"launch dots_y\.rows0_3x_128x192x256 \[dot_mfma\]", text), text
+    assert "[transpose]" not in text and ".operand" not in text, text

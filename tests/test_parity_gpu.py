@@ -1108,3 +1108,16 @@ def test_tightened_lowering_matches_oracle(generator, scale, seed, shift, hip_de
         floor = max(own, 1e-2 * largest)
         assert (np.abs(g - r)[m] <= tol * np.maximum(np.abs(r[m]), floor)).all(), \
             f"{generator} scale {scale} seed {seed} {k}: {float(np.abs(g - r)[m].max()):.3e} > {tol * floor:.3e}"
+
+
+@pytest.mark.parametrize("blocks,rows,k,n", [(3, 128, 256, 192), (8, 64, 520, 100), (2, 200, 64, 64)])
+def test_product_of_concatenated_row_blocks(blocks, rows, k, n, hip_device):
+    """concat([x_1^T, ..., x_b^T], 0) . B runs as one grouped launch of b products whose results are concatenated
+    (tests/test_library_cpu.py holds the plan); values against float64."""
+    print(f"[case] product of {blocks} concatenated row blocks {rows}x{k} . {k}x{n}", flush=True)
+    from test_library_cpu import _row_concat_product
+    proc, keep, want = _row_concat_product(blocks, rows, k, n, seed=blocks + rows)
+    hip_device.execute(proc, keep)
+    got = hip_device.get_tensor("y")
+    assert got.dim == [blocks * rows, n]
+    assert_close(got.data, want.reshape(-1), RED_RTOL * math.sqrt(k), "y", scale=float(np.abs(want).max()))
