@@ -739,3 +739,17 @@ def test_a_product_of_concatenated_row_blocks_is_one_grouped_launch():
     text = lower_describe(proc, keep)
     assert re.search(r"launch dots_y\.rows0_3x_128x192x256 \[dot_mfma\]", text), text
     assert "[transpose]" not in text and ".operand" not in text, text
+
+
+@pytest.mark.parametrize("m,n,k,expect", [(2048, 1024, 1024, "adhip_gemm_kn_64"),          # 512 small tiles, 128 large ones, short k
+                                          (2048, 1024, 4096, "adhip_gemm_kn_128_splitk"),  # long k: the large tile's rate pays for the slice sum
+                                          (1024, 1024, 2048, "adhip_gemm_kn_128_splitk"),  # only 256 small tiles
+                                          (4096, 4096, 512, "adhip_gemm_kn_256")])         # large output: the 256x128 tile
+def test_product_tile_choice(m, n, k, expect):
+    """Which tile and whether k is cut, for outputs between the sizes where the answer is obvious (plan only)."""
+    import numpy as np
+    z = lambda r, c: np.zeros(r * c, np.float32)  # noqa: E731
+    cmds = [IR.CreateMat(z(m, k), [m, k], "a"), IR.CreateMat(z(k, n), [k, n], "b"), IR.DotProduct(a="a", b="b", res="c"), IR.EX()]
+    text = lower_describe(IR.IRProcedure("main", cmds), {"c"})
+    names = re.findall(r"launch dot_\w+ \[dot_mfma\] kernel=(\w+)", text)
+    assert names == [expect], text
