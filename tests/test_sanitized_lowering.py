@@ -81,9 +81,38 @@ def test_parser_and_lowering_under_host_sanitizers(tmp_path):
     for name, build in builders.items():
         proc, deps = build(OracleDevice()).finish()
         bases.append(_dump(str(tmp_path), name, proc, deps))
+    _run_driver(bases, 60)
+
+
+def _run_driver(bases, mutations, extra_env=None):
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1", UBSAN_OPTIONS="halt_on_error=1:print_stacktrace=1")
-    res = subprocess.run([DRIVER, "60"] + bases, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
+    env.update(extra_env or {})
+    res = subprocess.run([DRIVER, str(mutations)] + bases, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
     tail = res.stdout[-4000:]
     assert res.returncode == 0, tail
     assert "runtime error" not in res.stdout and "AddressSanitizer" not in res.stdout, tail
     assert "intact:" in res.stdout and " 0 failed" in res.stdout, tail
+
+
+@pytest.mark.parametrize("tighten", ["0", "2"])
+def test_model_and_adversarial_programs_under_host_sanitizers(tighten, tmp_path):
+    """The passes that model-shaped and oversized programs bring into play -- row chains, products of concatenated row
+    blocks, wide references cut into parts, long expressions cut, the tightened lowering that follows a vector spill
+    (forced with ADHIP_TIGHTEN) -- under the same sanitizers."""
+    import adversarial_programs as A
+    from fuzz_models import random_model_program
+    if not os.path.exists(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")):
+        pytest.skip("no hipcc to build the sanitized driver with")
+    _build_driver()
+    bases = []
+    for scale, seeds in ((1, range(16)), (16, [0, 3, 8, 27]), (48, [2])):
+        for seed in seeds:
+            dev = _Capture()
+            try:
+                random_model_program(dev, seed, scale)
+            except AttributeError:
+                pass   # the capture device returns no values; the program was handed over before that matters
+            bases.append(_dump(str(tmp_path), f"model{scale}_{seed}", dev.proc, dev.deps))
+    for name, made in (("wide", A.wide_concat(100)), ("pieces", A.one_buffer_pieces(200)), ("gathers", A.gathers(39)), ("rider", A.rider(19))):
+        bases.append(_dump(str(tmp_path), name, made[0], made[1]))
+    _run_driver(bases, 8, {"ADHIP_TIGHTEN": tighten} if tighten != "0" else None)
